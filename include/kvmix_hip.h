@@ -1,0 +1,147 @@
+/*
+ * kvmix_hip.h -- C ABI of libkvmix_hip.so: the KVmix KV-cache hot path on gfx950.
+ *
+ * Plain C: device pointers, sizes, strides, a hipStream_t passed as void*.  No
+ * torch types.  Every call validates its arguments on the host, enqueues its
+ * kernels on `stream` and returns without synchronising.  Return value 0 is
+ * success; negative values are the KVMIX_ERR_* codes below (kvmix_strerror()
+ * gives the text, which for argument errors is the reference's TORCH_CHECK text).
+ * The library keeps no global mutable state: calls on different streams or from
+ * different threads are independent.
+ *
+ * Packed formats (`fmt`):
+ *   KVMIX_FMT_REF    the reference's layout.  bits 1/2/4: 32/bits codes per
+ *                    uint32, code i at bit i*bits.  bits 3: eleven codes per
+ *                    uint32 -- ten 3-bit codes at bits 0..29 and an eleventh
+ *                    clamped to 0..3 at bits 30..31 -- and the group is 11
+ *                    (quant_cuda/csrc/quantization_cuda.cu:573-584,617-621).
+ *   KVMIX_FMT_DENSE3 extension with no counterpart in the reference: 3-bit
+ *                    codes as a little-endian bit stream, 32 codes in three
+ *                    consecutive uint32, any group that is a multiple of 32.
+ */
+#ifndef KVMIX_HIP_H
+#define KVMIX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVMIX_OK 0
+#define KVMIX_ERR_BITS (-1)        /* bits not in {1,2,3,4} */
+#define KVMIX_ERR_GROUP3 (-2)      /* bits == 3 (reference format) needs group 11 */
+#define KVMIX_ERR_STEPS_GROUP (-3) /* last dimension not divisible by the group */
+#define KVMIX_ERR_STEPS_WORD (-4)  /* last dimension not divisible by codes per word */
+#define KVMIX_ERR_HEADS (-5)       /* query heads not divisible by kv heads */
+#define KVMIX_ERR_DTYPE (-6)       /* dtype tag not KVMIX_F16 / KVMIX_F32 */
+#define KVMIX_ERR_NULL (-7)        /* null pointer with a non-empty problem */
+#define KVMIX_ERR_SHAPE (-8)       /* negative size or a stride smaller than the row it spans */
+#define KVMIX_ERR_UNSUPPORTED (-9) /* group / word combination the packed layout cannot express */
+#define KVMIX_ERR_FORMAT (-10)     /* unknown fmt */
+#define KVMIX_ERR_WORKSPACE (-11)  /* workspace smaller than kvmix_gemv_workspace_bytes() */
+#define KVMIX_ERR_LAUNCH (-12)     /* hipGetLastError() after a launch was not hipSuccess */
+
+#define KVMIX_F16 0
+#define KVMIX_F32 1
+
+#define KVMIX_FMT_REF 0
+#define KVMIX_FMT_DENSE3 1
+/* quantizer only, bits == 3: the reference's value-append kernel packs the eleventh code
+ * of a word with the plain shift 10*3 after clamping to 0..7, so only its low two bits
+ * survive (quantization_cuda.cu:282-289 with j == 10; the reference calls this branch
+ * "placeholder logic", :463).  Kept so process_value_quantization_cuda stays literal. */
+#define KVMIX_FMT_REF3_WRAP 2
+
+/* how the returned scale is rounded (the codes always use (max-min)/qmax):
+ *   KVMIX_SCALE_RECIPROCAL  (max-min) * fp32(1/qmax) -- what the reference's
+ *        one-shot quantizer returns, because quantization_cuda.cu:711 divides a
+ *        tensor by an integer scalar through ATen's CUDA kernel, which multiplies
+ *        by the scalar's reciprocal;
+ *   KVMIX_SCALE_DIVIDE      (max-min) / qmax -- what the reference's append
+ *        kernels store (quantization_cuda.cu:49-51,149-151,234). */
+#define KVMIX_SCALE_RECIPROCAL 0
+#define KVMIX_SCALE_DIVIDE 1
+
+typedef void *kvmix_stream_t; /* hipStream_t */
+
+int kvmix_version(void);
+const char *kvmix_strerror(int code);
+
+/*
+ * Group quantize + bit-pack along the last dimension.
+ * Replaces quantize_pack_last_dim_cuda (quant_cuda/csrc/quantization_cuda.h:23-28,
+ * quantization_cuda.cu:631-721) and, through the strides, the "new" half of
+ * process_key_quantization_cuda / process_value_quantization_cuda
+ * (quantization_cuda.h:4-21, quantization_cuda.cu:298-537).
+ *
+ *   x      [outer, inner, steps]  fp16 or fp32 (x_dtype), unit stride along steps,
+ *          element strides x_outer_stride / x_inner_stride
+ *   code   [outer, inner, steps/vpw] uint32 words, word strides code_*_stride
+ *   scale, zero  [outer, inner, steps/group], same dtype as x, element strides sz_*_stride
+ *
+ * Keys (grouped per channel along tokens):  outer = B*Hkv, inner = D, steps = n.
+ * Values (grouped per token along head_dim): outer = B*Hkv, inner = n, steps = D.
+ * Writing at an offset into a larger pre-allocated cache is done by offsetting the
+ * output pointers and passing the cache's strides.
+ */
+int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t outer, int64_t inner, int64_t steps,
+                              int64_t x_outer_stride, int64_t x_inner_stride, int group, int bits,
+                              int fmt, int scale_mode, uint32_t *code, int64_t code_outer_stride,
+                              int64_t code_inner_stride, void *scale, void *zero,
+                              int64_t sz_outer_stride, int64_t sz_inner_stride, kvmix_stream_t stream);
+
+/*
+ * Key quantizer that reads the token-major fp16 tail directly and writes the
+ * channel-major packed layout, i.e. quantize_pack_last_dim_cuda applied to
+ * `tail[:, :, :n, :].transpose(2, 3).contiguous()` without materialising the
+ * transpose (the call site is models/modeling_llama_KVmix.py:131-133).
+ *
+ *   k      [outer, n, D] fp16, unit stride along D, element strides k_outer_stride / k_token_stride
+ *   code   [outer, D, n/vpw]; scale, zero [outer, D, n/group] fp16
+ * group must be 32 (bits 1/2/4, or 3 with KVMIX_FMT_DENSE3) or 11 (bits 3, KVMIX_FMT_REF).
+ */
+int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D,
+                                int64_t k_outer_stride, int64_t k_token_stride, int group, int bits,
+                                int fmt, int scale_mode, uint32_t *code, int64_t code_outer_stride,
+                                int64_t code_inner_stride, void *scale, void *zero,
+                                int64_t sz_outer_stride, int64_t sz_inner_stride, kvmix_stream_t stream);
+
+/*
+ * Fused dequantize + matrix-vector product over the packed cache.
+ * Replaces quantized_gemm (quant_cuda/csrc/dequantization_gemv_cuda.h:22-29,
+ * dequantization_gemv_cuda.cu:7-248):
+ *
+ *   out[s, m, n] = fp16( sum_k fp32(x[s, m, k]) *
+ *                        ( fp32(scale[s', k, grp(n)]) * code[s', k, n] + fp32(zero[s', k, grp(n)]) ) )
+ *   s' = s / heads_per_kv,   grp(n) = n / group,   fp32 accumulation.
+ *
+ *   x      [samples, M, K] fp16     (samples = B * query heads)
+ *   code   [samples/heads_per_kv, K, N/vpw] uint32, read in the stored layout (no transpose copy)
+ *   scale, zero [samples/heads_per_kv, K, N/group] fp16
+ *   out    [samples, M, N] fp16
+ * All strides are in elements of the respective array; rows are unit-stride.
+ *
+ * q.K^T is the case K = head_dim, N = quantized tokens (code = key codes [.., D, Tq/vpw]);
+ * p.V is the case K = quantized tokens, N = head_dim (code = value codes [.., Tq, D/vpw]).
+ * The reference kernel only produces row m = 0 (it ignores blockIdx.z); rows m >= 1 are
+ * computed here with the same formula.
+ *
+ * workspace: device scratch of at least kvmix_gemv_workspace_bytes() bytes for the same
+ * sizes (may be NULL when that returns 0).  Its contents are undefined afterwards.
+ */
+size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t K, int64_t N);
+
+int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride, int64_t x_row_stride,
+                         const uint32_t *code, int64_t code_batch_stride, int64_t code_row_stride,
+                         const void *scale, const void *zero, int64_t sz_batch_stride,
+                         int64_t sz_row_stride, int bits, int fmt, int64_t samples, int heads_per_kv,
+                         int64_t M, int64_t K, int64_t N, void *out, int64_t out_batch_stride,
+                         int64_t out_row_stride, void *workspace, size_t workspace_bytes,
+                         kvmix_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVMIX_HIP_H */

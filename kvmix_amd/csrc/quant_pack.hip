@@ -1,0 +1,435 @@
+// Group quantize + bit-pack kernels for the KV cache append path (gfx950).
+//
+// What is computed (per group of `group` consecutive values of the last dimension):
+//   mn = min, mx = max            (fp32, NaN-ignoring like fminf/fmaxf)
+//   scale = (mx - mn) / qmax      (IEEE fp32 division)
+//   code_i = clamp(roundf((x_i - mn) / scale), 0, qmax)     roundf = ties away from zero
+//   words  = codes packed LSB-first
+// following quant_cuda/csrc/quantization_cuda.cu:540-629 of the reference.  Unlike the
+// reference there is no fp32 staging copy of the input, no int32-per-element temporary
+// and no second packing kernel: min/max, codes and words stay in registers.
+//
+// Three kernels:
+//   quant_rows_g32_f16   fast path: fp16 input, group 32, four lanes per group, each lane
+//                        one 128-bit load (8 halves); quad shuffles for min/max and packing.
+//   quant_rows_generic   any group / dtype / format, one thread per lcm(group, codes-per-word)
+//                        values, serial like the reference (used for group 11, fp32 input,
+//                        unaligned rows).
+//   quant_key_tokens     keys straight from the token-major fp16 tail: one thread per channel
+//                        holds one group of tokens in registers (fuses the caller's transpose).
+
+#include "kvmix_common.h"
+
+namespace kvmix {
+
+struct QuantArgs {
+    const void *x;
+    uint32_t *code;
+    void *scale;
+    void *zero;
+    int64_t outer, inner, steps;
+    int64_t x_os, x_is;        // element strides of x
+    int64_t c_os, c_is;        // word strides of code
+    int64_t s_os, s_is;        // element strides of scale / zero
+    int group;
+    int bits;
+    int fmt;
+    int scale_mode;
+    float inv_qmax;
+};
+
+template <typename T>
+__device__ __forceinline__ float load_as_float(const T *p);
+template <>
+__device__ __forceinline__ float load_as_float<__half>(const __half *p)
+{
+    return __half2float(*p);
+}
+template <>
+__device__ __forceinline__ float load_as_float<float>(const float *p)
+{
+    return *p;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_from_float(T *p, float v);
+template <>
+__device__ __forceinline__ void store_from_float<__half>(__half *p, float v)
+{
+    *p = __float2half_rn(v);
+}
+template <>
+__device__ __forceinline__ void store_from_float<float>(float *p, float v)
+{
+    *p = v;
+}
+
+// ---------------------------------------------------------------------------------------
+// generic: one thread per `unit` = lcm(group, codes per word) consecutive values
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) quant_rows_generic(QuantArgs a, int unit, int64_t units_per_row,
+                                                          int64_t total_units)
+{
+    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (u >= total_units) return;
+    const int64_t row = u / units_per_row;
+    const int64_t ur = u - row * units_per_row;
+    const int64_t o = row / a.inner;
+    const int64_t i = row - o * a.inner;
+    const T *x = (const T *)a.x + o * a.x_os + i * a.x_is + ur * unit;
+    const int qmax = (1 << a.bits) - 1;
+    const bool ref3 = (a.bits == 3 && a.fmt != KVMIX_FMT_DENSE3);
+    const bool wrap11 = a.fmt == KVMIX_FMT_REF3_WRAP;
+    const int vpw = ref3 ? 11 : 32 / a.bits;  // dense3: handled by the bit buffer below
+    const int groups_per_unit = unit / a.group;
+    T *sc = (T *)a.scale + o * a.s_os + i * a.s_is + ur * groups_per_unit;
+    T *zr = (T *)a.zero + o * a.s_os + i * a.s_is + ur * groups_per_unit;
+    // words per unit: ref formats unit/vpw; dense3 unit*3/32
+    const int64_t words_per_unit = (a.bits == 3 && !ref3) ? (int64_t)unit * 3 / 32 : unit / vpw;
+    uint32_t *cw = a.code + o * a.c_os + i * a.c_is + ur * words_per_unit;
+
+    uint64_t buf = 0;
+    int filled = 0;
+    int pos3 = 0;  // position inside an 11-code word (reference 3-bit format)
+    for (int g = 0; g < groups_per_unit; g++) {
+        const T *xg = x + (int64_t)g * a.group;
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+        for (int j = 0; j < a.group; j++) {
+            float v = load_as_float<T>(xg + j);
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
+        }
+        const float range = mx - mn;
+        const float scale = range / (float)qmax;
+        store_from_float<T>(sc + g, scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+        store_from_float<T>(zr + g, mn);
+        for (int j = 0; j < a.group; j++) {
+            float v = load_as_float<T>(xg + j);
+            if (ref3) {
+                uint32_t q = quantize_code(v, mn, scale, (pos3 < 10 || wrap11) ? 7 : 3);
+                if (pos3 == 10) q &= 3u;  // only two bits of the word are left
+                buf |= (uint64_t)q << (pos3 < 10 ? 3 * pos3 : 30);
+                if (++pos3 == 11) {
+                    *cw++ = (uint32_t)buf;
+                    buf = 0;
+                    pos3 = 0;
+                }
+            } else {
+                uint32_t q = quantize_code(v, mn, scale, qmax);
+                buf |= (uint64_t)q << filled;
+                filled += a.bits;
+                if (filled >= 32) {
+                    *cw++ = (uint32_t)buf;
+                    buf >>= 32;
+                    filled -= 32;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// fast path: fp16, group 32, 4 lanes per group, 8 halves (one 128-bit load) per lane.
+// BITS = 1, 2, 4 (reference layout) or 3 with DENSE3 = true (bit-stream extension).
+// ---------------------------------------------------------------------------------------
+template <int BITS>
+__global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t groups_per_row,
+                                                          int64_t total_groups)
+{
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t g = tid >> 2;
+    const int j = (int)(tid & 3);
+    const bool active = g < total_groups;
+    if (!active) g = total_groups - 1;  // keep the quad's shuffles convergent
+    const int64_t row = g / groups_per_row;
+    const int64_t gr = g - row * groups_per_row;
+    const int64_t o = row / a.inner;
+    const int64_t i = row - o * a.inner;
+    const __half *x = (const __half *)a.x + o * a.x_os + i * a.x_is + gr * 32 + j * 8;
+
+    const uint4 raw = *reinterpret_cast<const uint4 *>(x);
+    float v[8];
+    {
+        const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            v[2 * t] = h16_to_f32((uint16_t)(r[t] & 0xffffu));
+            v[2 * t + 1] = h16_to_f32((uint16_t)(r[t] >> 16));
+        }
+    }
+    float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        mn = fminf(mn, v[t]);
+        mx = fmaxf(mx, v[t]);
+    }
+    mn = fminf(mn, __shfl_xor(mn, 1));
+    mx = fmaxf(mx, __shfl_xor(mx, 1));
+    mn = fminf(mn, __shfl_xor(mn, 2));
+    mx = fmaxf(mx, __shfl_xor(mx, 2));
+
+    constexpr int qmax = (1 << BITS) - 1;
+    const float range = mx - mn;
+    const float scale = range / (float)qmax;
+    uint32_t piece = 0;  // this lane's 8 codes, 8*BITS bits
+#pragma unroll
+    for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, qmax) << (t * BITS);
+
+    uint32_t *cw = a.code + o * a.c_os + i * a.c_is + gr * BITS;  // BITS words per group of 32
+    if (BITS == 4) {
+        if (active) cw[j] = piece;
+    } else if (BITS == 2) {
+        const uint32_t other = __shfl_xor(piece, 1);
+        if (active && (j & 1) == 0) cw[j >> 1] = piece | (other << 16);
+    } else if (BITS == 1) {
+        uint32_t w = piece << (8 * j);
+        w |= __shfl_xor(w, 1);
+        w |= __shfl_xor(w, 2);
+        if (active && j == 0) cw[0] = w;
+    } else {  // BITS == 3, bit stream: lane j holds stream bits [24j, 24j+24)
+        const uint32_t next = __shfl_down(piece, 1);  // lane j+1's piece (unused for j == 3)
+        uint32_t w;
+        if (j == 0)
+            w = piece | (next << 24);
+        else if (j == 1)
+            w = (piece >> 8) | (next << 16);
+        else
+            w = (piece >> 16) | (next << 8);
+        if (active && j < 3) cw[j] = w;
+    }
+    if (active && j == 0) {
+        __half *sc = (__half *)a.scale + o * a.s_os + i * a.s_is + gr;
+        *sc = __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+    }
+    if (active && j == 1) {
+        __half *zr = (__half *)a.zero + o * a.s_os + i * a.s_is + gr;
+        *zr = __float2half_rn(mn);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// keys from the token-major tail: k [outer, n, D] -> code [outer, D, n/vpw], groups of G
+// tokens per channel.  One thread per channel, one block row per (group, outer).
+// MODE: 1, 2, 4 = reference layout bits; 3 = reference 3-bit (G must be 11); 30 = dense 3-bit.
+// ---------------------------------------------------------------------------------------
+struct KeyTokArgs {
+    const __half *k;
+    uint32_t *code;
+    __half *scale;
+    __half *zero;
+    int64_t n, D;
+    int64_t k_os, k_ts;
+    int64_t c_os, c_is;
+    int64_t s_os, s_is;
+    int scale_mode;
+    float inv_qmax;
+};
+
+template <int G, int MODE>
+__global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
+{
+    constexpr int BITS = MODE == 30 ? 3 : MODE;
+    constexpr int qmax = (1 << BITS) - 1;
+    constexpr int WORDS = MODE == 3 ? 1 : (G * BITS) / 32;  // words per group
+    const int64_t d = (int64_t)blockIdx.z * blockDim.x + threadIdx.x;
+    if (d >= a.D) return;
+    const int64_t gi = blockIdx.x;
+    const int64_t o = blockIdx.y;
+    const __half *src = a.k + o * a.k_os + gi * G * a.k_ts + d;
+    float v[G];
+    float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+#pragma unroll
+    for (int t = 0; t < G; t++) {
+        v[t] = __half2float(src[t * a.k_ts]);
+        mn = fminf(mn, v[t]);
+        mx = fmaxf(mx, v[t]);
+    }
+    const float range = mx - mn;
+    const float scale = range / (float)qmax;
+    uint32_t w[WORDS];
+#pragma unroll
+    for (int t = 0; t < WORDS; t++) w[t] = 0;
+#pragma unroll
+    for (int t = 0; t < G; t++) {
+        if (MODE == 3) {
+            uint32_t q = quantize_code(v[t], mn, scale, t < 10 ? 7 : 3);
+            w[0] |= q << (t < 10 ? 3 * t : 30);
+        } else {
+            uint32_t q = quantize_code(v[t], mn, scale, qmax);
+            const int bit = t * BITS;
+            w[bit >> 5] |= q << (bit & 31);
+            if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+        }
+    }
+    uint32_t *cw = a.code + o * a.c_os + d * a.c_is + gi * WORDS;
+#pragma unroll
+    for (int t = 0; t < WORDS; t++) cw[t] = w[t];
+    a.scale[o * a.s_os + d * a.s_is + gi] =
+        __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+    a.zero[o * a.s_os + d * a.s_is + gi] = __float2half_rn(mn);
+}
+
+static int64_t gcd64(int64_t a, int64_t b)
+{
+    while (b) {
+        int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+// Validation shared by both entry points.  Returns the number of codes per word
+// through *vpw (0 for the dense 3-bit stream, whose unit is 32 codes in 3 words).
+static int check_format(int group, int bits, int fmt, int64_t steps, int *vpw)
+{
+    if (fmt != KVMIX_FMT_REF && fmt != KVMIX_FMT_DENSE3 && fmt != KVMIX_FMT_REF3_WRAP) return KVMIX_ERR_FORMAT;
+    if (bits != 1 && bits != 2 && bits != 3 && bits != 4) return KVMIX_ERR_BITS;
+    if (fmt != KVMIX_FMT_REF && bits != 3) return KVMIX_ERR_FORMAT;
+    if (bits == 3 && fmt != KVMIX_FMT_DENSE3) {
+        if (group != 11) return KVMIX_ERR_GROUP3;
+        if (steps % 11 != 0) return KVMIX_ERR_STEPS_GROUP;
+        *vpw = 11;
+        return KVMIX_OK;
+    }
+    if (group <= 0 || steps % group != 0) return KVMIX_ERR_STEPS_GROUP;
+    if (fmt == KVMIX_FMT_DENSE3) {
+        if (group % 32 != 0) return KVMIX_ERR_UNSUPPORTED;
+        *vpw = 0;
+        return KVMIX_OK;
+    }
+    if (steps % (32 / bits) != 0) return KVMIX_ERR_STEPS_WORD;
+    *vpw = 32 / bits;
+    return KVMIX_OK;
+}
+
+}  // namespace kvmix
+
+using namespace kvmix;
+
+extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t outer, int64_t inner,
+                                         int64_t steps, int64_t x_outer_stride, int64_t x_inner_stride,
+                                         int group, int bits, int fmt, int scale_mode, uint32_t *code,
+                                         int64_t code_outer_stride, int64_t code_inner_stride,
+                                         void *scale, void *zero, int64_t sz_outer_stride,
+                                         int64_t sz_inner_stride, kvmix_stream_t stream)
+{
+    int vpw = 0;
+    if (x_dtype != KVMIX_F16 && x_dtype != KVMIX_F32) return KVMIX_ERR_DTYPE;
+    if (outer < 0 || inner < 0 || steps < 0) return KVMIX_ERR_SHAPE;
+    int rc = check_format(group, bits, fmt, steps, &vpw);
+    if (rc != KVMIX_OK) return rc;
+    if (scale_mode != KVMIX_SCALE_RECIPROCAL && scale_mode != KVMIX_SCALE_DIVIDE) return KVMIX_ERR_FORMAT;
+    if (outer == 0 || inner == 0 || steps == 0) return KVMIX_OK;
+    if (!x || !code || !scale || !zero) return KVMIX_ERR_NULL;
+    const int64_t words = vpw ? steps / vpw : steps * 3 / 32;
+    const int64_t groups = steps / group;
+    if (x_inner_stride < steps || code_inner_stride < words || sz_inner_stride < groups) return KVMIX_ERR_SHAPE;
+    if (inner > 1 && (x_outer_stride < x_inner_stride || code_outer_stride < code_inner_stride ||
+                      sz_outer_stride < sz_inner_stride))
+        return KVMIX_ERR_SHAPE;
+
+    QuantArgs a;
+    a.x = x;
+    a.code = code;
+    a.scale = scale;
+    a.zero = zero;
+    a.outer = outer;
+    a.inner = inner;
+    a.steps = steps;
+    a.x_os = x_outer_stride;
+    a.x_is = x_inner_stride;
+    a.c_os = code_outer_stride;
+    a.c_is = code_inner_stride;
+    a.s_os = sz_outer_stride;
+    a.s_is = sz_inner_stride;
+    a.group = group;
+    a.bits = bits;
+    a.fmt = fmt;
+    a.scale_mode = scale_mode;
+    a.inv_qmax = 1.0f / (float)((1 << bits) - 1);
+    hipStream_t st = (hipStream_t)stream;
+
+    const bool ref3 = bits == 3 && fmt != KVMIX_FMT_DENSE3;
+    const bool aligned16 = ((uintptr_t)x % 16 == 0) && (x_outer_stride % 8 == 0) && (x_inner_stride % 8 == 0);
+    if (x_dtype == KVMIX_F16 && group == 32 && !ref3 && aligned16) {
+        const int64_t total_groups = outer * inner * groups;
+        const int64_t threads = total_groups * 4;
+        const unsigned blocks = (unsigned)((threads + 255) / 256);
+        switch (bits) {
+        case 1: hipLaunchKernelGGL(quant_rows_g32_f16<1>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
+        case 2: hipLaunchKernelGGL(quant_rows_g32_f16<2>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
+        case 3: hipLaunchKernelGGL(quant_rows_g32_f16<3>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
+        default: hipLaunchKernelGGL(quant_rows_g32_f16<4>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
+        }
+        return launch_status();
+    }
+    // generic path: a thread owns lcm(group, codes per word) values, i.e. whole groups and whole words
+    const int64_t word_span = vpw ? vpw : 32;
+    const int64_t unit = (int64_t)group / gcd64(group, word_span) * word_span;
+    if (steps % unit != 0 || unit > (1 << 20)) return KVMIX_ERR_UNSUPPORTED;
+    const int64_t units_per_row = steps / unit;
+    const int64_t total_units = outer * inner * units_per_row;
+    const unsigned blocks = (unsigned)((total_units + 255) / 256);
+    if (x_dtype == KVMIX_F16)
+        hipLaunchKernelGGL(quant_rows_generic<__half>, dim3(blocks), dim3(256), 0, st, a, (int)unit,
+                           units_per_row, total_units);
+    else
+        hipLaunchKernelGGL(quant_rows_generic<float>, dim3(blocks), dim3(256), 0, st, a, (int)unit,
+                           units_per_row, total_units);
+    return launch_status();
+}
+
+extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D,
+                                           int64_t k_outer_stride, int64_t k_token_stride, int group,
+                                           int bits, int fmt, int scale_mode, uint32_t *code,
+                                           int64_t code_outer_stride, int64_t code_inner_stride,
+                                           void *scale, void *zero, int64_t sz_outer_stride,
+                                           int64_t sz_inner_stride, kvmix_stream_t stream)
+{
+    int vpw = 0;
+    if (outer < 0 || n < 0 || D < 0) return KVMIX_ERR_SHAPE;
+    if (fmt == KVMIX_FMT_REF3_WRAP) return KVMIX_ERR_FORMAT;
+    int rc = check_format(group, bits, fmt, n, &vpw);
+    if (rc != KVMIX_OK) return rc;
+    const bool ref3 = bits == 3 && fmt == KVMIX_FMT_REF;
+    if (!ref3 && group != 32) return KVMIX_ERR_UNSUPPORTED;
+    if (scale_mode != KVMIX_SCALE_RECIPROCAL && scale_mode != KVMIX_SCALE_DIVIDE) return KVMIX_ERR_FORMAT;
+    if (outer == 0 || n == 0 || D == 0) return KVMIX_OK;
+    if (!k || !code || !scale || !zero) return KVMIX_ERR_NULL;
+    const int64_t words = vpw ? n / vpw : n * 3 / 32;
+    const int64_t groups = n / group;
+    if (k_token_stride < D || code_inner_stride < words || sz_inner_stride < groups) return KVMIX_ERR_SHAPE;
+    if (outer > 65535 || groups > 0x7fffffff) return KVMIX_ERR_SHAPE;
+
+    KeyTokArgs a;
+    a.k = (const __half *)k;
+    a.code = code;
+    a.scale = (__half *)scale;
+    a.zero = (__half *)zero;
+    a.n = n;
+    a.D = D;
+    a.k_os = k_outer_stride;
+    a.k_ts = k_token_stride;
+    a.c_os = code_outer_stride;
+    a.c_is = code_inner_stride;
+    a.s_os = sz_outer_stride;
+    a.s_is = sz_inner_stride;
+    a.scale_mode = scale_mode;
+    a.inv_qmax = 1.0f / (float)((1 << bits) - 1);
+    hipStream_t st = (hipStream_t)stream;
+    const int block = D >= 128 ? 128 : 64;
+    const dim3 grid((unsigned)groups, (unsigned)outer, (unsigned)((D + block - 1) / block));
+    if (ref3)
+        hipLaunchKernelGGL((quant_key_tokens<11, 3>), grid, dim3(block), 0, st, a);
+    else if (bits == 3)
+        hipLaunchKernelGGL((quant_key_tokens<32, 30>), grid, dim3(block), 0, st, a);
+    else if (bits == 4)
+        hipLaunchKernelGGL((quant_key_tokens<32, 4>), grid, dim3(block), 0, st, a);
+    else if (bits == 2)
+        hipLaunchKernelGGL((quant_key_tokens<32, 2>), grid, dim3(block), 0, st, a);
+    else
+        hipLaunchKernelGGL((quant_key_tokens<32, 1>), grid, dim3(block), 0, st, a);
+    return launch_status();
+}

@@ -1,0 +1,241 @@
+"""The reference's four operators (module `KVmix`, quant_cuda/csrc/pybind.cpp:6-15) on top of
+the gfx950 C ABI.  Names, positional argument order, return types and error texts follow the
+reference; the tensors are torch ROCm tensors, everything else is the HIP library.
+
+    quantize_pack_last_dim_cuda(input, group_length, quant_bits) -> (code, scale, min)
+    quantized_gemm(group_size, fA, qB, scales, zeros, bits) -> out
+    process_key_quantization_cuda(input, prev_code, prev_scale, prev_min, group_length, quant_bits)
+    process_value_quantization_cuda(input, prev_code, prev_scale, prev_min, group_length, quant_bits)
+
+All four launch on torch's current stream of the input's device and do not synchronise.
+"""
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float16: _lib.F16, torch.float32: _lib.F32}
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("KVmix operators run on the GPU only: got a tensor on " + str(t.device))
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _values_per_word(bits: int) -> int:
+    return 11 if bits == 3 else 32 // bits
+
+
+def _check_bits(bits: int) -> None:
+    if bits not in (1, 2, 3, 4):
+        raise RuntimeError("Supported quantization bits: 1, 2, 3, 4")
+
+
+def _rows3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:
+    """View a 4-D tensor [B, H, R, S] as [B*H, R, S] without copying when its strides allow it;
+    returns (tensor, outer_stride, inner_stride) in elements."""
+    B, H, R, S = t.shape
+    ok = (S <= 1 or t.stride(3) == 1) and (B <= 1 or t.stride(0) == H * t.stride(1))
+    if ok and R > 1 and t.stride(2) < S:
+        ok = False
+    if ok and H > 1 and t.stride(1) < t.stride(2):
+        ok = False
+    if not ok:
+        t = t.contiguous()
+    return t, (t.stride(1) if B * H > 1 else max(R * t.stride(2), 1)), (t.stride(2) if R > 1 else max(S, 1))
+
+
+def _quantize_into(x: torch.Tensor, group: int, bits: int, fmt: int, scale_mode: int,
+                   code: torch.Tensor, scale: torch.Tensor, mn: torch.Tensor) -> None:
+    """x [B,H,R,S]; code/scale/mn 4-D views (possibly slices of larger buffers) to fill."""
+    L = _lib.load()
+    B, H, R, S = x.shape
+    x, xo, xi = _rows3(x)
+    with torch.cuda.device(x.device):
+        _lib.check(L.kvmix_quant_pack_last_dim(
+            x.data_ptr(), _DT[x.dtype], B * H, R, S, xo, xi, group, bits, fmt, scale_mode,
+            code.data_ptr(), code.stride(1), code.stride(2),
+            scale.data_ptr(), mn.data_ptr(), scale.stride(1), scale.stride(2), _stream(x)))
+
+
+def quantize_pack_last_dim_cuda(input: torch.Tensor, group_length: int, quant_bits: int):
+    """Group-quantize the last dimension of a 4-D fp16/fp32 tensor and bit-pack the codes.
+
+    Reference: quantize_pack_last_dim_cuda, quant_cuda/csrc/quantization_cuda.cu:631-721.
+    Returns (code int32 [B,H,R,S/vpw], scale [B,H,R,S/g], min [B,H,R,S/g]); scale and min have the
+    input's dtype.  3-bit uses the reference's 11-codes-per-word layout and needs group_length 11."""
+    if quant_bits == 3 and group_length != 11:
+        raise RuntimeError("For 3-bit quantization, group_length must be 11")
+    if input.dtype not in _DT:
+        raise RuntimeError(f"expected scalar type Float or Half but found {input.dtype}")
+    if input.dim() != 4:
+        raise RuntimeError("input_tensor must be a 4D tensor")
+    _check_bits(quant_bits)
+    B, H, R, S = input.shape
+    if quant_bits == 3:
+        if S % 11 != 0:
+            raise RuntimeError("For 3-bit quantization, steps must be divisible by 11")
+    else:
+        if group_length <= 0 or S % group_length != 0:
+            raise RuntimeError("steps must be divisible by group_length")
+        if S % (32 // quant_bits) != 0:
+            raise RuntimeError("steps must be divisible by (32 / quant_bits)")
+    _need_gpu(input)
+    vpw = _values_per_word(quant_bits)
+    code = torch.empty((B, H, R, S // vpw), dtype=torch.int32, device=input.device)
+    scale = torch.empty((B, H, R, S // group_length), dtype=input.dtype, device=input.device)
+    mn = torch.empty_like(scale)
+    _quantize_into(input, group_length, quant_bits, _lib.FMT_REF, _lib.SCALE_RECIPROCAL, code, scale, mn)
+    return code, scale, mn
+
+
+def _batched3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:
+    """[B, H, R, S] -> (tensor, batch stride, row stride) with (B, H) collapsible, unit last stride."""
+    B, H, R, S = t.shape
+    ok = (S <= 1 or t.stride(3) == 1) and (B <= 1 or t.stride(0) == H * t.stride(1))
+    ok = ok and (R <= 1 or t.stride(2) >= S) and (H <= 1 or t.stride(1) >= t.stride(2))
+    if not ok:
+        t = t.contiguous()
+    bs = t.stride(1) if B * H > 1 else max(R * max(t.stride(2), S), 1)
+    rs = t.stride(2) if R > 1 else max(S, 1)
+    return t, bs, rs
+
+
+def quantized_gemm(group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: torch.Tensor,
+                   zeros: torch.Tensor, bits: int, fmt: int = _lib.FMT_REF) -> torch.Tensor:
+    """out[b,h,m,:] = fA[b,h,m,:] @ dequant(qB[b,h',:,:]) with h' = h // (nh // nh_kv).
+
+    Reference: quantized_gemm, quant_cuda/csrc/dequantization_gemv_cuda.cu:127-248.
+    fA [B,nh,M,K] f16; qB [B,nh_kv,K,N/vpw] i32; scales, zeros [B,nh_kv,K,N/g] f16 -> [B,nh,M,N] f16.
+    The packed operands are read in place (views of a larger cache buffer are fine); GQA inputs
+    may be passed un-repeated.  `fmt` is an extension (dense 3-bit); the default is the reference's."""
+    if fA.dim() != 4 or qB.dim() != 4:
+        raise RuntimeError("Input tensors must be 4-dimensional")
+    _check_bits(bits)
+    B, nh, M, K = fA.shape
+    nh_kv = qB.shape[1]
+    if nh_kv == 0 or nh % nh_kv != 0:
+        raise RuntimeError("Total heads must be divisible by KV heads")
+    if bits == 3 and fmt == _lib.FMT_REF and group_size != 11:
+        raise RuntimeError("For 3-bit quantization, group size must be 11")
+    if fA.dtype != torch.float16 or scales.dtype != torch.float16 or zeros.dtype != torch.float16:
+        raise RuntimeError("expected scalar type Half for fA, scales and zeros")
+    if qB.dtype != torch.int32:
+        raise RuntimeError("expected scalar type Int for qB")
+    _need_gpu(fA, qB, scales, zeros)
+    if scales.dim() != 4 or zeros.dim() != 4 or scales.shape != zeros.shape:
+        raise RuntimeError("scales and zeros must be 4-dimensional and of equal shape")
+    if qB.shape[0] != B or qB.shape[2] != K or scales.shape[:3] != qB.shape[:3]:
+        raise RuntimeError("shape mismatch between fA, qB and scales")
+    N = zeros.shape[-1] * group_size  # dequantization_gemv_cuda.cu:184
+    L = _lib.load()
+    fA, x_bs, x_rs = _batched3(fA)
+    qB, c_bs, c_rs = _batched3(qB)
+    scales, s_bs, s_rs = _batched3(scales)
+    zeros, z_bs, z_rs = _batched3(zeros)
+    if (z_bs, z_rs) != (s_bs, s_rs):
+        zeros = zeros.contiguous()
+        scales = scales.contiguous()
+        scales, s_bs, s_rs = _batched3(scales)
+        zeros, z_bs, z_rs = _batched3(zeros)
+    out = torch.empty((B, nh, M, N), dtype=torch.float16, device=fA.device)
+    ws_bytes = L.kvmix_gemv_workspace_bytes(B * nh, M, K, N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=fA.device) if ws_bytes else None
+    with torch.cuda.device(fA.device):
+        _lib.check(L.kvmix_quantized_gemv(
+            group_size, fA.data_ptr(), x_bs, x_rs, qB.data_ptr(), c_bs, c_rs,
+            scales.data_ptr(), zeros.data_ptr(), s_bs, s_rs, bits, fmt, B * nh, nh // nh_kv,
+            M, K, N, out.data_ptr(), M * N, N, ws.data_ptr() if ws is not None else None,
+            ws_bytes, _stream(fA)))
+    return out
+
+
+def _append_checks(input, prev_scale, prev_min):
+    if input.dim() != 4:
+        raise RuntimeError("input_tensor must be a 4D tensor")
+    if input.dtype not in _DT:
+        raise RuntimeError(f"expected scalar type Float or Half but found {input.dtype}")
+    if prev_scale.dtype != input.dtype or prev_min.dtype != input.dtype:
+        raise RuntimeError("previous_scale / previous_min must have the input's dtype")
+
+
+def process_key_quantization_cuda(input: torch.Tensor, previous_code: torch.Tensor,
+                                  previous_scale: torch.Tensor, previous_min: torch.Tensor,
+                                  group_length: int, quant_bits: int):
+    """Append form for keys: input [B,H,D,n] (groups along n) is quantized and returned
+    concatenated after previous_* along the last dimension.
+
+    Reference: process_key_quantization_cuda, quant_cuda/csrc/quantization_cuda.cu:298-411.
+    The returned scale is (max-min)/qmax rounded to the input dtype (the reference's append
+    kernels divide in-kernel, :49-51,:149-151)."""
+    _append_checks(input, previous_scale, previous_min)
+    _check_bits(quant_bits)
+    B, H, D, n = input.shape
+    if quant_bits == 3:
+        if group_length != 11:
+            raise RuntimeError("For 3-bit quantization, group_length must be 11")
+        if n % 11 != 0:
+            raise RuntimeError("new_steps must be divisible by 11 for 3-bit quantization")
+    elif group_length <= 0 or n % group_length != 0:
+        raise RuntimeError("new_steps must be divisible by group_length")
+    _need_gpu(input, previous_code, previous_scale, previous_min)
+    vpw = _values_per_word(quant_bits)
+    if quant_bits != 3 and (group_length % vpw != 0 or n % vpw != 0):
+        raise RuntimeError(_lib.strerror(-9))
+    ow, og = previous_code.shape[3], previous_scale.shape[3]
+    code = torch.empty((B, H, D, ow + n // vpw), dtype=torch.int32, device=input.device)
+    scale = torch.empty((B, H, D, og + n // group_length), dtype=input.dtype, device=input.device)
+    mn = torch.empty_like(scale)
+    code[..., :ow].copy_(previous_code.reshape(B, H, D, ow))
+    scale[..., :og].copy_(previous_scale.reshape(B, H, D, og))
+    mn[..., :og].copy_(previous_min.reshape(B, H, D, og))
+    if n > 0:
+        _quantize_into(input, group_length, quant_bits, _lib.FMT_REF, _lib.SCALE_DIVIDE,
+                       code[..., ow:], scale[..., og:], mn[..., og:])
+    return code, scale, mn
+
+
+def process_value_quantization_cuda(input: torch.Tensor, previous_code: torch.Tensor,
+                                    previous_scale: torch.Tensor, previous_min: torch.Tensor,
+                                    group_length: int, quant_bits: int):
+    """Append form for values: input [B,H,n,D] (groups along D) is quantized and returned
+    concatenated after previous_* along the token dimension.
+
+    Reference: process_value_quantization_cuda, quant_cuda/csrc/quantization_cuda.cu:413-537.
+    3-bit follows the reference's placeholder branch literally (plain 3*j shifts, so the
+    eleventh code of a word keeps only its low two bits)."""
+    _append_checks(input, previous_scale, previous_min)
+    _check_bits(quant_bits)
+    B, H, n, D = input.shape
+    if quant_bits == 3:
+        if group_length != 11:
+            raise RuntimeError("For 3-bit quantization, group_length must be 11")
+        if D % 11 != 0:
+            raise RuntimeError("head_dim must be divisible by 11 for 3-bit quantization")
+    elif group_length <= 0 or D % group_length != 0:
+        raise RuntimeError("head_dim must be divisible by group_length")
+    _need_gpu(input, previous_code, previous_scale, previous_min)
+    vpw = _values_per_word(quant_bits)
+    if quant_bits != 3 and (group_length % vpw != 0 or D % vpw != 0):
+        raise RuntimeError(_lib.strerror(-9))
+    old = previous_code.shape[2]
+    wpt, gpt = D // vpw, D // group_length
+    code = torch.empty((B, H, old + n, wpt), dtype=torch.int32, device=input.device)
+    scale = torch.empty((B, H, old + n, gpt), dtype=input.dtype, device=input.device)
+    mn = torch.empty_like(scale)
+    code[:, :, :old].copy_(previous_code.reshape(B, H, old, wpt))
+    scale[:, :, :old].copy_(previous_scale.reshape(B, H, old, gpt))
+    mn[:, :, :old].copy_(previous_min.reshape(B, H, old, gpt))
+    if n > 0:
+        fmt = _lib.FMT_REF3_WRAP if quant_bits == 3 else _lib.FMT_REF
+        _quantize_into(input, group_length, quant_bits, fmt, _lib.SCALE_DIVIDE,
+                       code[:, :, old:], scale[:, :, old:], mn[:, :, old:])
+    return code, scale, mn

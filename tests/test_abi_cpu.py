@@ -1,0 +1,110 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports every symbol
+declared in include/kvmix_hip.h, maps error codes to the reference's messages, and the
+Python operators reject bad arguments before touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from kvmix_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from kvmix_amd import build_ext
+
+        build_ext.build()
+    return _lib.load()
+
+
+def test_header_symbols_are_exported(lib):
+    header = open(os.path.join(ROOT, "include", "kvmix_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(kvmix_[a-z_0-9]+)\s*\(", header))
+    assert declared >= {"kvmix_version", "kvmix_strerror", "kvmix_quant_pack_last_dim",
+                        "kvmix_quant_pack_key_tokens", "kvmix_gemv_workspace_bytes",
+                        "kvmix_quantized_gemv"}
+    for name in declared:
+        assert hasattr(lib, name), name
+    from kvmix_amd import _lib
+    assert set(_lib.EXPORTS) == declared
+
+
+def test_version_and_error_text(lib):
+    from kvmix_amd import _lib
+
+    assert lib.kvmix_version() >= 100
+    assert _lib.strerror(0) == "ok"
+    assert "1, 2, 3, 4" in _lib.strerror(-1)
+    assert "group_length must be 11" in _lib.strerror(-2)
+    assert "divisible by group_length" in _lib.strerror(-3)
+    assert "32 / quant_bits" in _lib.strerror(-4)
+    assert "divisible by KV heads" in _lib.strerror(-5)
+    codes = {_lib.strerror(c) for c in range(-12, 0)}
+    assert len(codes) == 12  # distinct text per code
+    with pytest.raises(RuntimeError, match="KV heads"):
+        _lib.check(-5)
+
+
+def test_host_validation_needs_no_gpu(lib):
+    """Argument errors are detected on the host before any launch (safe without a GPU)."""
+    q = lib.kvmix_quant_pack_last_dim
+    one = ctypes.c_void_p(16)
+    args = lambda **kw: [kw.get("x", one), kw.get("dt", 0), 1, 1, kw.get("steps", 64), 64, 64,
+                         kw.get("g", 32), kw.get("bits", 4), kw.get("fmt", 0), 0, one, 8, 8, one, one, 2, 2, None]
+    assert q(*args(bits=5)) == -1
+    assert q(*args(bits=3, g=32)) == -2
+    assert q(*args(g=48)) == -3
+    assert q(*args(bits=1, g=16, steps=48)) == -4
+    assert q(*args(dt=7)) == -6
+    assert q(*args(x=None)) == -7
+    assert q(*args(fmt=9)) == -10
+    g = lib.kvmix_quantized_gemv
+    gargs = lambda **kw: [kw.get("g", 32), one, 128, 128, one, 1024, 16, one, one, 512, 4, kw.get("bits", 4), 0,
+                          kw.get("samples", 4), kw.get("hpk", 1), 1, kw.get("K", 8), 128, one, 128, 128,
+                          None, 0, None]
+    assert g(*gargs(bits=0)) == -1
+    assert g(*gargs(samples=3, hpk=2)) == -5
+    assert g(*gargs(bits=3)) == -2
+    assert g(*gargs(g=48)) == -3
+    assert g(*gargs(g=4)) == -9     # a word of eight 4-bit codes would straddle two groups
+    assert lib.kvmix_gemv_workspace_bytes(32, 1, 4096, 128) > 0
+    assert lib.kvmix_gemv_workspace_bytes(0, 1, 4096, 128) == 0
+
+
+def test_python_ops_reject_bad_arguments_like_the_reference():
+    import KVmix
+
+    x = torch.zeros(1, 1, 2, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="For 3-bit quantization, group_length must be 11"):
+        KVmix.quantize_pack_last_dim_cuda(x, 32, 3)
+    with pytest.raises(RuntimeError, match="input_tensor must be a 4D tensor"):
+        KVmix.quantize_pack_last_dim_cuda(x[0], 32, 4)
+    with pytest.raises(RuntimeError, match="steps must be divisible by group_length"):
+        KVmix.quantize_pack_last_dim_cuda(x, 48, 4)
+    with pytest.raises(RuntimeError, match="steps must be divisible by 11"):
+        KVmix.quantize_pack_last_dim_cuda(x, 11, 3)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        KVmix.quantize_pack_last_dim_cuda(x, 32, 4)  # CPU tensors are refused: there is no CPU fallback
+    q = torch.zeros(1, 2, 64, 4, dtype=torch.int32)
+    s = torch.zeros(1, 2, 64, 1, dtype=torch.float16)
+    a = torch.zeros(1, 3, 1, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="Total heads must be divisible by KV heads"):
+        KVmix.quantized_gemm(32, a, q, s, s, 4)
+    with pytest.raises(RuntimeError, match="Supported quantization bits: 1, 2, 3, 4"):
+        KVmix.quantized_gemm(32, a[:, :2], q, s, s, 8)
+    with pytest.raises(RuntimeError, match="For 3-bit quantization, group size must be 11"):
+        KVmix.quantized_gemm(32, a[:, :2], q, s, s, 3)
+    with pytest.raises(RuntimeError, match="Input tensors must be 4-dimensional"):
+        KVmix.quantized_gemm(32, a[0], q, s, s, 4)
+    with pytest.raises(RuntimeError, match="new_steps must be divisible by group_length"):
+        KVmix.process_key_quantization_cuda(x, q[..., :0], s[..., :0], s[..., :0], 48, 4)
+    with pytest.raises(RuntimeError, match="head_dim must be divisible by 11"):
+        KVmix.process_value_quantization_cuda(x, q[..., :0], s[..., :0], s[..., :0], 11, 3)
+    assert sorted(KVmix.__all__) == sorted(["quantized_gemm", "quantize_pack_last_dim_cuda",
+                                            "process_value_quantization_cuda", "process_key_quantization_cuda"])

@@ -1,0 +1,235 @@
+"""GPU parity of the fused dequant-GEMV kernels against the CPU oracle
+(reference: quant_cuda/csrc/dequantization_gemv_cuda.cu:7-248).  Tolerance: see helpers.gemv_close
+(1e-3 relative plus the fp32 accumulation term)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import gemv_close, kv_like, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def tt(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def run_case(oracle, dev, bits, g, B, nh, nkv, K, N, seed=0, M=1):
+    import KVmix
+
+    rng = np.random.default_rng(seed)
+    w = kv_like(rng, (B, nkv, K, N), outlier_axis=2, n_outliers=min(2, K))
+    code, scale, zero = oracle.quantize_pack_last_dim(w, g, bits)
+    x = rng.standard_normal((B, nh, M, K)).astype(np.float16)
+    want16, want64, abs64 = oracle.quantized_gemm(g, x, code, scale, zero, bits, want_f64=True)
+    got = KVmix.quantized_gemm(g, tt(x, dev), tt(code, dev), tt(scale, dev), tt(zero, dev), bits)
+    assert got.shape == (B, nh, M, N) and got.dtype == torch.float16
+    got = got.cpu().numpy()
+    ok, worst = gemv_close(got, want64, abs64)
+    assert ok, ("vs float64", bits, g, K, N, worst)
+    ok, worst = gemv_close(got, want16.astype(np.float64), abs64)
+    assert ok, ("vs reference-order fp32", bits, g, K, N, worst)
+    return got
+
+
+QK = [(4, 32), (2, 32), (1, 32), (3, 11)]
+
+
+@pytest.mark.parametrize("bits,g", QK)
+def test_qk_shape(oracle, dev, bits, g):
+    """q.K^T: K = head_dim 128, N = quantized tokens (ragged counts included)."""
+    for tokens in (g, g * 3, g * 65, g * 131):
+        run_case(oracle, dev, bits, g, B=2, nh=4, nkv=4, K=128, N=tokens, seed=tokens)
+
+
+@pytest.mark.parametrize("bits,g", [(4, 32), (2, 32), (1, 32)])
+def test_pv_shape(oracle, dev, bits, g):
+    """p.V: K = quantized tokens, N = head_dim 128 (64 and 256 too); split-K and tails."""
+    for tokens in (1, 15, 32, 100, 257, 2048 + 17):
+        run_case(oracle, dev, bits, g, B=1, nh=4, nkv=4, K=tokens, N=128, seed=tokens)
+    run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=333, N=64, seed=5)
+    run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=333, N=256, seed=6)
+    run_case(oracle, dev, bits, g, B=40, nh=32, nkv=32, K=96, N=128, seed=7)   # many samples: no split
+
+
+@pytest.mark.parametrize("bits,g", QK)
+def test_gqa_head_mapping(oracle, dev, bits, g):
+    run_case(oracle, dev, bits, g, B=2, nh=8, nkv=2, K=128, N=g * 8 * (1 if bits != 3 else 1), seed=21)
+    if bits != 3:
+        run_case(oracle, dev, bits, g, B=2, nh=8, nkv=2, K=200, N=128, seed=22)
+
+
+@pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
+def test_generic_shapes(oracle, dev, bits, g):
+    """Group sizes and shapes outside the fast kernels (including a 3-bit p.V shape)."""
+    unit = int(np.lcm(g, oracle.values_per_word(bits)))
+    run_case(oracle, dev, bits, g, B=1, nh=2, nkv=1, K=37, N=unit * 5, seed=31)
+    run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=260, N=unit * 2, seed=32)
+
+
+def test_rows_beyond_m1_use_the_same_formula(oracle, dev):
+    run_case(oracle, dev, 4, 32, B=1, nh=2, nkv=2, K=128, N=256, seed=41, M=3)
+    run_case(oracle, dev, 2, 32, B=1, nh=2, nkv=1, K=300, N=128, seed=42, M=2)
+
+
+@pytest.mark.parametrize("bits,g", QK)
+def test_closed_form_cases(oracle, dev, bits, g):
+    import KVmix
+
+    rng = np.random.default_rng(bits)
+    B, nh, K = 1, 2, 128
+    N = int(np.lcm(g, oracle.values_per_word(bits))) * 6
+    qmax = (1 << bits) - 1
+    q = rng.integers(0, qmax + 1, size=(B, nh, K, N))
+    if bits == 3:
+        q[..., 10::11] &= 3
+    code = oracle.pack_np(q, bits)
+    ones = np.ones((B, nh, K, N // g), np.float16)
+    zeros = np.zeros_like(ones)
+    x1 = np.ones((B, nh, 1, K), np.float16)
+    # all-ones x, scale 1, zero 0 -> exact integer column sums
+    out = KVmix.quantized_gemm(g, tt(x1, dev), tt(code, dev), tt(ones, dev), tt(zeros, dev), bits).cpu().numpy()
+    assert np.array_equal(out.astype(np.int64)[:, :, 0], q.sum(axis=2))
+    # one-hot x -> one dequantized row, bit-exact after fp16 rounding
+    scale = (rng.random((B, nh, K, N // g)) + 0.5).astype(np.float16)
+    zero = rng.standard_normal((B, nh, K, N // g)).astype(np.float16)
+    e = np.zeros((B, nh, 1, K), np.float16)
+    e[..., 77] = 1
+    out = KVmix.quantized_gemm(g, tt(e, dev), tt(code, dev), tt(scale, dev), tt(zero, dev), bits).cpu().numpy()
+    row = np.repeat(scale.astype(np.float64), g, -1)[:, :, 77] * q[:, :, 77] + np.repeat(zero.astype(np.float64), g, -1)[:, :, 77]
+    assert same_bits(out[:, :, 0], row.astype(np.float16))
+    # scale 0 -> sum_k x[k] zero[k, n/g]
+    x = rng.standard_normal((B, nh, 1, K)).astype(np.float16)
+    out = KVmix.quantized_gemm(g, tt(x, dev), tt(code, dev), tt(zeros, dev), tt(zero, dev), bits).cpu().numpy()
+    want = np.repeat(np.einsum("bhmk,bhkg->bhmg", x.astype(np.float64), zero.astype(np.float64)), g, -1)
+    ab = np.repeat(np.einsum("bhmk,bhkg->bhmg", np.abs(x.astype(np.float64)), np.abs(zero.astype(np.float64))), g, -1)
+    ok, worst = gemv_close(out, want, ab)
+    assert ok, worst
+
+
+def test_strided_views_of_a_larger_cache_and_sliced_probabilities(oracle, dev):
+    """Operands passed as views (capacity-padded cache, p[..., :Tq] slice) are read in place."""
+    import KVmix
+
+    rng = np.random.default_rng(8)
+    B, H, D, Tq, cap = 2, 4, 128, 96, 256
+    k = kv_like(rng, (B, H, D, Tq))
+    code, scale, zero = oracle.quantize_pack_last_dim(k, 32, 4)
+    cbuf = torch.zeros(B, H, D, cap // 8, dtype=torch.int32, device=dev)
+    sbuf = torch.zeros(B, H, D, cap // 32, dtype=torch.float16, device=dev)
+    zbuf = torch.zeros_like(sbuf)
+    cbuf[..., : Tq // 8] = tt(code, dev)
+    sbuf[..., : Tq // 32] = tt(scale, dev)
+    zbuf[..., : Tq // 32] = tt(zero, dev)
+    q = rng.standard_normal((B, H, 1, D)).astype(np.float16)
+    got = KVmix.quantized_gemm(32, tt(q, dev), cbuf[..., : Tq // 8], sbuf[..., : Tq // 32], zbuf[..., : Tq // 32], 4)
+    _, w64, a64 = oracle.quantized_gemm(32, q, code, scale, zero, 4, want_f64=True)
+    ok, worst = gemv_close(got.cpu().numpy(), w64, a64)
+    assert ok, worst
+    # p.V with p a slice of the probability row (models/modeling_llama_KVmix.py:205-206)
+    v = kv_like(rng, (B, H, Tq, D))
+    code, scale, zero = oracle.quantize_pack_last_dim(v, 32, 2)
+    p = rng.random((B, H, 1, Tq + 40)).astype(np.float16)
+    got = KVmix.quantized_gemm(32, tt(p, dev)[..., :Tq], tt(code, dev), tt(scale, dev), tt(zero, dev), 2)
+    _, w64, a64 = oracle.quantized_gemm(32, np.ascontiguousarray(p[..., :Tq]), code, scale, zero, 2, want_f64=True)
+    ok, worst = gemv_close(got.cpu().numpy(), w64, a64)
+    assert ok, worst
+
+
+def test_empty_k_gives_zeros(dev):
+    import KVmix
+
+    q = torch.zeros(1, 2, 1, 0, dtype=torch.float16, device=dev)
+    code = torch.zeros(1, 2, 0, 16, dtype=torch.int32, device=dev)
+    sz = torch.zeros(1, 2, 0, 4, dtype=torch.float16, device=dev)
+    out = KVmix.quantized_gemm(32, q, code, sz, sz, 4)
+    assert out.shape == (1, 2, 1, 128) and (out == 0).all()
+
+
+def test_config0_single_layer(oracle, dev):
+    """BASELINE config 0: B=1, 32 heads, head_dim 128, 4096 tokens, 4-bit, group 32, 128-token
+    fp16 window; K, V ~N(0,1) with 4 outlier channels per head x10; codes bit-exact, q.K^T and
+    softmax.V within tolerance of the oracle."""
+    import KVmix
+
+    torch.manual_seed(0)
+    B, H, D, T, R, g, bits = 1, 32, 128, 4096, 128, 32, 4
+    K = torch.randn(B, H, T, D).half()
+    V = torch.randn(B, H, T, D).half()
+    for h in range(H):
+        ch = torch.randperm(D)[:4]
+        K[:, h, :, ch] *= 10
+        V[:, h, :, ch] *= 10
+    q = torch.randn(B, H, 1, D).half()
+    Tq = T - R
+    Kq_in = K[:, :, :Tq].transpose(2, 3).contiguous()
+    Vq_in = V[:, :, :Tq].contiguous()
+    kc, ks, km = KVmix.quantize_pack_last_dim_cuda(Kq_in.to(dev), g, bits)
+    vc, vs, vm = KVmix.quantize_pack_last_dim_cuda(Vq_in.to(dev), g, bits)
+    okc, oks, okm = oracle.quantize_pack_last_dim(Kq_in.numpy(), g, bits)
+    ovc, ovs, ovm = oracle.quantize_pack_last_dim(Vq_in.numpy(), g, bits)
+    for a, b in ((kc, okc), (ks, oks), (km, okm), (vc, ovc), (vs, ovs), (vm, ovm)):
+        assert same_bits(a.cpu().numpy(), b)
+    att_q = KVmix.quantized_gemm(g, q.to(dev), kc, ks, km, bits)
+    o16, o64, a64 = oracle.quantized_gemm(g, q.numpy(), okc, oks, okm, bits, want_f64=True)
+    ok, worst = gemv_close(att_q.cpu().numpy(), o64, a64)
+    assert ok, worst
+    # the rest of the decode step exactly as models/modeling_llama_KVmix.py:184-211 does it
+    att_f = torch.matmul(q.to(dev), K[:, :, Tq:].to(dev).transpose(2, 3))
+    w = torch.cat([att_q.float(), att_f.float()], -1) / (D ** 0.5)
+    p = torch.softmax(w, dim=-1, dtype=torch.float32).half()
+    out = KVmix.quantized_gemm(g, p[..., :Tq], vc, vs, vm, bits) + torch.matmul(p[..., Tq:], V[:, :, Tq:].to(dev))
+    # oracle on the same probabilities (isolates the p.V kernel), then end to end
+    pn = p.cpu().numpy()
+    _, v64, va64 = oracle.quantized_gemm(g, np.ascontiguousarray(pn[..., :Tq]), ovc, ovs, ovm, bits, want_f64=True)
+    got_q = KVmix.quantized_gemm(g, p[..., :Tq], vc, vs, vm, bits).cpu().numpy()
+    ok, worst = gemv_close(got_q, v64, va64)
+    assert ok, worst
+    cache = (okc, K[:, :, Tq:].numpy(), oks, okm, ovc, V[:, :, Tq:].numpy(), ovs, ovm, T)
+    k_new = np.zeros((B, H, 0, D), np.float16)
+    want_out, want_p, _ = oracle.attention_decode_step(q.numpy(), k_new, k_new, cache, bits, bits, 1.0, 1.0, g)
+    np.testing.assert_allclose(pn.astype(np.float64), want_p.astype(np.float64), rtol=4e-3, atol=1e-5)
+    np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want_out.astype(np.float64), rtol=4e-3, atol=4e-3)
+
+
+def test_full_size_properties_b16_t8192(dev):
+    """Target shape (B=16, 32 heads, 8064 quantized tokens, head_dim 128), checked through
+    properties that need no CPU oracle: integer column sums (exact), one-hot rows (exact),
+    and agreement with torch's own fp32 matmul of the dequantized cache on a slice."""
+    import KVmix
+
+    torch.manual_seed(1)
+    B, H, D, Tq, g = 16, 32, 128, 8064, 32
+    for bits in (4, 2):
+        qmax = (1 << bits) - 1
+        vpw = 32 // bits
+        # keys: [B,H,D,Tq/vpw]
+        kcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq // vpw), dtype=torch.int64, device=dev).to(torch.int32)
+        ones = torch.ones(B, H, D, Tq // g, dtype=torch.float16, device=dev)
+        shifts = torch.arange(0, 32, bits, device=dev, dtype=torch.int32)
+        x1 = torch.ones(B, H, 1, D, dtype=torch.float16, device=dev)
+        out = KVmix.quantized_gemm(g, x1, kcode, ones, torch.zeros_like(ones), bits)
+        sums = torch.zeros(B, H, Tq, dtype=torch.int32, device=dev)
+        for b0 in range(0, B, 4):
+            qk = ((kcode[b0:b0 + 4].unsqueeze(-1) >> shifts) & qmax).reshape(4, H, D, Tq)
+            sums[b0:b0 + 4] = qk.sum(2)
+        assert torch.equal(out[:, :, 0].to(torch.int32), sums)          # sums <= 128*15 are exact in fp16
+        # values: [B,H,Tq,D/vpw]; one-hot p picks one dequantized row exactly
+        vcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D // vpw), dtype=torch.int64, device=dev).to(torch.int32)
+        vs = (torch.rand(B, H, Tq, D // g, device=dev) + 0.5).half()
+        vz = torch.randn(B, H, Tq, D // g, device=dev).half()
+        p = torch.zeros(B, H, 1, Tq, dtype=torch.float16, device=dev)
+        row = 5003
+        p[..., row] = 1
+        out = KVmix.quantized_gemm(g, p, vcode, vs, vz, bits)
+        qv = ((vcode[:, :, row].unsqueeze(-1) >> shifts) & qmax).reshape(B, H, D).float()
+        want = (vs[:, :, row].float().repeat_interleave(g, -1) * qv + vz[:, :, row].float().repeat_interleave(g, -1)).half()
+        assert torch.equal(out[:, :, 0], want)
+        # dense check on two batch entries with torch's fp32 matmul
+        pr = torch.softmax(torch.randn(2, H, 1, Tq, device=dev), -1).half()
+        out = KVmix.quantized_gemm(g, pr, vcode[:2], vs[:2], vz[:2], bits).float()
+        qv = ((vcode[:2].unsqueeze(-1) >> shifts) & qmax).reshape(2, H, Tq, D).float()
+        deq = vs[:2].float().repeat_interleave(g, -1) * qv + vz[:2].float().repeat_interleave(g, -1)
+        ref = torch.matmul(pr.float(), deq)
+        ab = torch.matmul(pr.float().abs(), deq.abs())
+        assert ((out - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
