@@ -8,23 +8,34 @@
 // (dequantization_gemv_cuda.cu:154-171); here nothing is copied.
 //
 // The sum is split as  sum_k (x_k * scale_k) * code_kn  +  sum_k x_k * zero_k : the second
-// term is one fma per (k, group) instead of one per element, and the first needs one
-// int->float conversion and one fma per element.  All accumulation is fp32.
+// term is one fma per (k, group) instead of one per element, and the first needs no
+// int->float conversion (see mix2 below).  All accumulation is fp32.
+//
+// Memory plan (the kernels are HBM-bound; measured on MI355X, 2-byte loads of scale/zero
+// issued per lane cost a third of the run time, so they never happen):
+//   * packed codes: one 128/64/32-bit load per lane and row, straight to registers;
+//   * scale, zero and x: fetched with 128-bit loads by whichever lane the address falls to,
+//     combined (x*scale, or (scale, zero) pairs) and parked in a wave-private LDS tile, from
+//     which the consuming lane reads one dword per row.  Wave-private means no block barrier
+//     in the streaming loop.
 //
 // Kernels
 //   gemv_cols   q.K^T shape (K = head_dim small, N = tokens large).  A lane owns one
-//               quantization group of N (32 codes, or one 11-code word in the reference's
-//               3-bit format) and walks down the K rows: no cross-lane reduction at all.
-//               The K rows are split over the waves of the block, partials meet in LDS.
-//               x (the query) is staged in LDS as fp32.
-//   gemv_rows   p.V shape (K = tokens large, N = head_dim small).  A lane owns one group
-//               of one row; a wave covers 64/(N/32) rows per load.  Per-lane fp32
-//               accumulators, butterfly reduction across the row lanes, LDS across waves,
-//               split-K across blocks with fp32 partials in the workspace.
+//               quantization group of N (32 codes, or one 11-code word of the reference's
+//               3-bit format) for a quarter / half / all of the K rows (RQ = 4 / 2 / 1 row
+//               sections per wave); the sections meet in a butterfly over lanes at the end.
+//   gemv_rows   p.V shape (K = tokens large, N = head_dim small).  A lane owns one group of
+//               one row; a wave walks a contiguous chunk of rows, 8 row tiles in flight.
+//               Butterfly across the row lanes, LDS across waves, optional split-K across
+//               blocks with fp32 partials in the caller's workspace.
 //   gemv_generic  any shape/group: one thread per packed word, serial over K.
 //   reduce_splits sums the split-K partials and stores fp16.
 
 #include "kvmix_common.h"
+
+#ifndef KVMIX_TARGET_WAVES
+#define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
+#endif
 
 namespace kvmix {
 
@@ -53,63 +64,87 @@ struct GemvArgs {
 template <int MODE>
 struct Fmt {
     static constexpr int BITS = MODE == 30 ? 3 : MODE;
-    static constexpr int VALS = MODE == 3 ? 11 : 32;                  // codes per group unit
+    static constexpr int VALS = MODE == 3 ? 11 : 32;                       // codes per group unit
     static constexpr int WORDS = MODE == 3 ? 1 : (MODE == 30 ? 3 : MODE);  // words per group unit
 };
 
-// 4-byte-aligned vector of W words: lets the compiler use one wide load where rows are
-// only dword aligned (global memory tolerates dword-aligned wide loads on gfx9).
+// Vectors with relaxed alignment: the compiler still emits one wide global load, and gfx9
+// global memory accepts any byte alignment (a misaligned access only costs extra cycles).
 template <int W>
 struct __attribute__((packed, aligned(4))) Words {
     uint32_t v[W];
 };
+struct __attribute__((packed, aligned(2))) Half8 {
+    uint16_t v[8];
+};
+
+// Integer codes are fed to the multiplier as fp16 SUBNORMALS: a 16-bit pattern p < 2048 read
+// as binary16 is exactly p * 2^-24 (the first two binades share one ulp).  Masking a field of
+// the packed word in place therefore yields two fp16 operands (low and high half of the
+// register) with no shift and no int->float conversion, and v_fma_mix_f32 multiplies an fp32
+// by an fp16 half directly into an fp32 accumulator.  The 2^-24 and the field's bit offset are
+// folded into the fp32 multiplier (powers of two: exact).
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void mix2(float q, uint32_t m, float &acc_lo, float &acc_hi)
+{
+    const half2_t h = __builtin_bit_cast(half2_t, m);
+    acc_lo = fmaf(q, (float)h.x, acc_lo);
+    acc_hi = fmaf(q, (float)h.y, acc_hi);
+}
+
+__device__ __forceinline__ void mix1(float q, uint32_t m, float &acc)
+{
+    const half2_t h = __builtin_bit_cast(half2_t, m);
+    acc = fmaf(q, (float)h.x, acc);
+}
 
 // acc[i] += qs * code_i for the VALS codes held in w[]; qs = x_k * scale_k.
 template <int MODE>
 __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, float *acc)
 {
+    const float q0 = qs * 16777216.0f;  // 2^24 undoes the subnormal scaling
     if constexpr (MODE == 4) {
-        const float qs16 = qs * 0.0625f;  // exact: the high nibble is read as 16*code
+        const float q1 = q0 * 0.0625f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t lo = w[j] & 0x0F0F0F0Fu, hi = w[j] & 0xF0F0F0F0u;
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                acc[8 * j + 2 * b] = fmaf(qs, (float)((lo >> (8 * b)) & 0xffu), acc[8 * j + 2 * b]);
-                acc[8 * j + 2 * b + 1] = fmaf(qs16, (float)((hi >> (8 * b)) & 0xffu), acc[8 * j + 2 * b + 1]);
-            }
+            const uint32_t v = w[j], v8 = w[j] >> 8;
+            float *a = acc + 8 * j;  // nibble i sits at bit 4i: low half 0..3, high half 4..7
+            mix2(q0, v & 0x000F000Fu, a[0], a[4]);
+            mix2(q1, v & 0x00F000F0u, a[1], a[5]);
+            mix2(q0, v8 & 0x000F000Fu, a[2], a[6]);
+            mix2(q1, v8 & 0x00F000F0u, a[3], a[7]);
         }
     } else if constexpr (MODE == 2) {
-        const float q1 = qs, q4 = qs * 0.25f, q16 = qs * 0.0625f, q64 = qs * 0.015625f;
+        const float q1 = q0 * 0.25f, q2 = q0 * 0.0625f, q3 = q0 * 0.015625f;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const uint32_t m0 = w[j] & 0x03030303u, m1 = w[j] & 0x0C0C0C0Cu, m2 = w[j] & 0x30303030u,
-                           m3 = w[j] & 0xC0C0C0C0u;
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                float *a = acc + 16 * j + 4 * b;
-                a[0] = fmaf(q1, (float)((m0 >> (8 * b)) & 0xffu), a[0]);
-                a[1] = fmaf(q4, (float)((m1 >> (8 * b)) & 0xffu), a[1]);
-                a[2] = fmaf(q16, (float)((m2 >> (8 * b)) & 0xffu), a[2]);
-                a[3] = fmaf(q64, (float)((m3 >> (8 * b)) & 0xffu), a[3]);
-            }
+            const uint32_t v = w[j], v8 = w[j] >> 8;
+            float *a = acc + 16 * j;  // code i at bit 2i: low half 0..7, high half 8..15
+            mix2(q0, v & 0x00030003u, a[0], a[8]);
+            mix2(q1, v & 0x000C000Cu, a[1], a[9]);
+            mix2(q2, v & 0x00300030u, a[2], a[10]);
+            mix2(q3, v & 0x00C000C0u, a[3], a[11]);
+            mix2(q0, v8 & 0x00030003u, a[4], a[12]);
+            mix2(q1, v8 & 0x000C000Cu, a[5], a[13]);
+            mix2(q2, v8 & 0x00300030u, a[6], a[14]);
+            mix2(q3, v8 & 0x00C000C0u, a[7], a[15]);
         }
     } else if constexpr (MODE == 1) {
         float qv[8];
-        qv[0] = qs;
+        qv[0] = q0;
 #pragma unroll
         for (int s = 1; s < 8; s++) qv[s] = qv[s - 1] * 0.5f;
+        const uint32_t v = w[0], v8 = w[0] >> 8;  // bit i: low half 0..15, high half 16..31
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const uint32_t m = w[0] & (0x01010101u << s);
-#pragma unroll
-            for (int b = 0; b < 4; b++)
-                acc[8 * b + s] = fmaf(qv[s], (float)((m >> (8 * b)) & 0xffu), acc[8 * b + s]);
+            mix2(qv[s], v & (0x00010001u << s), acc[s], acc[16 + s]);
+            mix2(qv[s], v8 & (0x00010001u << s), acc[8 + s], acc[24 + s]);
         }
     } else if constexpr (MODE == 3) {
 #pragma unroll
-        for (int i = 0; i < 10; i++) acc[i] = fmaf(qs, (float)((w[0] >> (3 * i)) & 7u), acc[i]);
-        acc[10] = fmaf(qs, (float)(w[0] >> 30), acc[10]);
+        for (int i = 0; i < 10; i++) mix1(q0, (w[0] >> (3 * i)) & 7u, acc[i]);
+        mix1(q0, w[0] >> 30, acc[10]);
     } else {  // dense 3-bit stream over three words
         const uint64_t lo = (uint64_t)w[0] | ((uint64_t)w[1] << 32);
         const uint64_t hi = (uint64_t)w[1] | ((uint64_t)w[2] << 32);
@@ -117,103 +152,196 @@ __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, flo
         for (int i = 0; i < 32; i++) {
             const int bit = 3 * i;
             const uint32_t c = bit < 32 ? (uint32_t)(lo >> bit) & 7u : (uint32_t)(hi >> (bit - 32)) & 7u;
-            acc[i] = fmaf(qs, (float)c, acc[i]);
+            mix1(q0, c, acc[i]);
         }
     }
 }
 
+// LDS traffic between lanes of ONE wave: the wave's instructions execute in order, so a
+// ds_read issued after a ds_write sees it; this only stops the compiler from moving them.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // ---------------------------------------------------------------------------------------
-// gemv_cols: lanes along N (one group per lane), waves split K.  blockDim = (64, KW).
-// grid = (ceil(groups/64), samples, M).  Dynamic LDS: K floats (x) + KW*VALS*64 floats.
+// gemv_cols<MODE, RQ>
+//   wave tile  = GL = 64/RQ consecutive groups of N;  lane = (rq, gl): row section rq, group gl
+//   row chunk  = KC = 2048/GL rows (8 KiB of (scale, zero) pairs per wave in LDS); inside a
+//                chunk every lane walks KC/RQ = 32 rows of its section, 8 rows per load batch
+//   block = (64, NW) waves on NW neighbouring tiles; grid = (tiles/NW, samples, M)
 // ---------------------------------------------------------------------------------------
-template <int MODE>
-__global__ void __launch_bounds__(256) gemv_cols(GemvArgs a)
+constexpr int kColsWaves = 4;
+
+template <int MODE, int RQ>
+__global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
 {
     using F = Fmt<MODE>;
     constexpr int VALS = F::VALS, WORDS = F::WORDS;
-    extern __shared__ float lds[];
-    float *xs = lds;
-    float *red = lds + ((a.K + 63) & ~(int64_t)63);
+    constexpr int GL = kWave / RQ;      // groups per wave tile
+    constexpr int KC = 2048 / GL;       // rows per chunk
+    constexpr int RPL = KC / RQ;        // rows per lane per chunk (= 32)
+    constexpr int U = 8;                // rows whose code loads are in flight together
+    constexpr int SEGS = GL / 8;        // 8-group segments per staged row
+    static_assert(RPL == 32 && RPL % U == 0, "chunk geometry");
+
+    __shared__ uint32_t sz_lds[kColsWaves][KC * GL];  // (scale | zero << 16) per (row, group)
+    __shared__ float x_lds[kColsWaves][KC];
 
     const int lane = threadIdx.x;
     const int wy = threadIdx.y;
-    const int KW = blockDim.y;
+    const int rq = lane / GL;
+    const int gl = lane % GL;
     const int64_t sample = blockIdx.y;
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
     const int64_t ngroups = a.N / VALS;
-    const int64_t G = (int64_t)blockIdx.x * kWave + lane;
-    const bool active = G < ngroups;
+    const int64_t g0 = ((int64_t)blockIdx.x * kColsWaves + wy) * GL;
+    if (g0 >= ngroups) return;  // whole wave outside (there is no block-level barrier below)
+    const int64_t G = g0 + gl;
+    const bool col_ok = G < ngroups;
+    const int64_t Gc = col_ok ? G : ngroups - 1;  // clamped: loads stay in bounds, results dropped
 
-    const __half *xp = a.x + sample * a.x_bs + m * a.x_rs;
-    for (int64_t k = wy * kWave + lane; k < a.K; k += KW * kWave) xs[k] = __half2float(xp[k]);
-    __syncthreads();
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
+    const uint32_t *cp = a.code + kv * a.c_bs + Gc * WORDS;
+    const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
+    const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
+    uint32_t *szw = sz_lds[wy];
+    float *xw = x_lds[wy];
 
     float acc[VALS];
 #pragma unroll
     for (int i = 0; i < VALS; i++) acc[i] = 0.f;
     float zsum = 0.f;
 
-    if (active) {
-        const int64_t kper = (a.K + KW - 1) / KW;
-        const int64_t k0 = wy * kper;
-        const int64_t k1 = k0 + kper < a.K ? k0 + kper : a.K;
-        const uint32_t *cp = a.code + kv * a.c_bs + G * WORDS + k0 * a.c_rs;
-        const __half *sp = a.scale + kv * a.s_bs + G + k0 * a.s_rs;
-        const __half *zp = a.zero + kv * a.s_bs + G + k0 * a.s_rs;
-#pragma unroll 4
-        for (int64_t k = k0; k < k1; k++) {
-            const Words<WORDS> w = *reinterpret_cast<const Words<WORDS> *>(cp);
-            const float s = __half2float(*sp);
-            const float z = __half2float(*zp);
-            const float xv = xs[k];
-            zsum = fmaf(xv, z, zsum);
-            accumulate_unit<MODE>(w.v, xv * s, acc);
-            cp += a.c_rs;
-            sp += a.s_rs;
-            zp += a.s_rs;
-        }
-    }
+    for (int64_t kc = 0; kc < a.K; kc += KC) {
+        const int rows = (int)(a.K - kc < KC ? a.K - kc : KC);
+        // ---- stage (scale, zero) of rows [kc, kc+rows) x groups [g0, g0+GL) and x[kc..] ----
 #pragma unroll
-    for (int i = 0; i < VALS; i++) acc[i] += zsum;
+        for (int it = 0; it < (KC * SEGS) / kWave; it++) {
+            const int idx = it * kWave + lane;
+            const int row = idx / SEGS, seg = idx % SEGS;
+            const int64_t col = g0 + seg * 8;
+            uint16_t sv[8], zv[8];
+            if (row < rows && col + 8 <= ngroups) {
+                const Half8 s8 = *reinterpret_cast<const Half8 *>(sp + (kc + row) * a.s_rs + col);
+                const Half8 z8 = *reinterpret_cast<const Half8 *>(zp + (kc + row) * a.s_rs + col);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    sv[e] = s8.v[e];
+                    zv[e] = z8.v[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const bool ok = row < rows && col + e < ngroups;
+                    sv[e] = ok ? sp[(kc + row) * a.s_rs + col + e] : (uint16_t)0;
+                    zv[e] = ok ? zp[(kc + row) * a.s_rs + col + e] : (uint16_t)0;
+                }
+            }
+            uint4 lo, hi;
+            lo.x = sv[0] | ((uint32_t)zv[0] << 16);
+            lo.y = sv[1] | ((uint32_t)zv[1] << 16);
+            lo.z = sv[2] | ((uint32_t)zv[2] << 16);
+            lo.w = sv[3] | ((uint32_t)zv[3] << 16);
+            hi.x = sv[4] | ((uint32_t)zv[4] << 16);
+            hi.y = sv[5] | ((uint32_t)zv[5] << 16);
+            hi.z = sv[6] | ((uint32_t)zv[6] << 16);
+            hi.w = sv[7] | ((uint32_t)zv[7] << 16);
+            uint4 *dst = reinterpret_cast<uint4 *>(szw + row * GL + seg * 8);
+            dst[0] = lo;
+            dst[1] = hi;
+        }
+        for (int r = lane; r < KC; r += kWave) xw[r] = r < rows ? h16_to_f32(xp[kc + r]) : 0.f;
+        wave_lds_fence();
 
-    __half *op = a.out + sample * a.o_bs + m * a.o_rs + G * VALS;
-    if (KW == 1) {
-        if (active) {
+        // ---- stream the codes: lane walks rows [rq*RPL, rq*RPL + RPL) of the chunk ----
+        const int r0 = rq * RPL;
+#pragma unroll 1
+        for (int b = 0; b < RPL; b += U) {
+            Words<WORDS> w[U];
 #pragma unroll
-            for (int i = 0; i < VALS; i++) op[i] = __float2half_rn(acc[i]);
+            for (int u = 0; u < U; u++) {
+                int64_t k = kc + r0 + b + u;
+                k = k < a.K ? k : a.K - 1;  // rows past the end: x was staged as 0
+                w[u] = *reinterpret_cast<const Words<WORDS> *>(cp + k * a.c_rs);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int r = r0 + b + u;
+                const half2_t sz = __builtin_bit_cast(half2_t, szw[r * GL + gl]);
+                const float xv = xw[r];
+                zsum = fmaf(xv, (float)sz.y, zsum);
+                accumulate_unit<MODE>(w[u].v, xv * (float)sz.x, acc);
+            }
         }
-        return;
+        wave_lds_fence();  // the next chunk overwrites the tile
     }
-    // cross-wave reduction: red[wy][i][lane]
+
+    // ---- combine the RQ row sections (butterfly over lanes), store fp16 ----
 #pragma unroll
-    for (int i = 0; i < VALS; i++) red[(wy * VALS + i) * kWave + lane] = acc[i];
-    __syncthreads();
-    if (!active) return;
-    for (int i = wy; i < VALS; i += KW) {
-        float r = 0.f;
-        for (int w = 0; w < KW; w++) r += red[(w * VALS + i) * kWave + lane];
-        op[i] = __float2half_rn(r);
+    for (int i = 0; i < VALS; i++) {
+        float v = acc[i] + zsum;
+#pragma unroll
+        for (int off = GL; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+        acc[i] = v;
+    }
+    if (!col_ok) return;
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + G * VALS;
+    if constexpr (VALS % RQ == 0 && (VALS / RQ) % 2 == 0) {
+        // every lane holds all sums: section rq stores its share of the group's outputs
+        constexpr int PER = VALS / RQ;
+#pragma unroll
+        for (int s = 0; s < RQ; s++) {
+            if (rq == s) {
+#pragma unroll
+                for (int i = 0; i < PER; i += 2) {
+                    const uint32_t pk =
+                        f32_to_h16(acc[s * PER + i]) | ((uint32_t)f32_to_h16(acc[s * PER + i + 1]) << 16);
+                    __builtin_memcpy(op + s * PER + i, &pk, 4);
+                }
+            }
+        }
+    } else {
+        if (rq == 0) {
+#pragma unroll
+            for (int i = 0; i < VALS; i++) op[i] = f32_to_h16(acc[i]);
+        }
     }
 }
 
 // ---------------------------------------------------------------------------------------
-// gemv_rows: lanes along (row, group); LPR = N/32 lanes per row; blockDim = (64, KW).
-// grid = (splits, samples, M).  Static LDS: KW * N floats.
+// gemv_rows<MODE, LPR>
+//   LPR = N/32 lanes per row (one 32-code group each), RPW = 64/LPR rows per tile,
+//   chunk = 8 tiles = 512/LPR rows: its scale array is 512 halves = one 128-bit load per lane.
+//   The lane that loads scale/zero element e also loads that row's x, forms x*scale (to LDS,
+//   fp32) and accumulates x*zero privately; the zero term is reduced once at the end.
+//   Chunks of a block's row range go round-robin to its KW waves.
+//   block = (64, KW); grid = (splits, samples, M); dynamic LDS = KW * (512 + N) floats.
+//   Requires scale/zero rows to be contiguous (row stride == LPR).
 // ---------------------------------------------------------------------------------------
+constexpr int kRowsMaxWaves = 16;
+
 template <int MODE, int LPR>
-__global__ void __launch_bounds__(256) gemv_rows(GemvArgs a)
+__global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
 {
     using F = Fmt<MODE>;
     constexpr int VALS = F::VALS, WORDS = F::WORDS;
     static_assert(VALS == 32, "gemv_rows handles 32-code groups");
-    constexpr int RPW = kWave / LPR;  // rows per wave per step
-    constexpr int KWMAX = 4;
-    __shared__ float red[KWMAX][LPR * VALS];
+    static_assert(LPR <= 8 && 8 % LPR == 0, "one staging lane covers whole rows");
+    constexpr int RPW = kWave / LPR;   // rows per tile
+    constexpr int TILES = 8;           // tiles per chunk, all in flight
+    constexpr int CH = TILES * RPW;    // rows per chunk (= 512 / LPR)
+    constexpr int RPS = 8 / LPR;       // rows covered by one staging lane's 8 halves
 
+    extern __shared__ float lds[];
     const int lane = threadIdx.x;
     const int wy = threadIdx.y;
     const int KW = blockDim.y;
+    float *qw = lds + wy * (CH * LPR);                  // this wave's x*scale tile
+    float *red = lds + KW * (CH * LPR);                 // [KW][LPR*VALS] block reduction
     const int r = lane / LPR;
     const int j = lane % LPR;
     const int64_t sample = blockIdx.y;
@@ -222,44 +350,101 @@ __global__ void __launch_bounds__(256) gemv_rows(GemvArgs a)
     const int64_t kbeg = (int64_t)blockIdx.x * a.rows_per_split;
     const int64_t kend = kbeg + a.rows_per_split < a.K ? kbeg + a.rows_per_split : a.K;
 
-    const __half *xp = a.x + sample * a.x_bs + m * a.x_rs;
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
     const uint32_t *cp = a.code + kv * a.c_bs + j * WORDS;
-    const __half *sp = a.scale + kv * a.s_bs + j;
-    const __half *zp = a.zero + kv * a.s_bs + j;
+    const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
+    const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
 
     float acc[VALS];
 #pragma unroll
     for (int i = 0; i < VALS; i++) acc[i] = 0.f;
-    float zsum = 0.f;
+    float zacc[LPR];  // x*zero sums of the elements this lane staged, by group
+#pragma unroll
+    for (int i = 0; i < LPR; i++) zacc[i] = 0.f;
 
-#pragma unroll 4
-    for (int64_t kt = kbeg + wy * RPW; kt < kend; kt += KW * RPW) {
-        const int64_t k = kt + r;
-        if (k < kend) {
-            const Words<WORDS> w = *reinterpret_cast<const Words<WORDS> *>(cp + k * a.c_rs);
-            const float s = __half2float(sp[k * a.s_rs]);
-            const float z = __half2float(zp[k * a.s_rs]);
-            const float xv = __half2float(xp[k]);
-            zsum = fmaf(xv, z, zsum);
-            accumulate_unit<MODE>(w.v, xv * s, acc);
+    const int e0 = lane * 8;    // first element of the chunk's [CH][LPR] scale array this lane stages
+    const int row0 = e0 / LPR;  // its 8 elements are RPS whole rows
+
+    for (int64_t k0 = kbeg + (int64_t)wy * CH; k0 < kend; k0 += (int64_t)KW * CH) {
+        const int rows = (int)(kend - k0 < CH ? kend - k0 : CH);
+        // ---- small operands first (so waiting for them leaves the code loads in flight) ----
+        uint16_t sv[8], zv[8], xh[RPS];
+        if (row0 + RPS <= rows) {
+            const Half8 s8 = *reinterpret_cast<const Half8 *>(sp + k0 * LPR + e0);
+            const Half8 z8 = *reinterpret_cast<const Half8 *>(zp + k0 * LPR + e0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                sv[e] = s8.v[e];
+                zv[e] = z8.v[e];
+            }
+#pragma unroll
+            for (int q = 0; q < RPS; q++) xh[q] = xp[k0 + row0 + q];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const bool ok = (e0 + e) / LPR < rows;
+                sv[e] = ok ? sp[k0 * LPR + e0 + e] : (uint16_t)0;
+                zv[e] = ok ? zp[k0 * LPR + e0 + e] : (uint16_t)0;
+            }
+#pragma unroll
+            for (int q = 0; q < RPS; q++) xh[q] = row0 + q < rows ? xp[k0 + row0 + q] : (uint16_t)0;
         }
+        // ---- the chunk's packed codes: 8 tiles in flight ----
+        Words<WORDS> w[TILES];
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            int row = t * RPW + r;
+            row = row < rows ? row : rows - 1;  // clamped rows meet x*scale == 0
+            w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (k0 + row) * a.c_rs);
+        }
+        // ---- x*scale to LDS, x*zero into the private sums ----
+        {
+            float qv[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float xv = h16_to_f32(xh[e / LPR]);
+                qv[e] = xv * h16_to_f32(sv[e]);
+                zacc[e % LPR] = fmaf(xv, h16_to_f32(zv[e]), zacc[e % LPR]);
+            }
+            float4 *dst = reinterpret_cast<float4 *>(qw + e0);
+            dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
+            dst[1] = make_float4(qv[4], qv[5], qv[6], qv[7]);
+        }
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const float qs = qw[(t * RPW + r) * LPR + j];
+            accumulate_unit<MODE>(w[t].v, qs, acc);
+        }
+        wave_lds_fence();
     }
+
+    // zero term: zacc[g] summed over all lanes of the wave (every lane staged other rows)
+#pragma unroll
+    for (int g = 0; g < LPR; g++) {
+        float v = zacc[g];
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+        zacc[g] = v;
+    }
+    float zterm = 0.f;
+#pragma unroll
+    for (int g = 0; g < LPR; g++) zterm = (j == g) ? zacc[g] : zterm;
 #pragma unroll
     for (int i = 0; i < VALS; i++) {
-        float v = acc[i] + zsum;
+        float v = acc[i];
 #pragma unroll
         for (int off = LPR; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-        acc[i] = v;
+        acc[i] = v + zterm;
     }
     if (r == 0) {
 #pragma unroll
-        for (int i = 0; i < VALS; i++) red[wy][j * VALS + i] = acc[i];
+        for (int i = 0; i < VALS; i++) red[wy * (LPR * VALS) + j * VALS + i] = acc[i];
     }
     __syncthreads();
-    const int t = wy * kWave + lane;
-    if (t < LPR * VALS) {
+    for (int t = wy * kWave + lane; t < LPR * VALS; t += KW * kWave) {
         float v = 0.f;
-        for (int w = 0; w < KW; w++) v += red[w][t];
+        for (int w = 0; w < KW; w++) v += red[w * (LPR * VALS) + t];
         if (a.splits == 1)
             a.out[sample * a.o_bs + m * a.o_rs + t] = __float2half_rn(v);
         else
@@ -329,35 +514,51 @@ __global__ void __launch_bounds__(256) gemv_generic(GemvArgs a)
 
 // --------------------------- host side ---------------------------
 
-constexpr int kRowsKW = 4;          // waves per block in gemv_rows
-constexpr int kColsKW = 4;          // waves per block in gemv_cols
-constexpr int64_t kTargetBlocks = 1024;  // ~4 blocks of 4 waves on each of 256 CUs
-constexpr int64_t kColsMaxK = 4096;
+constexpr int64_t kTargetWaves = KVMIX_TARGET_WAVES;
 
 static bool rows_shape_ok(int64_t N) { return N == 64 || N == 128 || N == 256; }
 
-// split-K factor of gemv_rows for a problem (same function sizes the workspace)
-static int choose_splits(int64_t batch_rows, int64_t K, int64_t N)
+struct RowsPlan {
+    int waves;   // waves per block
+    int splits;  // blocks along K
+    int64_t rows_per_split;
+};
+
+// How gemv_rows covers K for `batch_rows` = samples*M independent outputs.
+static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N)
 {
-    if (!rows_shape_ok(N) || batch_rows <= 0) return 1;
-    const int64_t lpr = N / 32;
-    const int64_t tile = (int64_t)kRowsKW * (kWave / lpr);  // rows one block covers per step
-    int64_t want = (kTargetBlocks + batch_rows - 1) / batch_rows;
-    int64_t most = (K + 2 * tile - 1) / (2 * tile);  // at least two steps per block
-    if (most < 1) most = 1;
-    if (want > most) want = most;
-    if (want > 256) want = 256;
-    return (int)(want < 1 ? 1 : want);
+    RowsPlan p{4, 1, K > 0 ? K : 1};
+    if (!rows_shape_ok(N) || batch_rows <= 0 || K <= 0) return p;
+    const int64_t chunk = 512 / (N / 32);            // rows one wave takes per step
+    const int64_t chunks = (K + chunk - 1) / chunk;  // units of parallelism along K
+    int64_t want = (kTargetWaves + batch_rows - 1) / batch_rows;  // waves wanted per output row
+    if (want > chunks) want = chunks;
+    if (want < 1) want = 1;
+    int64_t waves = want < kRowsMaxWaves ? want : kRowsMaxWaves;
+    if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
+    int64_t splits = (want + waves - 1) / waves;
+    if (splits > 64) splits = 64;
+    int64_t rps = (K + splits - 1) / splits;
+    rps = (rps + chunk - 1) / chunk * chunk;
+    splits = (K + rps - 1) / rps;
+    p.waves = (int)waves;
+    p.splits = (int)(splits < 1 ? 1 : splits);
+    p.rows_per_split = rps;
+    return p;
 }
 
 template <int MODE>
-static void launch_rows(const GemvArgs &a, int64_t samples, hipStream_t st)
+static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
 {
-    const dim3 grid((unsigned)a.splits, (unsigned)samples, (unsigned)a.M), block(kWave, kRowsKW);
+    const RowsPlan p = plan_rows(samples * a.M, a.K, a.N);
+    a.splits = p.splits;
+    a.rows_per_split = p.rows_per_split;
+    const dim3 grid((unsigned)a.splits, (unsigned)samples, (unsigned)a.M), block(kWave, p.waves);
+    const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)(512 + a.N);
     switch (a.N / 32) {
-    case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((gemv_rows<MODE, 4>), grid, block, 0, st, a); break;
-    default: hipLaunchKernelGGL((gemv_rows<MODE, 8>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2>), grid, block, lds, st, a); break;
+    case 4: hipLaunchKernelGGL((gemv_rows<MODE, 4>), grid, block, lds, st, a); break;
+    default: hipLaunchKernelGGL((gemv_rows<MODE, 8>), grid, block, lds, st, a); break;
     }
     if (a.splits > 1) {
         const dim3 g2((unsigned)((a.N + 255) / 256), (unsigned)samples, (unsigned)a.M);
@@ -365,19 +566,48 @@ static void launch_rows(const GemvArgs &a, int64_t samples, hipStream_t st)
     }
 }
 
-template <int MODE>
-static void launch_cols(const GemvArgs &a, int64_t samples, hipStream_t st)
+template <int MODE, int RQ>
+static void launch_cols_rq(const GemvArgs &a, int64_t samples, hipStream_t st)
 {
     constexpr int VALS = Fmt<MODE>::VALS;
+    constexpr int GL = kWave / RQ;
     const int64_t groups = a.N / VALS;
-    const dim3 grid((unsigned)((groups + kWave - 1) / kWave), (unsigned)samples, (unsigned)a.M);
-    const int kw = a.K >= 4 * kColsKW ? kColsKW : 1;
-    const size_t lds = sizeof(float) * (size_t)(((a.K + 63) & ~(int64_t)63) + (kw > 1 ? kw * VALS * kWave : 0));
-    hipLaunchKernelGGL(gemv_cols<MODE>, grid, dim3(kWave, kw), lds, st, a);
+    const int64_t tiles = (groups + GL - 1) / GL;
+    const dim3 grid((unsigned)((tiles + kColsWaves - 1) / kColsWaves), (unsigned)samples, (unsigned)a.M);
+    hipLaunchKernelGGL((gemv_cols<MODE, RQ>), grid, dim3(kWave, kColsWaves), 0, st, a);
+}
+
+#ifndef KVMIX_COLS_RQ
+#define KVMIX_COLS_RQ 0  // 0 = choose by problem size
+#endif
+
+template <int MODE>
+static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    // more row sections per wave = more, narrower waves: take the widest tile that still
+    // gives the chip enough waves
+    constexpr int VALS = Fmt<MODE>::VALS;
+    const int64_t groups = a.N / VALS;
+    const int64_t batch = samples * a.M;
+    int rq = KVMIX_COLS_RQ;
+    if (rq == 0) {
+        if (batch * ((groups + 63) / 64) >= kTargetWaves)
+            rq = 1;
+        else if (batch * ((groups + 31) / 32) >= kTargetWaves)
+            rq = 2;
+        else
+            rq = 4;
+    }
+    if (rq == 4 && a.K >= 128)
+        launch_cols_rq<MODE, 4>(a, samples, st);
+    else if (rq >= 2 && a.K >= 64)
+        launch_cols_rq<MODE, 2>(a, samples, st);
+    else
+        launch_cols_rq<MODE, 1>(a, samples, st);
 }
 
 template <int MODE>
-static void launch_generic(const GemvArgs &a, int64_t samples, hipStream_t st)
+static void launch_generic(GemvArgs &a, int64_t samples, hipStream_t st)
 {
     constexpr int VALS = MODE == 30 ? 32 : (MODE == 3 ? 11 : 32 / MODE);
     const int64_t units = a.N / VALS;
@@ -392,8 +622,8 @@ using namespace kvmix;
 extern "C" size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t K, int64_t N)
 {
     if (samples <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
-    const int splits = choose_splits(samples * M, K, N);
-    return splits > 1 ? (size_t)(samples * M) * (size_t)splits * (size_t)N * sizeof(float) : 0;
+    const RowsPlan p = plan_rows(samples * M, K, N);
+    return p.splits > 1 ? (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float) : 0;
 }
 
 extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride,
@@ -426,7 +656,7 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     const int64_t words = N / unit_vals * unit_words, groups = N / group;
     if (code_row_stride < words || sz_row_stride < groups || x_row_stride < K || out_row_stride < N)
         return KVMIX_ERR_SHAPE;
-    if (samples > 65535 * 16 || M > 65535) return KVMIX_ERR_SHAPE;
+    if (samples > 65535 || M > 65535) return KVMIX_ERR_SHAPE;  // grid.y / grid.z limits
 
     GemvArgs a;
     a.x = (const __half *)x;
@@ -449,13 +679,13 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     a.heads_per_kv = heads_per_kv;
     a.group = group;
     a.splits = 1;
-    a.rows_per_split = K;
+    a.rows_per_split = K > 0 ? K : 1;
     hipStream_t st = (hipStream_t)stream;
-    if (samples > 65535) return KVMIX_ERR_SHAPE;  // grid.y limit
 
     const bool fast_group = ref3 ? true : group == 32;
-    const bool rows_ok = fast_group && !ref3 && rows_shape_ok(N);
-    const bool cols_ok = fast_group && K <= kColsMaxK;
+    // gemv_rows reads a chunk's scale/zero as one flat array: rows must be contiguous
+    const bool rows_ok = fast_group && !ref3 && rows_shape_ok(N) && sz_row_stride == N / 32 && K > 0;
+    const bool cols_ok = fast_group && K > 0;
     // p.V shape: few columns, many rows.  q.K^T shape: the opposite.
     const bool use_rows = rows_ok && (K >= 2 * N || !cols_ok);
 
@@ -469,17 +699,11 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     }
 
     if (use_rows) {
-        a.splits = choose_splits(samples * M, K, N);
-        if (a.splits > 1) {
-            const size_t need = (size_t)(samples * M) * (size_t)a.splits * (size_t)N * sizeof(float);
+        const RowsPlan p = plan_rows(samples * M, K, N);
+        if (p.splits > 1) {
+            const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
             if (!workspace || workspace_bytes < need) return KVMIX_ERR_WORKSPACE;
         }
-        const int64_t tile = (int64_t)kRowsKW * (kWave / (N / 32));
-        int64_t rps = (K + a.splits - 1) / a.splits;
-        rps = (rps + tile - 1) / tile * tile;
-        a.rows_per_split = rps;
-        a.splits = (int)((K + rps - 1) / rps);
-        if (a.splits < 1) a.splits = 1;
         switch (mode) {
         case 1: launch_rows<1>(a, samples, st); break;
         case 2: launch_rows<2>(a, samples, st); break;
