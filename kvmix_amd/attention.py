@@ -1,0 +1,175 @@
+"""Host-side mirror of the reference's attention glue around the KVmix operators.
+
+`KVmixAttention.forward` reproduces what `LlamaAttention_KVmix.forward`
+(models/modeling_llama_KVmix.py:105-283) and `MistralAttention_KVmix.forward`
+(models/modeling_mistral_KVmix.py:150-329) do between RoPE and the output projection:
+append to the fp16 tails, flush the oldest tail tokens through the quantizer, q.K^T over the
+packed keys + fp16 tail, fp32 softmax, p.V over the packed values + fp16 tail, and hand back the
+reference's 9-entry cache tuple
+
+    (Kcode [B,Hkv,D,Tqk/vpw] i32, K_tail [B,Hkv,Lk,D] f16, Kscale [B,Hkv,D,Tqk/g] f16, Kmin,
+     Vcode [B,Hkv,Tqv,D/vpw] i32, V_tail [B,Hkv,Lv,D] f16, Vscale [B,Hkv,Tqv,D/g] f16, Vmin, kv_seq_len)
+
+Projections, RoPE and the decoder stack belong to the model and are not part of this module.
+Differences from the reference, all of them copies it makes and this does not:
+GQA operands go to `quantized_gemm` un-repeated (the kernel maps query head h to kv head
+h // n_rep; the reference materialises n_rep copies, models/modeling_llama_KVmix.py:176-178),
+and the fp16 tail is multiplied through a grouped view instead of a repeated tensor.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+
+# Residual ratio the reference's profiler assigns to each bit width (myprofileKV.py:75-80).
+RESIDUAL_RATIO_BY_BITS = {4: 0.3, 3: 0.2, 2: 0.2, 1: 0.1}
+
+
+def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """models/modeling_llama_KVmix.py:19-28 (kept for callers that still want the copy)."""
+    batch, num_key_value_heads, slen, head_dim = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    hidden_states = hidden_states[:, :, None, :, :].expand(batch, num_key_value_heads, n_rep, slen, head_dim)
+    return hidden_states.reshape(batch, num_key_value_heads * n_rep, slen, head_dim)
+
+
+def flush_length(tail_len: int, ratio: float, group: int, residual_length: Optional[int] = None,
+                 prompt: bool = False) -> int:
+    """Number of oldest tail tokens to quantize now.
+
+    Ratio rule (models/modeling_llama_KVmix.py:119-127,152-155 and, for the prompt, :219-224):
+    keep int(ratio * L) tokens in fp16, quantize the rest rounded down to a multiple of the group.
+    Fixed window (residual_length = R): once the tail holds R tokens, flush floor(R/g)*g; for a
+    prompt, everything but the newest R tokens, rounded down to a multiple of the group."""
+    if residual_length is not None:
+        if prompt:
+            return (max(tail_len - residual_length, 0) // group) * group
+        return (residual_length // group) * group if tail_len >= residual_length else 0
+    keep = int(ratio * tail_len)
+    if tail_len > keep and keep >= 0:
+        return ((tail_len - keep) // group) * group
+    return 0
+
+
+def _cat(old: Optional[torch.Tensor], new: torch.Tensor, dim: int) -> torch.Tensor:
+    return new if old is None else torch.cat([old, new], dim=dim)
+
+
+def _grouped_matmul_qk(q: torch.Tensor, k_tail: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """q [B,nh,Q,D] x k_tail [B,Hkv,L,D]^T -> [B,nh,Q,L] without repeating k_tail."""
+    B, nh, Q, D = q.shape
+    Hkv, L = k_tail.shape[1], k_tail.shape[2]
+    if n_rep == 1:
+        return torch.matmul(q, k_tail.transpose(2, 3))
+    out = torch.matmul(q.reshape(B, Hkv, n_rep * Q, D), k_tail.transpose(2, 3))
+    return out.reshape(B, nh, Q, L)
+
+
+def _grouped_matmul_pv(p: torch.Tensor, v_tail: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """p [B,nh,Q,L] x v_tail [B,Hkv,L,D] -> [B,nh,Q,D] without repeating v_tail."""
+    B, nh, Q, L = p.shape
+    Hkv, D = v_tail.shape[1], v_tail.shape[3]
+    if n_rep == 1:
+        return torch.matmul(p, v_tail)
+    out = torch.matmul(p.reshape(B, Hkv, n_rep * Q, L), v_tail)
+    return out.reshape(B, nh, Q, D)
+
+
+class KVmixAttention:
+    """The KV-cache part of one attention layer (no weights)."""
+
+    def __init__(self, k_bits: int, v_bits: int, k_residual_ratio: Optional[float] = None,
+                 v_residual_ratio: Optional[float] = None, group_size: int = 32,
+                 residual_length: Optional[int] = None):
+        self.k_bits, self.v_bits = k_bits, v_bits
+        self.k_residual_ratio = RESIDUAL_RATIO_BY_BITS[k_bits] if k_residual_ratio is None else k_residual_ratio
+        self.v_residual_ratio = RESIDUAL_RATIO_BY_BITS[v_bits] if v_residual_ratio is None else v_residual_ratio
+        self.Vgroup_size = group_size
+        self.Kgroup_size = 11 if k_bits == 3 else group_size  # models/modeling_llama_KVmix.py:49-52
+        self.residual_length = residual_length
+
+    # -- flush helpers ---------------------------------------------------------------------
+    def _flush_keys(self, k_tail, code, scale, mn, prompt=False):
+        n = flush_length(k_tail.shape[-2], self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
+        if n > 0:
+            chunk = k_tail[:, :, :n, :]
+            k_tail = k_tail[:, :, n:, :]
+            c, s, m = ops.quantize_pack_last_dim_cuda(chunk.transpose(2, 3).contiguous(), self.Kgroup_size, self.k_bits)
+            code, scale, mn = _cat(code, c, 3), _cat(scale, s, 3), _cat(mn, m, 3)
+        return k_tail, code, scale, mn
+
+    def _flush_values(self, v_tail, code, scale, mn, prompt=False):
+        n = flush_length(v_tail.shape[-2], self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
+        if n > 0:
+            chunk = v_tail[:, :, :n, :]
+            v_tail = v_tail[:, :, n:, :]
+            c, s, m = ops.quantize_pack_last_dim_cuda(chunk.contiguous(), self.Vgroup_size, self.v_bits)
+            code, scale, mn = _cat(code, c, 2), _cat(scale, s, 2), _cat(mn, m, 2)
+        return v_tail, code, scale, mn
+
+    # -- the step --------------------------------------------------------------------------
+    def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
+                past_key_value: Optional[Tuple] = None, attention_mask: Optional[torch.Tensor] = None,
+                use_cache: bool = True):
+        """query_states [B,nh,Q,D], key/value_states [B,Hkv,Q,D] (fp16, after RoPE).
+        Returns (attn_output [B,nh,Q,D] fp16, attn_weights fp16, past_key_value or None)."""
+        B, nh, q_len, D = query_states.shape
+        n_rep = nh // key_states.shape[1]
+        kv_seq_len = key_states.shape[-2] + (past_key_value[-1] if past_key_value is not None else 0)
+
+        if past_key_value is not None:
+            kc, k_tail, ks, km, vc, v_tail, vs, vm, _ = past_key_value
+            k_tail = key_states if k_tail is None else torch.cat([k_tail, key_states], dim=2)
+            v_tail = value_states if v_tail is None else torch.cat([v_tail, value_states], dim=2)
+            k_tail, kc, ks, km = self._flush_keys(k_tail, kc, ks, km)
+            v_tail, vc, vs, vm = self._flush_values(v_tail, vc, vs, vm)
+
+            att_full = _grouped_matmul_qk(query_states, k_tail, n_rep)
+            if kc is not None:
+                att_quant = ops.quantized_gemm(self.Kgroup_size, query_states, kc, ks, km, self.k_bits)
+                attn_weights = torch.cat([att_quant.to(torch.float32), att_full.to(torch.float32)], dim=-1)
+            else:
+                attn_weights = att_full.to(torch.float32)
+            attn_weights = attn_weights / math.sqrt(D)
+            if attention_mask is not None:
+                if attention_mask.shape[-2:] != attn_weights.shape[-2:]:
+                    raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
+                                     f"{attn_weights.shape}")
+                attn_weights = attn_weights + attention_mask
+                attn_weights = torch.clamp(attn_weights, min=torch.finfo(attn_weights.dtype).min)
+            attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
+
+            if vc is None:
+                attn_output = _grouped_matmul_pv(attn_weights, v_tail, n_rep)
+            else:
+                lv = v_tail.shape[-2]
+                tq = attn_weights.shape[-1] - lv
+                out_quant = ops.quantized_gemm(self.Vgroup_size, attn_weights[..., :tq], vc, vs, vm, self.v_bits)
+                out_full = _grouped_matmul_pv(attn_weights[..., tq:], v_tail, n_rep)
+                attn_output = out_quant + out_full
+        else:
+            # prompt: dense fp16 attention; the cache keeps the oldest tokens quantized
+            # (models/modeling_llama_KVmix.py:213-266)
+            k_tail, kc, ks, km = self._flush_keys(key_states, None, None, None, prompt=True)
+            v_tail, vc, vs, vm = self._flush_values(value_states, None, None, None, prompt=True)
+            k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
+            attn_weights = _grouped_matmul_qk(query_states, key_states, n_rep) / math.sqrt(D)
+            if attention_mask is not None:
+                if attention_mask.shape[-2:] != attn_weights.shape[-2:]:
+                    raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
+                                     f"{attn_weights.shape}")
+                attn_weights = attn_weights + attention_mask
+                attn_weights = torch.clamp(attn_weights, min=torch.finfo(attn_weights.dtype).min)
+            attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
+            attn_output = _grouped_matmul_pv(attn_weights, value_states, n_rep)
+
+        cache = (kc, k_tail, ks, km, vc, v_tail, vs, vm, kv_seq_len) if use_cache else None
+        return attn_output, attn_weights, cache
+
+    __call__ = forward

@@ -97,6 +97,33 @@ def quantize_pack_last_dim_cuda(input: torch.Tensor, group_length: int, quant_bi
     return code, scale, mn
 
 
+def quantize_pack_dense3(input: torch.Tensor, group_length: int = 32):
+    """Extension (no reference counterpart): 3-bit codes with qmax 7 for every value, stored as a
+    little-endian bit stream (32 codes in three uint32), group a multiple of 32.  Same min / max /
+    scale / rounding arithmetic as quantize_pack_last_dim_cuda.  Pair with
+    quantized_gemm(..., bits=3, fmt=FMT_DENSE3).
+    Returns (code int32 [B,H,R,3S/32], scale [B,H,R,S/g], min [B,H,R,S/g])."""
+    if input.dtype not in _DT:
+        raise RuntimeError(f"expected scalar type Float or Half but found {input.dtype}")
+    if input.dim() != 4:
+        raise RuntimeError("input_tensor must be a 4D tensor")
+    B, H, R, S = input.shape
+    if group_length <= 0 or group_length % 32 != 0:
+        raise RuntimeError("dense 3-bit needs a group_length that is a multiple of 32")
+    if S % group_length != 0:
+        raise RuntimeError("steps must be divisible by group_length")
+    _need_gpu(input)
+    code = torch.empty((B, H, R, S * 3 // 32), dtype=torch.int32, device=input.device)
+    scale = torch.empty((B, H, R, S // group_length), dtype=input.dtype, device=input.device)
+    mn = torch.empty_like(scale)
+    _quantize_into(input, group_length, 3, _lib.FMT_DENSE3, _lib.SCALE_RECIPROCAL, code, scale, mn)
+    return code, scale, mn
+
+
+FMT_REF = _lib.FMT_REF
+FMT_DENSE3 = _lib.FMT_DENSE3
+
+
 def _batched3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:
     """[B, H, R, S] -> (tensor, batch stride, row stride) with (B, H) collapsible, unit last stride."""
     B, H, R, S = t.shape

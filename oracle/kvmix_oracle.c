@@ -272,6 +272,97 @@ int kvo_quantize_pack_last_dim_f16(const uint16_t *x, int64_t rows, int64_t step
 }
 
 /* ------------------------------------------------------------------------- */
+/* Dense 3-bit stream -- an EXTENSION with no counterpart in the reference     */
+/* (the reference's 3-bit is the 11-per-word format above).  Same min / max /  */
+/* scale / round / clamp arithmetic with qmax = 7 for every value; code i of a */
+/* row occupies stream bits [3i, 3i+3), little-endian across uint32 words, so  */
+/* 32 codes fill exactly three words.  group_length must be a multiple of 32.  */
+/* Pinned only by closed forms and round trips (tests/test_oracle_dense3.py):  */
+/* no reference parity is possible for this format.                            */
+/* ------------------------------------------------------------------------- */
+
+int kvo_quantize_pack_dense3(const float *x, int64_t rows, int64_t steps, int group_length,
+                             int scale_mode, int32_t *code, float *scale, float *mn)
+{
+    if (group_length <= 0 || group_length % 32 != 0) return KVO_ERR_DIVISIBLE;
+    if (steps % group_length != 0) return KVO_ERR_DIVISIBLE;
+    const int64_t words = steps * 3 / 32, groups = steps / group_length;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        uint32_t *cw = (uint32_t *)code + r * words;
+        for (int64_t w = 0; w < words; w++) cw[w] = 0;
+        for (int64_t gi = 0; gi < groups; gi++) {
+            const float *xg = x + r * steps + gi * group_length;
+            float lo, hi;
+            group_min_max(xg, group_length, &lo, &hi);
+            const float sc = (hi - lo) / 7.0f;
+            mn[r * groups + gi] = lo;
+            scale[r * groups + gi] = scale_mode == 0 ? (hi - lo) * (1.0f / 7.0f) : sc;
+            for (int i = 0; i < group_length; i++) {
+                const int64_t bit = (gi * group_length + i) * 3;
+                const uint64_t q = quantize_one(xg[i], lo, sc, 7);
+                const uint64_t spread = q << (bit % 32);
+                cw[bit / 32] |= (uint32_t)spread;
+                if ((bit % 32) > 29) cw[bit / 32 + 1] |= (uint32_t)(spread >> 32);
+            }
+        }
+    }
+    return KVO_OK;
+}
+
+static uint32_t extract_dense3(const uint32_t *row_words, int64_t n)
+{
+    const int64_t bit = 3 * n;
+    uint64_t two = row_words[bit / 32];
+    if ((bit % 32) > 29) two |= (uint64_t)row_words[bit / 32 + 1] << 32;
+    return (uint32_t)(two >> (bit % 32)) & 7u;
+}
+
+void kvo_unpack_dense3_row(const int32_t *code, int64_t n_values, int32_t *out)
+{
+    for (int64_t n = 0; n < n_values; n++) out[n] = (int32_t)extract_dense3((const uint32_t *)code, n);
+}
+
+/* dense-3 form of kvo_quantized_gemm (sequential fp32 accumulation; float64 side outputs) */
+int kvo_quantized_gemm_dense3(int group_size, const uint16_t *fA, int64_t a_batch_stride, int64_t lda,
+                              const int32_t *qB, const uint16_t *scales, const uint16_t *zeros,
+                              int64_t BH, int heads_per_kv, int64_t M, int64_t K, int64_t N,
+                              uint16_t *out, double *out64, double *abs64)
+{
+    if (heads_per_kv <= 0 || BH % heads_per_kv != 0) return KVO_ERR_HEADS;
+    if (group_size <= 0 || group_size % 32 != 0 || N % group_size != 0) return KVO_ERR_DIVISIBLE;
+    const int64_t words = N * 3 / 32, groups = N / group_size;
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t s = 0; s < BH; s++) {
+        for (int64_t m = 0; m < M; m++) {
+            const int64_t kv = s / heads_per_kv;
+            const uint16_t *x = fA + s * a_batch_stride + m * lda;
+            for (int64_t n = 0; n < N; n++) {
+                float acc = 0.f;
+                double acc64 = 0.0, a64 = 0.0;
+                for (int64_t k = 0; k < K; k++) {
+                    const uint32_t *row = (const uint32_t *)qB + (kv * K + k) * words;
+                    const float c = (float)extract_dense3(row, n);
+                    const float sc = kvo_half_to_float(scales[(kv * K + k) * groups + n / group_size]);
+                    const float zr = kvo_half_to_float(zeros[(kv * K + k) * groups + n / group_size]);
+                    const float xv = kvo_half_to_float(x[k]);
+                    const float wv = sc * c + zr;
+                    acc += wv * xv;
+                    const double wd = (double)sc * (double)c + (double)zr;
+                    acc64 += wd * (double)xv;
+                    a64 += fabs(wd) * fabs((double)xv);
+                }
+                const int64_t o = (s * M + m) * N + n;
+                if (out) out[o] = kvo_float_to_half(acc);
+                if (out64) out64[o] = acc64;
+                if (abs64) abs64[o] = a64;
+            }
+        }
+    }
+    return KVO_OK;
+}
+
+/* ------------------------------------------------------------------------- */
 /* process_key_quantization_cuda          quantization_cuda.cu:298-411        */
 /*   x_new [rows, new_steps] (rows = B*H*D), groups along the steps           */
 /*   out_* [rows, old + new]; the old part is a copy of prev_*                */

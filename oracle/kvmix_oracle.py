@@ -73,6 +73,10 @@ def lib() -> ctypes.CDLL:
         L.kvo_float_to_half.restype = ctypes.c_uint16
         L.kvo_float_to_half.argtypes = [ctypes.c_float]
         L.kvo_set_num_threads.argtypes = [i32]
+        L.kvo_quantize_pack_dense3.argtypes = [vp, i64, i64, i32, i32, vp, vp, vp]
+        L.kvo_unpack_dense3_row.argtypes = [vp, i64, vp]
+        L.kvo_quantized_gemm_dense3.argtypes = [i32, vp, i64, i64, vp, vp, vp, i64, i32, i64, i64, i64,
+                                                vp, vp, vp]
         _lib = L
     return _lib
 
@@ -231,6 +235,68 @@ def quantize_pack_last_dim_np(x: np.ndarray, group_length: int, quant_bits: int,
         with np.errstate(over="ignore"):
             scale_out, mn = scale_out.astype(np.float16), mn.astype(np.float16)
     return code, scale_out, mn
+
+
+# ---------------------------------------------------------------------------
+# dense 3-bit stream (extension; no reference counterpart)
+# ---------------------------------------------------------------------------
+
+def quantize_pack_dense3(x: np.ndarray, group_length: int = 32, scale_mode: int = SCALE_RECIPROCAL):
+    """3-bit codes (qmax 7 everywhere) as a little-endian bit stream: 32 codes in 3 words."""
+    if x.ndim != 4:
+        raise RuntimeError("input_tensor must be a 4D tensor")
+    is_half = x.dtype == np.float16
+    xf = np.ascontiguousarray(x, dtype=np.float32)
+    B, H, R, S = xf.shape
+    g = max(group_length, 1)
+    code = np.zeros((B, H, R, S * 3 // 32), np.int32)
+    scale = np.zeros((B, H, R, S // g), np.float32)
+    mn = np.zeros_like(scale)
+    _check(lib().kvo_quantize_pack_dense3(_p(xf), B * H * R, S, group_length, scale_mode, _p(code),
+                                          _p(scale), _p(mn)))
+    if is_half:
+        scale, mn = scale.astype(np.float16), mn.astype(np.float16)
+    return code, scale, mn
+
+
+def pack_dense3_np(q: np.ndarray) -> np.ndarray:
+    """codes [..., S] (0..7) -> words [..., 3S/32]: code i at stream bits [3i, 3i+3)."""
+    q = np.asarray(q).astype(np.uint8)
+    bits = ((q[..., None] >> np.arange(3, dtype=np.uint8)) & 1).reshape(q.shape[:-1] + (q.shape[-1] * 3,))
+    by = np.packbits(bits, axis=-1, bitorder="little")
+    return np.ascontiguousarray(by).view(np.uint32).view(np.int32)
+
+
+def unpack_dense3_np(code: np.ndarray) -> np.ndarray:
+    by = np.ascontiguousarray(code).view(np.uint8)
+    bits = np.unpackbits(by, axis=-1, bitorder="little")
+    bits = bits.reshape(bits.shape[:-1] + (bits.shape[-1] // 3, 3)).astype(np.int32)
+    return bits[..., 0] | (bits[..., 1] << 1) | (bits[..., 2] << 2)
+
+
+def dequantize_dense3_np(code, scales, zeros, group_size=32) -> np.ndarray:
+    q = unpack_dense3_np(code).astype(np.float32)
+    s = np.repeat(scales.astype(np.float32), group_size, axis=-1)
+    z = np.repeat(zeros.astype(np.float32), group_size, axis=-1)
+    return (s * q).astype(np.float32) + z
+
+
+def quantized_gemm_dense3(group_size, fA, qB, scales, zeros, want_f64=False):
+    B, nh, M, K = fA.shape
+    nh_kv = qB.shape[1]
+    if nh % nh_kv:
+        raise RuntimeError(_ERRORS[-4])
+    N = zeros.shape[-1] * group_size
+    a = np.ascontiguousarray(fA, np.float16)
+    q = np.ascontiguousarray(qB, np.int32)
+    s = np.ascontiguousarray(scales, np.float16)
+    z = np.ascontiguousarray(zeros, np.float16)
+    out = np.zeros((B, nh, M, N), np.float16)
+    o64 = np.zeros((B, nh, M, N), np.float64) if want_f64 else None
+    a64 = np.zeros((B, nh, M, N), np.float64) if want_f64 else None
+    _check(lib().kvo_quantized_gemm_dense3(group_size, _p(a), M * K, K, _p(q), _p(s), _p(z), B * nh,
+                                           nh // nh_kv, M, K, N, _p(out), _p(o64), _p(a64)))
+    return (out, o64, a64) if want_f64 else out
 
 
 # ---------------------------------------------------------------------------

@@ -1,0 +1,97 @@
+"""The attention glue (kvmix_amd.attention.KVmixAttention) on the GPU against the oracle's
+restatement of models/modeling_llama_KVmix.py:105-283: same flush decisions, bit-exact cache
+contents, outputs within tolerance, for MHA and GQA, ratio and fixed-window policies."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import kv_like, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def to_t(a, dev):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def cache_np(c):
+    return tuple(x.cpu().numpy() if torch.is_tensor(x) else x for x in c)
+
+
+def same_cache(got, want):
+    for i, (g, w) in enumerate(zip(cache_np(got), want)):
+        if w is None or isinstance(w, int):
+            assert g == w or (g is None and w is None), i
+        else:
+            assert same_bits(g, w), i
+
+
+@pytest.mark.parametrize("k_bits,v_bits,nkv,window", [(4, 4, 4, None), (3, 2, 2, None), (2, 4, 1, None),
+                                                      (1, 1, 4, None), (4, 2, 2, 64), (3, 4, 4, 48)])
+def test_decode_steps_follow_the_oracle(oracle, dev, k_bits, v_bits, nkv, window):
+    from kvmix_amd.attention import RESIDUAL_RATIO_BY_BITS, KVmixAttention
+
+    rng = np.random.default_rng(k_bits * 10 + v_bits)
+    B, nh, D, g = 2, 4, 128, 32
+    att = KVmixAttention(k_bits, v_bits, group_size=g, residual_length=window)
+    cache_o = (None,) * 8 + (0,)
+    cache_g = (None,) * 8 + (0,)
+    kr, vr = RESIDUAL_RATIO_BY_BITS[k_bits], RESIDUAL_RATIO_BY_BITS[v_bits]
+    for step in range(100):
+        k = kv_like(rng, (B, nkv, 1, D))
+        v = kv_like(rng, (B, nkv, 1, D))
+        q = rng.standard_normal((B, nh, 1, D)).astype(np.float16)
+        out_o, p_o, cache_o = oracle.attention_decode_step(q, k, v, cache_o, k_bits, v_bits, kr, vr, group_size=g,
+                                                           fixed_window=window)
+        out_g, p_g, cache_g = att(to_t(q, dev), to_t(k, dev), to_t(v, dev), cache_g)
+        same_cache(cache_g, cache_o)
+        np.testing.assert_allclose(p_g.cpu().numpy().astype(np.float64), p_o.astype(np.float64), rtol=5e-3, atol=2e-5)
+        np.testing.assert_allclose(out_g.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
+    assert cache_o[0] is not None and cache_o[4] is not None
+
+
+def test_prompt_then_decode(oracle, dev):
+    """Prompt branch: dense attention output, cache = oldest tokens quantized by the ratio rule
+    (models/modeling_llama_KVmix.py:213-273); the first decode step then flushes several groups."""
+    from kvmix_amd.attention import KVmixAttention, flush_length
+
+    rng = np.random.default_rng(3)
+    B, nh, nkv, D, T, g = 1, 8, 2, 128, 300, 32
+    att = KVmixAttention(3, 2, group_size=g)
+    K = kv_like(rng, (B, nkv, T, D), outlier_axis=3)
+    V = kv_like(rng, (B, nkv, T, D), outlier_axis=3)
+    Q = rng.standard_normal((B, nh, T, D)).astype(np.float16)
+    mask = np.triu(np.full((T, T), np.finfo(np.float32).min, np.float32), 1)[None, None]
+    out, p, cache = att(to_t(Q, dev), to_t(K, dev), to_t(V, dev), None, attention_mask=to_t(mask, dev))
+    nqk = flush_length(T, 0.2, 11)
+    nqv = flush_length(T, 0.2, 32)
+    assert nqk == 231 and nqv == 224 and cache[-1] == T
+    kc, ks, km = oracle.quantize_pack_last_dim(np.ascontiguousarray(K[:, :, :nqk].transpose(0, 1, 3, 2)), 11, 3)
+    vc, vs, vm = oracle.quantize_pack_last_dim(np.ascontiguousarray(V[:, :, :nqv]), 32, 2)
+    same_cache(cache, (kc, K[:, :, nqk:], ks, km, vc, V[:, :, nqv:], vs, vm, T))
+    # dense causal attention in float64
+    rep = nh // nkv
+    w = np.einsum("bhqd,bhtd->bhqt", Q.astype(np.float64), np.repeat(K.astype(np.float64), rep, 1)) / np.sqrt(D) + mask
+    w = np.exp(w - w.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    want = np.einsum("bhqt,bhtd->bhqd", w, np.repeat(V.astype(np.float64), rep, 1))
+    np.testing.assert_allclose(out.cpu().numpy().astype(np.float64), want, rtol=1e-2, atol=5e-2)  # fp16 probabilities, |V| up to ~40 in the outlier channels
+    # decode continues from the prompt cache on both sides
+    cache_o = cache_np(cache)
+    for step in range(3):
+        k = kv_like(rng, (B, nkv, 1, D))
+        v = kv_like(rng, (B, nkv, 1, D))
+        q = rng.standard_normal((B, nh, 1, D)).astype(np.float16)
+        out_o, p_o, cache_o = oracle.attention_decode_step(q, k, v, cache_o, 3, 2, 0.2, 0.2, group_size=g)
+        out_g, p_g, cache = att(to_t(q, dev), to_t(k, dev), to_t(v, dev), cache)
+        same_cache(cache, cache_o)
+        np.testing.assert_allclose(out_g.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
+
+
+def test_mask_shape_error(dev):
+    from kvmix_amd.attention import KVmixAttention
+
+    att = KVmixAttention(4, 4)
+    q = torch.zeros(1, 2, 1, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError, match="does not match"):
+        att(q, q, q, (None,) * 8 + (0,), attention_mask=torch.zeros(1, 1, 1, 7, device=dev))
