@@ -1,0 +1,424 @@
+#!/usr/bin/env python3
+"""Benchmark of the KVmix KV-cache hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): full 32-layer Llama-2-7B KV shape (32 heads x 128, MHA),
+batch 8, 8192 tokens of context, mixed per-layer bits from a seeded vector (8 layers 4-bit,
+16 layers 3-bit, 8 layers 2-bit; keys and values drawn independently), group 32, 128-token fp16
+residual window.  One "step" = for every layer: quantize-and-pack one flush of the residual window
+(keys and values) + the fused dequant-GEMV pair q.K^T and p.V over the packed cache.
+
+3-bit keys use the reference's 11-codes-per-word layout (group 11, 8063 quantized tokens, the flush
+is 121 tokens); 3-bit values have no working reference form and use the dense 3-bit extension.
+
+Prints one JSON line.  `value` = algorithmic HBM bytes of a step / step time, inputs resident in
+HBM.  `roofline` describes the kernel that takes the most time in the step, timed with events on
+the launch stream.  `cpu_baseline` times the CPU oracle on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def layer_bits(num_layers: int = 32, seed: int = 1):
+    rng = np.random.default_rng(seed)
+    base = np.array([4] * (num_layers // 4) + [3] * (num_layers // 2) + [2] * (num_layers // 4))
+    kb = rng.permutation(base)
+    vb = rng.permutation(base)
+    return [int(b) for b in kb], [int(b) for b in vb]
+
+
+def bytes_per_token(bits: int, fmt: str, D: int = 128) -> float:
+    """Stored bytes per (batch, kv-head) per quantized token: codes + fp16 scale + fp16 zero."""
+    if fmt == "ref3":
+        return D * 4 / 11 * 2          # one word and one (scale, zero) pair per 11 tokens, per channel
+    if fmt == "dense3":
+        return D * 3 / 8 + 4 * (D // 32)
+    return D * bits / 8 + 4 * (D // 32)
+
+
+class Layer:
+    pass
+
+
+def synth_kv(torch, B, H, T, D, dev, gen):
+    x = torch.randn(B, H, T, D, device=dev, dtype=torch.float16, generator=gen)
+    ch = torch.stack([torch.randperm(D, device=dev, generator=gen)[:4] for _ in range(H)])  # [H,4]
+    idx = ch[None, :, None, :].expand(B, H, T, 4)
+    x.scatter_(3, idx, x.gather(3, idx) * 10)
+    return x
+
+
+def build_layers(torch, ops, lib, B, H, D, T, R, kbits, vbits, dev):
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    layers = []
+    for kb, vb in zip(kbits, vbits):
+        L = Layer()
+        L.kb, L.vb = kb, vb
+        L.kfmt = "ref3" if kb == 3 else f"b{kb}"
+        L.vfmt = "dense3" if vb == 3 else f"b{vb}"
+        L.kg = 11 if kb == 3 else 32
+        L.Tqk = ((T - R) // L.kg) * L.kg  # ref3: 8063 = 11 * 733 for T=8192, R=128 (tail 129)
+        L.Tqv = ((T - R) // 32) * 32
+        L.nk = (R // L.kg) * L.kg         # tokens per key flush (128, or 121 for ref3)
+        L.nv = (R // 32) * 32
+        K = synth_kv(torch, B, H, T, D, dev, gen)
+        kin = K[:, :, :L.Tqk].transpose(2, 3).contiguous()
+        L.kc, L.ks, L.kz = ops.quantize_pack_last_dim_cuda(kin, L.kg, kb)
+        L.ktail = K[:, :, L.Tqk:L.Tqk + L.nk].contiguous()  # token-major chunk to flush
+        del K, kin
+        V = synth_kv(torch, B, H, T, D, dev, gen)
+        vin = V[:, :, :L.Tqv].contiguous()
+        if vb == 3:
+            L.vc, L.vs, L.vz = ops.quantize_pack_dense3(vin, 32)
+        else:
+            L.vc, L.vs, L.vz = ops.quantize_pack_last_dim_cuda(vin, 32, vb)
+        L.vtail = V[:, :, L.Tqv:L.Tqv + L.nv].contiguous()
+        del V, vin
+        L.q = torch.randn(B, H, 1, D, device=dev, dtype=torch.float16, generator=gen)
+        L.p = torch.softmax(torch.randn(B, H, 1, L.Tqv, device=dev, generator=gen), -1).half()
+        # outputs (fixed buffers: the state of the cache does not change between steps)
+        L.logits = torch.empty(B, H, 1, L.Tqk, device=dev, dtype=torch.float16)
+        L.out = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+        kw = L.nk // 11 if kb == 3 else L.nk * kb // 32
+        L.fk_code = torch.empty(B, H, D, kw, device=dev, dtype=torch.int32)
+        L.fk_s = torch.empty(B, H, D, L.nk // L.kg, device=dev, dtype=torch.float16)
+        L.fk_z = torch.empty_like(L.fk_s)
+        vw = D * 3 // 32 if vb == 3 else D * vb // 32
+        L.fv_code = torch.empty(B, H, L.nv, vw, device=dev, dtype=torch.int32)
+        L.fv_s = torch.empty(B, H, L.nv, D // 32, device=dev, dtype=torch.float16)
+        L.fv_z = torch.empty_like(L.fv_s)
+        wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, L.Tqv, D)
+        L.ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+        L.wsb = wsb
+        # algorithmic bytes
+        L.bytes_qk = B * H * L.Tqk * bytes_per_token(kb, "ref3" if kb == 3 else "")
+        L.bytes_pv = B * H * L.Tqv * bytes_per_token(vb, "dense3" if vb == 3 else "")
+        L.bytes_fk = B * H * L.nk * (2 * D + bytes_per_token(kb, "ref3" if kb == 3 else ""))
+        L.bytes_fv = B * H * L.nv * (2 * D + bytes_per_token(vb, "dense3" if vb == 3 else ""))
+        layers.append(L)
+    return layers
+
+
+def make_calls(torch, _lib, lib, layers, B, H, D, stream):
+    """Pre-bound C-ABI calls, one list entry per kernel launch group: (tag, bytes, fn)."""
+    calls = []
+    for L in layers:
+        kfmt = _lib.FMT_REF
+        vfmt = _lib.FMT_DENSE3 if L.vb == 3 else _lib.FMT_REF
+
+        def fk(L=L):
+            return lib.kvmix_quant_pack_key_tokens(
+                L.ktail.data_ptr(), B * H, L.nk, D, L.ktail.stride(1), L.ktail.stride(2), L.kg, L.kb, kfmt,
+                _lib.SCALE_RECIPROCAL, L.fk_code.data_ptr(), L.fk_code.stride(1), L.fk_code.stride(2),
+                L.fk_s.data_ptr(), L.fk_z.data_ptr(), L.fk_s.stride(1), L.fk_s.stride(2), stream)
+
+        def fv(L=L, vfmt=vfmt):
+            return lib.kvmix_quant_pack_last_dim(
+                L.vtail.data_ptr(), _lib.F16, B * H, L.nv, D, L.vtail.stride(1), L.vtail.stride(2), 32, L.vb, vfmt,
+                _lib.SCALE_RECIPROCAL, L.fv_code.data_ptr(), L.fv_code.stride(1), L.fv_code.stride(2),
+                L.fv_s.data_ptr(), L.fv_z.data_ptr(), L.fv_s.stride(1), L.fv_s.stride(2), stream)
+
+        def qk(L=L):
+            return lib.kvmix_quantized_gemv(
+                L.kg, L.q.data_ptr(), D, D, L.kc.data_ptr(), L.kc.stride(1), L.kc.stride(2), L.ks.data_ptr(),
+                L.kz.data_ptr(), L.ks.stride(1), L.ks.stride(2), L.kb, kfmt, B * H, 1, 1, D, L.Tqk,
+                L.logits.data_ptr(), L.Tqk, L.Tqk, None, 0, stream)
+
+        def pv(L=L, vfmt=vfmt):
+            return lib.kvmix_quantized_gemv(
+                32, L.p.data_ptr(), L.Tqv, L.Tqv, L.vc.data_ptr(), L.vc.stride(1), L.vc.stride(2), L.vs.data_ptr(),
+                L.vz.data_ptr(), L.vs.stride(1), L.vs.stride(2), L.vb, vfmt, B * H, 1, 1, L.Tqv, D,
+                L.out.data_ptr(), D, D, L.ws.data_ptr(), L.wsb, stream)
+
+        calls += [(f"quant_key_tokens[{L.kfmt}]", L.bytes_fk, fk), (f"quant_rows[{L.vfmt}]", L.bytes_fv, fv),
+                  (f"gemv_cols[{L.kfmt}]", L.bytes_qk, qk), (f"gemv_rows[{L.vfmt}]", L.bytes_pv, pv)]
+    return calls
+
+
+def run_step(calls):
+    for _, _, fn in calls:
+        rc = fn()
+        if rc != 0:
+            raise RuntimeError(f"kvmix call failed: {rc}")
+
+
+def time_kernels(torch, calls, reps=3):
+    """Per kernel kind: average duration of one launch (events on the launch stream), over the
+    step's own launches (each on its own layer's buffers, so nothing is served from cache)."""
+    kinds = {}
+    for tag, nbytes, fn in calls:
+        kinds.setdefault(tag, []).append((nbytes, fn))
+    out = {}
+    for tag, lst in kinds.items():
+        for _, fn in lst:
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            for _, fn in lst:
+                fn()
+        e.record()
+        torch.cuda.synchronize()
+        n = reps * len(lst)
+        out[tag] = {"launches_per_step": len(lst), "avg_us": s.elapsed_time(e) * 1e3 / n,
+                    "bytes_per_launch": float(np.mean([b for b, _ in lst]))}
+    return out
+
+
+def cpu_baseline(layers, kbits, vbits, B, H, D, T, R, sample_layers=None, budget_s=20.0):
+    """The CPU oracle (scalar C restatement of the reference kernels, OpenMP over rows) on the
+    step's own data, layer by layer at full batch (one flush + the GEMV pair each), until about
+    `budget_s` seconds of CPU time are spent or the layers run out."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import kvmix_oracle as O
+
+    O.lib()
+    rng = np.random.default_rng(0)
+    total_bytes, total_t = 0.0, 0.0
+    done = 0
+    for li in range(len(layers) if sample_layers is None else sample_layers):
+        if total_t > budget_s:
+            break
+        done += 1
+        L = layers[li]
+        kc = L.kc.cpu().numpy()
+        ks, kz = L.ks.cpu().numpy(), L.kz.cpu().numpy()
+        vc = L.vc.cpu().numpy()
+        vs, vz = L.vs.cpu().numpy(), L.vz.cpu().numpy()
+        q = L.q.cpu().numpy()
+        p = L.p.cpu().numpy()
+        ktail = np.ascontiguousarray(L.ktail.cpu().numpy().transpose(0, 1, 3, 2))
+        vtail = L.vtail.cpu().numpy()
+        t0 = time.perf_counter()
+        O.quantize_pack_last_dim(ktail, L.kg, L.kb)
+        if L.vb == 3:
+            O.quantize_pack_dense3(vtail, 32)
+        else:
+            O.quantize_pack_last_dim(vtail, 32, L.vb)
+        O.quantized_gemm(L.kg, q, kc, ks, kz, L.kb, mode=O.GEMM_SEQUENTIAL)
+        if L.vb == 3:
+            O.quantized_gemm_dense3(32, p, vc, vs, vz)
+        else:
+            O.quantized_gemm(32, p, vc, vs, vz, L.vb, mode=O.GEMM_SEQUENTIAL)
+        total_t += time.perf_counter() - t0
+        total_bytes += L.bytes_qk + L.bytes_pv + L.bytes_fk + L.bytes_fv
+    return {"value": round(total_bytes / total_t / 1e9, 3), "unit": "GB/s", "cores": int(O.num_threads()),
+            "kind": "port",
+            "sample": f"layers 0..{done - 1} of the step at full batch (one flush + q.K^T + p.V each, "
+                      f"{total_bytes / 1e9:.2f} GB algorithmic), {total_t:.1f} s of CPU time, "
+                      f"C oracle with OpenMP on {int(O.num_threads())} threads"}
+
+
+def target_shape_extra(torch, _lib, lib, dev, stream):
+    """The shape the target is quoted on: B=16, 32 heads, T=8192 (8064 quantized), 4- and 2-bit."""
+    B, H, D, Tq = 16, 32, 128, 8064
+    res = {}
+    for bits in (4, 2):
+        sets = []
+        for _ in range(3):  # three buffer sets (~1 GB at 4 bits) so the Infinity Cache cannot serve them
+            kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+            ks = torch.rand(B, H, D, Tq // 32, device=dev).half()
+            kz = torch.randn(B, H, D, Tq // 32, device=dev).half()
+            vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+            vs = torch.rand(B, H, Tq, D // 32, device=dev).half()
+            vz = torch.randn(B, H, Tq, D // 32, device=dev).half()
+            sets.append((kc, ks, kz, vc, vs, vz))
+        q = torch.randn(B, H, 1, D, device=dev).half()
+        p = torch.softmax(torch.randn(B, H, 1, Tq, device=dev), -1).half()
+        lo = torch.empty(B, H, 1, Tq, device=dev, dtype=torch.float16)
+        o = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+        wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, Tq, D)
+        ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+
+        def qk(i):
+            kc, ks, kz = sets[i % 3][:3]
+            return lib.kvmix_quantized_gemv(32, q.data_ptr(), D, D, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(),
+                                            kz.data_ptr(), ks.stride(1), ks.stride(2), bits, 0, B * H, 1, 1, D, Tq,
+                                            lo.data_ptr(), Tq, Tq, None, 0, stream)
+
+        def pv(i):
+            vc, vs, vz = sets[i % 3][3:]
+            return lib.kvmix_quantized_gemv(32, p.data_ptr(), Tq, Tq, vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(),
+                                            vz.data_ptr(), vs.stride(1), vs.stride(2), bits, 0, B * H, 1, 1, Tq, D,
+                                            o.data_ptr(), D, D, ws.data_ptr(), wsb, stream)
+
+        nbytes = B * H * Tq * bytes_per_token(bits, "")
+        for name, fn in (("qk", qk), ("pv", pv)):
+            for i in range(6):
+                assert fn(i) == 0
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for i in range(30):
+                fn(i)
+            e.record()
+            torch.cuda.synchronize()
+            us = s.elapsed_time(e) * 1e3 / 30
+            res[f"{name}_{bits}bit"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                        "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        del sets
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-target-shape", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain 1 GiB device copies (a known-size kernel to scale HBM counters by)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every (batch, kv-head) slice is independent; "
+              "see DESIGN.md for how the path would shard). Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from kvmix_amd import _lib, ops
+
+    lib = _lib.load()  # fails loudly if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, D, T, R = args.batch, 32, 128, args.context, 128
+    kbits, vbits = layer_bits(args.layers)
+    layers = build_layers(torch, ops, lib, B, H, D, T, R, kbits, vbits, dev)
+    torch.cuda.synchronize()
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    side = torch.cuda.Stream()
+    mode = "eager"
+    graph = None
+    with torch.cuda.stream(side):
+        calls = make_calls(torch, _lib, lib, layers, B, H, D, side.cuda_stream)
+        run_step(calls)
+        side.synchronize()
+        per_kernel = time_kernels(torch, calls)
+        if not args.no_graph:
+            try:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    run_step(calls)
+                mode = "hipgraph"
+            except Exception as ex:  # capture unsupported: stay eager
+                graph = None
+                mode = f"eager (graph capture failed: {type(ex).__name__})"
+
+        def step():
+            if graph is not None:
+                graph.replay()
+            else:
+                run_step(calls)
+
+        for _ in range(args.warmup):
+            step()
+        side.synchronize()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        s.record(side)
+        for _ in range(args.steps):
+            step()
+        e.record(side)
+        side.synchronize()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ev_ms = s.elapsed_time(e)
+
+    ms_per_step = wall * 1e3 / args.steps
+    step_bytes = sum(b for _, b, _ in calls)
+    gemv_bytes = sum(b for t, b, _ in calls if t.startswith("gemv"))
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel of the step
+    dom = max(per_kernel.items(), key=lambda kv: kv[1]["launches_per_step"] * kv[1]["avg_us"])
+    dname, d = dom
+    achieved = d["bytes_per_launch"] / d["avg_us"] / 1e3
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(dname)
+        except Exception:
+            traffic = None
+    gemv_us = sum(v["launches_per_step"] * v["avg_us"] for k, v in per_kernel.items() if k.startswith("gemv"))
+    quant_us = sum(v["launches_per_step"] * v["avg_us"] for k, v in per_kernel.items() if k.startswith("quant"))
+    quant_bytes = step_bytes - gemv_bytes
+
+    result = {
+        "metric": "fused dequant-GEMV HBM GB/s (% peak) + decode tok/s, Llama-2-7B mixed-bit KV",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32 codes / fp16 scale,zero / fp32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: 32-layer Llama-2-7B KV shape, mixed per-layer bits, one flush + q.K^T + p.V per layer",
+            "batch": B, "context": T, "heads": H, "head_dim": D, "group": 32, "residual": R, "layers": args.layers,
+            "k_bits": kbits, "v_bits": vbits, "k3_format": "reference 11-per-word (group 11)",
+            "v3_format": "dense 3-bit stream (extension)", "launch": mode,
+        },
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "decode_tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
+        "step_bytes": int(step_bytes),
+        "event_ms_per_step": round(ev_ms / args.steps, 4),
+        "gemv_only": {"bytes": int(gemv_bytes), "us": round(gemv_us, 1), "GBps": round(gemv_bytes / gemv_us / 1e3, 1),
+                      "frac_of_peak": round(gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS, 4)},
+        "quantizer_only": {"bytes": int(quant_bytes), "us": round(quant_us, 1),
+                           "GBps": round(quant_bytes / quant_us / 1e3, 1)},
+        "kernels": {k: {"launches_per_step": v["launches_per_step"], "avg_us": round(v["avg_us"], 2),
+                        "GBps": round(v["bytes_per_launch"] / v["avg_us"] / 1e3, 1)} for k, v in per_kernel.items()},
+        "roofline": {"kernel": dname, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "bytes_per_launch": int(d["bytes_per_launch"]), "avg_launch_us": round(d["avg_us"], 2)},
+    }
+    print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H, D, T, R)
+
+
+def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H, D, T, R):
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(layers, kbits, vbits, B, H, D, T, R)
+    if not args.no_target_shape:
+        # free the 32-layer cache first: the target-shape buffers need ~3 GB of their own
+        for L in layers:
+            L.__dict__.clear()
+        torch.cuda.empty_cache()
+        result["target_shape_B16_T8192"] = target_shape_extra(torch, _lib, lib, dev,
+                                                              torch.cuda.current_stream().cuda_stream)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -157,6 +157,23 @@ __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, flo
     }
 }
 
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin in launch order, so
+// neighbours in launch order never share an L2.  This maps the launch-order index to a
+// logical index such that CONSECUTIVE logical indices run on the SAME XCD: column tiles of
+// one cache row (they share the 128-byte lines that straddle tile borders) and query heads
+// of one kv head (they read the same packed data) then meet in one L2.
+constexpr int kXcds = 8;
+__device__ __forceinline__ void xcd_swizzled_block(int64_t &bx, int64_t &by)
+{
+    const int64_t nx = gridDim.x, n = nx * (int64_t)gridDim.y;
+    const int64_t l = (int64_t)blockIdx.y * nx + blockIdx.x;
+    const int64_t xcd = l % kXcds, slot = l / kXcds;
+    const int64_t per = n / kXcds, rem = n % kXcds;
+    const int64_t j = xcd * per + (xcd < rem ? xcd : rem) + slot;
+    bx = j % nx;
+    by = j / nx;
+}
+
 // LDS traffic between lanes of ONE wave: the wave's instructions execute in order, so a
 // ds_read issued after a ds_write sees it; this only stops the compiler from moving them.
 __device__ __forceinline__ void wave_lds_fence()
@@ -194,11 +211,12 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     const int wy = threadIdx.y;
     const int rq = lane / GL;
     const int gl = lane % GL;
-    const int64_t sample = blockIdx.y;
+    int64_t bx, sample;
+    xcd_swizzled_block(bx, sample);
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
     const int64_t ngroups = a.N / VALS;
-    const int64_t g0 = ((int64_t)blockIdx.x * kColsWaves + wy) * GL;
+    const int64_t g0 = (bx * kColsWaves + wy) * GL;
     if (g0 >= ngroups) return;  // whole wave outside (there is no block-level barrier below)
     const int64_t G = g0 + gl;
     const bool col_ok = G < ngroups;
@@ -344,10 +362,11 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     float *red = lds + KW * (CH * LPR);                 // [KW][LPR*VALS] block reduction
     const int r = lane / LPR;
     const int j = lane % LPR;
-    const int64_t sample = blockIdx.y;
+    int64_t split, sample;
+    xcd_swizzled_block(split, sample);
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
-    const int64_t kbeg = (int64_t)blockIdx.x * a.rows_per_split;
+    const int64_t kbeg = split * a.rows_per_split;
     const int64_t kend = kbeg + a.rows_per_split < a.K ? kbeg + a.rows_per_split : a.K;
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
@@ -448,7 +467,7 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
         if (a.splits == 1)
             a.out[sample * a.o_bs + m * a.o_rs + t] = __float2half_rn(v);
         else
-            a.partial[((sample * a.M + m) * a.splits + blockIdx.x) * a.N + t] = v;
+            a.partial[((sample * a.M + m) * a.splits + split) * a.N + t] = v;
     }
 }
 
