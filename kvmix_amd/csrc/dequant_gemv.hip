@@ -66,6 +66,8 @@ struct Fmt {
     static constexpr int BITS = MODE == 30 ? 3 : MODE;
     static constexpr int VALS = MODE == 3 ? 11 : 32;                       // codes per group unit
     static constexpr int WORDS = MODE == 3 ? 1 : (MODE == 30 ? 3 : MODE);  // words per group unit
+    // accumulate_unit leaves the 3-bit formats' sums scaled by 2^-59 (see there)
+    static constexpr float OUT_SCALE = (MODE == 3 || MODE == 30) ? 576460752303423488.0f : 1.0f;
 };
 
 // Vectors with relaxed alignment: the compiler still emits one wide global load, and gfx9
@@ -103,7 +105,7 @@ __device__ __forceinline__ void mix1(float q, uint32_t m, float &acc)
 template <int MODE>
 __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, float *acc)
 {
-    const float q0 = qs * 16777216.0f;  // 2^24 undoes the subnormal scaling
+    [[maybe_unused]] const float q0 = qs * 16777216.0f;  // 2^24 undoes the fp16-subnormal scaling
     if constexpr (MODE == 4) {
         const float q1 = q0 * 0.0625f;
 #pragma unroll
@@ -141,18 +143,40 @@ __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, flo
             mix2(qv[s], v & (0x00010001u << s), acc[s], acc[16 + s]);
             mix2(qv[s], v8 & (0x00010001u << s), acc[8 + s], acc[24 + s]);
         }
-    } else if constexpr (MODE == 3) {
+    } else {
+        // 3-bit formats: fields are not byte- or half-aligned, so the fp16 trick would need an
+        // extract per code.  Instead a masked field of a 32-bit word is read as an fp32
+        // SUBNORMAL: a pattern p < 2^24 is exactly p * 2^-149, so `word & (7 << o)` is
+        // code * 2^(o-149) and one v_and_b32 + one v_fmac_f32 (both 2-operand encodings, the
+        // cheapest VALU class) handle a code.  The multiplier carries 2^(90-o); the sums come
+        // out scaled by 2^(90-149) = 2^-59, undone by Fmt::OUT_SCALE.  2^90 keeps x*scale*2^90
+        // finite for any fp16 x and scale, and the products stay far above the fp32 subnormals.
+        float mq[4];
+        mq[0] = qs * 1237940039285380274899124224.0f;  // 2^90
 #pragma unroll
-        for (int i = 0; i < 10; i++) mix1(q0, (w[0] >> (3 * i)) & 7u, acc[i]);
-        mix1(q0, w[0] >> 30, acc[10]);
-    } else {  // dense 3-bit stream over three words
-        const uint64_t lo = (uint64_t)w[0] | ((uint64_t)w[1] << 32);
-        const uint64_t hi = (uint64_t)w[1] | ((uint64_t)w[2] << 32);
+        for (int s = 1; s < 4; s++) mq[s] = mq[s - 1] * 0.125f;  // offsets 0, 3, 6, 9
+        if constexpr (MODE == 3) {
+            // word = ten 3-bit codes at bits 0..29 + a 2-bit code at bits 30..31
+            const uint32_t v[3] = {w[0], w[0] >> 12, w[0] >> 24};
 #pragma unroll
-        for (int i = 0; i < 32; i++) {
-            const int bit = 3 * i;
-            const uint32_t c = bit < 32 ? (uint32_t)(lo >> bit) & 7u : (uint32_t)(hi >> (bit - 32)) & 7u;
-            mix1(q0, c, acc[i]);
+            for (int i = 0; i < 11; i++) {
+                const uint32_t mask = (i == 10 ? 3u : 7u) << (3 * (i % 4));
+                acc[i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & mask), acc[i]);
+            }
+        } else {
+            // 96-bit stream, code i at bits [3i, 3i+3): eight 12-bit windows of four codes
+            uint32_t v[8];
+            v[0] = w[0];
+            v[1] = w[0] >> 12;
+            v[2] = __builtin_amdgcn_alignbit(w[1], w[0], 24);
+            v[3] = w[1] >> 4;
+            v[4] = w[1] >> 16;
+            v[5] = __builtin_amdgcn_alignbit(w[2], w[1], 28);
+            v[6] = w[2] >> 8;
+            v[7] = w[2] >> 20;
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+                acc[i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & (7u << (3 * (i % 4)))), acc[i]);
         }
     }
 }
@@ -184,27 +208,38 @@ __device__ __forceinline__ void wave_lds_fence()
 }
 
 // ---------------------------------------------------------------------------------------
-// gemv_cols<MODE, RQ>
-//   wave tile  = GL = 64/RQ consecutive groups of N;  lane = (rq, gl): row section rq, group gl
-//   row chunk  = KC = 2048/GL rows (8 KiB of (scale, zero) pairs per wave in LDS); inside a
-//                chunk every lane walks KC/RQ = 32 rows of its section, 8 rows per load batch
-//   block = (64, NW) waves on NW neighbouring tiles; grid = (tiles/NW, samples, M)
+// gemv_cols<MODE, RQ, UPL>
+//   A lane owns UPL consecutive group units of N (one unit = one (scale, zero) pair: 32 codes,
+//   or one 11-code word of the reference's 3-bit format) for one of RQ sections of the K rows.
+//   wave tile  = TU = (64/RQ) * UPL consecutive units; the LAST tile of a row is shifted left
+//                so that it ends exactly at N: every lane of every tile is whole (the overlap
+//                is recomputed and stored twice with identical values), so there are no edge
+//                cases along N.  The host only takes this kernel when N holds >= TU units.
+//   row chunk  = KC = 2048/TU rows: 8 KiB of (scale, zero) half2 pairs per wave in LDS, staged
+//                with four 128-bit loads per array per lane; inside a chunk a lane walks
+//                KC/RQ = 32/UPL rows of its section, 8 rows of packed codes in flight.
+//   Rows past K (last chunk only) are read from row K-1 and meet x == 0.
+//   block = (64, 4) waves on neighbouring tiles; grid = (tiles/4, samples, M), XCD-swizzled.
+// Offsets inside one (batch, kv-head) slice are 32-bit (the host checks the extents).
 // ---------------------------------------------------------------------------------------
 constexpr int kColsWaves = 4;
 
-template <int MODE, int RQ>
+template <int MODE, int RQ, int UPL>
 __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
 {
     using F = Fmt<MODE>;
     constexpr int VALS = F::VALS, WORDS = F::WORDS;
-    constexpr int GL = kWave / RQ;      // groups per wave tile
-    constexpr int KC = 2048 / GL;       // rows per chunk
-    constexpr int RPL = KC / RQ;        // rows per lane per chunk (= 32)
+    constexpr int GL = kWave / RQ;      // lanes per row section
+    constexpr int TU = GL * UPL;        // units per wave tile
+    constexpr int KC = 2048 / TU;       // rows per chunk
+    constexpr int RPL = KC / RQ;        // rows per lane per chunk (= 32 / UPL)
     constexpr int U = 8;                // rows whose code loads are in flight together
-    constexpr int SEGS = GL / 8;        // 8-group segments per staged row
-    static_assert(RPL == 32 && RPL % U == 0, "chunk geometry");
+    constexpr int SEGS = TU / 8;        // 8-unit segments per staged row
+    constexpr int NIT = (KC * SEGS) / kWave;
+    constexpr int LW = WORDS * UPL;     // packed words per lane per row
+    static_assert(RPL % U == 0 && NIT == 4 && TU % 8 == 0, "chunk geometry");
 
-    __shared__ uint32_t sz_lds[kColsWaves][KC * GL];  // (scale | zero << 16) per (row, group)
+    __shared__ uint32_t sz_lds[kColsWaves][KC * TU];  // (scale | zero << 16) per (row, unit)
     __shared__ float x_lds[kColsWaves][KC];
 
     const int lane = threadIdx.x;
@@ -215,117 +250,127 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     xcd_swizzled_block(bx, sample);
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
-    const int64_t ngroups = a.N / VALS;
-    const int64_t g0 = (bx * kColsWaves + wy) * GL;
-    if (g0 >= ngroups) return;  // whole wave outside (there is no block-level barrier below)
-    const int64_t G = g0 + gl;
-    const bool col_ok = G < ngroups;
-    const int64_t Gc = col_ok ? G : ngroups - 1;  // clamped: loads stay in bounds, results dropped
+    const int K = (int)a.K;
+    const int nunits = (int)(a.N / VALS);
+    int t0 = (int)(bx * kColsWaves + wy) * TU;  // first unit of this wave's tile
+    if (t0 >= nunits) return;                   // whole wave outside (no block barrier below)
+    t0 = t0 + TU <= nunits ? t0 : nunits - TU;  // last tile: shifted left, still whole
+    const int unit0 = t0 + gl * UPL;            // this lane's first unit
+    const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
-    const uint32_t *cp = a.code + kv * a.c_bs + Gc * WORDS;
+    const uint32_t *cp = a.code + kv * a.c_bs;
     const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
     const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
     uint32_t *szw = sz_lds[wy];
     float *xw = x_lds[wy];
 
-    float acc[VALS];
+    float acc[UPL][VALS];
+    float zsum[UPL];
 #pragma unroll
-    for (int i = 0; i < VALS; i++) acc[i] = 0.f;
-    float zsum = 0.f;
+    for (int j = 0; j < UPL; j++) {
+        zsum[j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < VALS; i++) acc[j][i] = 0.f;
+    }
 
-    for (int64_t kc = 0; kc < a.K; kc += KC) {
-        const int rows = (int)(a.K - kc < KC ? a.K - kc : KC);
-        // ---- stage (scale, zero) of rows [kc, kc+rows) x groups [g0, g0+GL) and x[kc..] ----
+    const int r0 = rq * RPL;  // this lane's rows inside a chunk: [r0, r0 + RPL)
+    const uint32_t lane_word0 = (uint32_t)unit0 * WORDS;
+
+    for (int kc = 0; kc < K; kc += KC) {
+        const int rows = K - kc < KC ? K - kc : KC;
+        // ---- stage (scale, zero) of rows [kc, kc+rows) x units [t0, t0+TU), and x ----
+        {
+            Half8 s8[NIT], z8[NIT];
 #pragma unroll
-        for (int it = 0; it < (KC * SEGS) / kWave; it++) {
-            const int idx = it * kWave + lane;
-            const int row = idx / SEGS, seg = idx % SEGS;
-            const int64_t col = g0 + seg * 8;
-            uint16_t sv[8], zv[8];
-            if (row < rows && col + 8 <= ngroups) {
-                const Half8 s8 = *reinterpret_cast<const Half8 *>(sp + (kc + row) * a.s_rs + col);
-                const Half8 z8 = *reinterpret_cast<const Half8 *>(zp + (kc + row) * a.s_rs + col);
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    sv[e] = s8.v[e];
-                    zv[e] = z8.v[e];
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const bool ok = row < rows && col + e < ngroups;
-                    sv[e] = ok ? sp[(kc + row) * a.s_rs + col + e] : (uint16_t)0;
-                    zv[e] = ok ? zp[(kc + row) * a.s_rs + col + e] : (uint16_t)0;
-                }
+            for (int it = 0; it < NIT; it++) {
+                const int idx = it * kWave + lane;
+                const int row = idx / SEGS, seg = idx % SEGS;
+                const int rowc = kc + (row < rows ? row : rows - 1);
+                const uint32_t off = (uint32_t)rowc * s_rs + (uint32_t)(t0 + seg * 8);
+                s8[it] = *reinterpret_cast<const Half8 *>(sp + off);
+                z8[it] = *reinterpret_cast<const Half8 *>(zp + off);
             }
-            uint4 lo, hi;
-            lo.x = sv[0] | ((uint32_t)zv[0] << 16);
-            lo.y = sv[1] | ((uint32_t)zv[1] << 16);
-            lo.z = sv[2] | ((uint32_t)zv[2] << 16);
-            lo.w = sv[3] | ((uint32_t)zv[3] << 16);
-            hi.x = sv[4] | ((uint32_t)zv[4] << 16);
-            hi.y = sv[5] | ((uint32_t)zv[5] << 16);
-            hi.z = sv[6] | ((uint32_t)zv[6] << 16);
-            hi.w = sv[7] | ((uint32_t)zv[7] << 16);
-            uint4 *dst = reinterpret_cast<uint4 *>(szw + row * GL + seg * 8);
-            dst[0] = lo;
-            dst[1] = hi;
+#pragma unroll
+            for (int it = 0; it < NIT; it++) {
+                const int idx = it * kWave + lane;
+                uint32_t pk[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) pk[e] = s8[it].v[e] | ((uint32_t)z8[it].v[e] << 16);
+                uint4 *dst = reinterpret_cast<uint4 *>(szw + (idx / SEGS) * TU + (idx % SEGS) * 8);
+                dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+            }
+            for (int r = lane; r < KC; r += kWave) xw[r] = r < rows ? h16_to_f32(xp[kc + r]) : 0.f;
         }
-        for (int r = lane; r < KC; r += kWave) xw[r] = r < rows ? h16_to_f32(xp[kc + r]) : 0.f;
         wave_lds_fence();
 
-        // ---- stream the codes: lane walks rows [rq*RPL, rq*RPL + RPL) of the chunk ----
-        const int r0 = rq * RPL;
+        // ---- stream the codes ----
+        const bool full = rows == KC;
 #pragma unroll 1
         for (int b = 0; b < RPL; b += U) {
-            Words<WORDS> w[U];
+            Words<LW> w[U];
+            const int kfirst = kc + r0 + b;
+            if (full) {
+                const uint32_t off0 = (uint32_t)kfirst * c_rs + lane_word0;
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                int64_t k = kc + r0 + b + u;
-                k = k < a.K ? k : a.K - 1;  // rows past the end: x was staged as 0
-                w[u] = *reinterpret_cast<const Words<WORDS> *>(cp + k * a.c_rs);
+                for (int u = 0; u < U; u++)
+                    w[u] = *reinterpret_cast<const Words<LW> *>(cp + (off0 + (uint32_t)u * c_rs));
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const int k = kfirst + u < K ? kfirst + u : K - 1;
+                    w[u] = *reinterpret_cast<const Words<LW> *>(cp + ((uint32_t)k * c_rs + lane_word0));
+                }
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int r = r0 + b + u;
-                const half2_t sz = __builtin_bit_cast(half2_t, szw[r * GL + gl]);
                 const float xv = xw[r];
-                zsum = fmaf(xv, (float)sz.y, zsum);
-                accumulate_unit<MODE>(w[u].v, xv * (float)sz.x, acc);
+#pragma unroll
+                for (int j = 0; j < UPL; j++) {
+                    const half2_t sz = __builtin_bit_cast(half2_t, szw[r * TU + gl * UPL + j]);
+                    zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
+                    accumulate_unit<MODE>(w[u].v + j * WORDS, xv * (float)sz.x, acc[j]);
+                }
             }
         }
         wave_lds_fence();  // the next chunk overwrites the tile
     }
 
     // ---- combine the RQ row sections (butterfly over lanes), store fp16 ----
+    constexpr float kOut = F::OUT_SCALE;
 #pragma unroll
-    for (int i = 0; i < VALS; i++) {
-        float v = acc[i] + zsum;
+    for (int j = 0; j < UPL; j++) {
 #pragma unroll
-        for (int off = GL; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-        acc[i] = v;
+        for (int i = 0; i < VALS; i++) {
+            float v = fmaf(acc[j][i], kOut, zsum[j]);
+#pragma unroll
+            for (int off = GL; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+            acc[j][i] = v;
+        }
     }
-    if (!col_ok) return;
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + G * VALS;
-    if constexpr (VALS % RQ == 0 && (VALS / RQ) % 2 == 0) {
-        // every lane holds all sums: section rq stores its share of the group's outputs
-        constexpr int PER = VALS / RQ;
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
+    constexpr int TOT = UPL * VALS;  // consecutive outputs of this lane
+    if constexpr (TOT % (2 * RQ) == 0) {
+        // every lane of a column holds all sums: section rq stores its share
+        constexpr int PER = TOT / RQ;
 #pragma unroll
         for (int s = 0; s < RQ; s++) {
             if (rq == s) {
 #pragma unroll
                 for (int i = 0; i < PER; i += 2) {
-                    const uint32_t pk =
-                        f32_to_h16(acc[s * PER + i]) | ((uint32_t)f32_to_h16(acc[s * PER + i + 1]) << 16);
-                    __builtin_memcpy(op + s * PER + i, &pk, 4);
+                    const int e = s * PER + i;
+                    const uint32_t pk = f32_to_h16(acc[e / VALS][e % VALS]) |
+                                        ((uint32_t)f32_to_h16(acc[(e + 1) / VALS][(e + 1) % VALS]) << 16);
+                    __builtin_memcpy(op + e, &pk, 4);
                 }
             }
         }
     } else {
         if (rq == 0) {
 #pragma unroll
-            for (int i = 0; i < VALS; i++) op[i] = f32_to_h16(acc[i]);
+            for (int e = 0; e < TOT; e++) op[e] = f32_to_h16(acc[e / VALS][e % VALS]);
         }
     }
 }
@@ -384,46 +429,56 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     const int e0 = lane * 8;    // first element of the chunk's [CH][LPR] scale array this lane stages
     const int row0 = e0 / LPR;  // its 8 elements are RPS whole rows
 
-    for (int64_t k0 = kbeg + (int64_t)wy * CH; k0 < kend; k0 += (int64_t)KW * CH) {
-        const int rows = (int)(kend - k0 < CH ? kend - k0 : CH);
-        // ---- small operands first (so waiting for them leaves the code loads in flight) ----
-        uint16_t sv[8], zv[8], xh[RPS];
-        if (row0 + RPS <= rows) {
-            const Half8 s8 = *reinterpret_cast<const Half8 *>(sp + k0 * LPR + e0);
-            const Half8 z8 = *reinterpret_cast<const Half8 *>(zp + k0 * LPR + e0);
+    const uint32_t c_rs = (uint32_t)a.c_rs;
+    const int kb32 = (int)kbeg, ke32 = (int)kend;
+    for (int k0 = kb32 + wy * CH; k0 < ke32; k0 += KW * CH) {
+        const int rows = ke32 - k0 < CH ? ke32 - k0 : CH;
+        const bool full = rows == CH;
+        // ---- all loads of the chunk, none behind a branch that would drain the queue ----
+        // small operands first (so waiting for them leaves the code loads in flight); a lane
+        // whose staging rows are cut by the end of the range reads the last whole window (in
+        // bounds: the host routes K < 8 elsewhere) and is repaired below
+        int kr = k0 + row0;
+        kr = kr + RPS <= ke32 ? kr : ke32 - RPS;
+        kr = kr < 0 ? 0 : kr;
+        Half8 s8 = *reinterpret_cast<const Half8 *>(sp + (uint32_t)kr * LPR);
+        Half8 z8 = *reinterpret_cast<const Half8 *>(zp + (uint32_t)kr * LPR);
+        uint16_t xh[RPS];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                sv[e] = s8.v[e];
-                zv[e] = z8.v[e];
-            }
+        for (int q = 0; q < RPS; q++) xh[q] = xp[k0 + row0 + q < ke32 ? k0 + row0 + q : ke32 - 1];
+        Words<WORDS> w[TILES];
+        if (full) {
+            const uint32_t off0 = (uint32_t)(k0 + r) * c_rs;
 #pragma unroll
-            for (int q = 0; q < RPS; q++) xh[q] = xp[k0 + row0 + q];
+            for (int t = 0; t < TILES; t++)
+                w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (off0 + (uint32_t)(t * RPW) * c_rs));
         } else {
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                int row = t * RPW + r;
+                row = row < rows ? row : rows - 1;  // clamped rows meet x*scale == 0
+                w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (uint32_t)(k0 + row) * c_rs);
+            }
+        }
+        // ---- x*scale to LDS, x*zero into the private sums ----
+        if (!full && row0 + RPS > rows) {
+            // edge lane of the last chunk: element loads for the rows that exist
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const bool ok = (e0 + e) / LPR < rows;
-                sv[e] = ok ? sp[k0 * LPR + e0 + e] : (uint16_t)0;
-                zv[e] = ok ? zp[k0 * LPR + e0 + e] : (uint16_t)0;
+                const uint32_t off = (uint32_t)k0 * LPR + (ok ? e0 + e : 0);
+                const uint16_t s1 = sp[off], z1 = zp[off];
+                s8.v[e] = ok ? s1 : (uint16_t)0;
+                z8.v[e] = ok ? z1 : (uint16_t)0;
             }
-#pragma unroll
-            for (int q = 0; q < RPS; q++) xh[q] = row0 + q < rows ? xp[k0 + row0 + q] : (uint16_t)0;
         }
-        // ---- the chunk's packed codes: 8 tiles in flight ----
-        Words<WORDS> w[TILES];
-#pragma unroll
-        for (int t = 0; t < TILES; t++) {
-            int row = t * RPW + r;
-            row = row < rows ? row : rows - 1;  // clamped rows meet x*scale == 0
-            w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (k0 + row) * a.c_rs);
-        }
-        // ---- x*scale to LDS, x*zero into the private sums ----
         {
             float qv[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const float xv = h16_to_f32(xh[e / LPR]);
-                qv[e] = xv * h16_to_f32(sv[e]);
-                zacc[e % LPR] = fmaf(xv, h16_to_f32(zv[e]), zacc[e % LPR]);
+                const float xv = (full || row0 + e / LPR < rows) ? h16_to_f32(xh[e / LPR]) : 0.f;
+                qv[e] = xv * h16_to_f32(s8.v[e]);
+                zacc[e % LPR] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[e % LPR]);
             }
             float4 *dst = reinterpret_cast<float4 *>(qw + e0);
             dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
@@ -454,7 +509,7 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
         float v = acc[i];
 #pragma unroll
         for (int off = LPR; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-        acc[i] = v + zterm;
+        acc[i] = fmaf(v, F::OUT_SCALE, zterm);
     }
     if (r == 0) {
 #pragma unroll
@@ -528,7 +583,7 @@ __global__ void __launch_bounds__(256) gemv_generic(GemvArgs a)
     }
     __half *op = a.out + sample * a.o_bs + m * a.o_rs + u * VALS;
 #pragma unroll
-    for (int i = 0; i < VALS; i++) op[i] = __float2half_rn(acc[i] + zsum);
+    for (int i = 0; i < VALS; i++) op[i] = __float2half_rn(fmaf(acc[i], Fmt<MODE>::OUT_SCALE, zsum));
 }
 
 // --------------------------- host side ---------------------------
@@ -585,44 +640,62 @@ static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
     }
 }
 
-template <int MODE, int RQ>
-static void launch_cols_rq(const GemvArgs &a, int64_t samples, hipStream_t st)
-{
-    constexpr int VALS = Fmt<MODE>::VALS;
-    constexpr int GL = kWave / RQ;
-    const int64_t groups = a.N / VALS;
-    const int64_t tiles = (groups + GL - 1) / GL;
-    const dim3 grid((unsigned)((tiles + kColsWaves - 1) / kColsWaves), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL((gemv_cols<MODE, RQ>), grid, dim3(kWave, kColsWaves), 0, st, a);
-}
-
 #ifndef KVMIX_COLS_RQ
 #define KVMIX_COLS_RQ 0  // 0 = choose by problem size
 #endif
+
+// units one lane owns in gemv_cols: enough for a 128-bit code load per lane and row
+template <int MODE>
+struct ColsUpl {
+    static constexpr int value = MODE == 3 ? 4 : 1;
+};
+
+template <int MODE, int RQ, int UPL>
+static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    constexpr int VALS = Fmt<MODE>::VALS;
+    constexpr int TU = (kWave / RQ) * UPL;
+    const int64_t units = a.N / VALS;
+    const int64_t tiles = (units + TU - 1) / TU;
+    const dim3 grid((unsigned)((tiles + kColsWaves - 1) / kColsWaves), (unsigned)samples, (unsigned)a.M);
+    hipLaunchKernelGGL((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, kColsWaves), 0, st, a);
+}
+
+// smallest tile (in units) any gemv_cols configuration of this mode needs
+template <int MODE>
+static int64_t cols_min_units()
+{
+    // (the reference 3-bit format is not instantiated with four row sections: with four
+    // units per lane that configuration needs more registers than a wave may have)
+    return (MODE == 3 ? 32 : 16) * ColsUpl<MODE>::value;
+}
 
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
     // more row sections per wave = more, narrower waves: take the widest tile that still
-    // gives the chip enough waves
+    // gives the chip enough waves and fits into N
     constexpr int VALS = Fmt<MODE>::VALS;
-    const int64_t groups = a.N / VALS;
+    constexpr int UPL = ColsUpl<MODE>::value;
+    const int64_t units = a.N / VALS;
     const int64_t batch = samples * a.M;
     int rq = KVMIX_COLS_RQ;
     if (rq == 0) {
-        if (batch * ((groups + 63) / 64) >= kTargetWaves)
+        if (batch * ((units + 64 * UPL - 1) / (64 * UPL)) >= kTargetWaves)
             rq = 1;
-        else if (batch * ((groups + 31) / 32) >= kTargetWaves)
+        else if (batch * ((units + 32 * UPL - 1) / (32 * UPL)) >= kTargetWaves)
             rq = 2;
         else
             rq = 4;
     }
-    if (rq == 4 && a.K >= 128)
-        launch_cols_rq<MODE, 4>(a, samples, st);
-    else if (rq >= 2 && a.K >= 64)
-        launch_cols_rq<MODE, 2>(a, samples, st);
+    while (rq < 4 && units < (64 / rq) * UPL) rq *= 2;  // the tile must fit into N
+    if constexpr (MODE == 3) rq = rq > 2 ? 2 : rq;
+    if (rq == 4) {
+        if constexpr (MODE != 3) launch_cols_cfg<MODE, 4, UPL>(a, samples, st);
+    } else if (rq == 2)
+        launch_cols_cfg<MODE, 2, UPL>(a, samples, st);
     else
-        launch_cols_rq<MODE, 1>(a, samples, st);
+        launch_cols_cfg<MODE, 1, UPL>(a, samples, st);
 }
 
 template <int MODE>
@@ -701,10 +774,15 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     a.rows_per_split = K > 0 ? K : 1;
     hipStream_t st = (hipStream_t)stream;
 
-    const bool fast_group = ref3 ? true : group == 32;
+    // the fast kernels index one (batch, kv-head) slice with 32-bit offsets
+    const bool small = K < (1 << 30) && N < (1 << 30) && (K + 1) * code_row_stride < (1ll << 30) &&
+                       (K + 1) * sz_row_stride < (1ll << 30);
+    const bool fast_group = small && (ref3 ? true : group == 32);
     // gemv_rows reads a chunk's scale/zero as one flat array: rows must be contiguous
-    const bool rows_ok = fast_group && !ref3 && rows_shape_ok(N) && sz_row_stride == N / 32 && K > 0;
-    const bool cols_ok = fast_group && K > 0;
+    const bool rows_ok = fast_group && !ref3 && rows_shape_ok(N) && sz_row_stride == N / 32 && K >= 8;
+    // gemv_cols needs one whole wave tile of group units along N
+    const int64_t min_units = mode == 3 ? cols_min_units<3>() : cols_min_units<4>();
+    const bool cols_ok = fast_group && K > 0 && N / (ref3 ? 11 : 32) >= min_units;
     // p.V shape: few columns, many rows.  q.K^T shape: the opposite.
     const bool use_rows = rows_ok && (K >= 2 * N || !cols_ok);
 
