@@ -187,13 +187,13 @@ __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, flo
 // one cache row (they share the 128-byte lines that straddle tile borders) and query heads
 // of one kv head (they read the same packed data) then meet in one L2.
 constexpr int kXcds = 8;
-__device__ __forceinline__ void xcd_swizzled_block(int64_t &bx, int64_t &by)
+__device__ __forceinline__ void xcd_swizzled_block(int64_t &bx, int64_t &by, bool enable)
 {
     const int64_t nx = gridDim.x, n = nx * (int64_t)gridDim.y;
     const int64_t l = (int64_t)blockIdx.y * nx + blockIdx.x;
     const int64_t xcd = l % kXcds, slot = l / kXcds;
     const int64_t per = n / kXcds, rem = n % kXcds;
-    const int64_t j = xcd * per + (xcd < rem ? xcd : rem) + slot;
+    const int64_t j = enable ? xcd * per + (xcd < rem ? xcd : rem) + slot : l;
     bx = j % nx;
     by = j / nx;
 }
@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     const int rq = lane / GL;
     const int gl = lane % GL;
     int64_t bx, sample;
-    xcd_swizzled_block(bx, sample);
+    xcd_swizzled_block(bx, sample, true);
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
     const int K = (int)a.K;
@@ -277,63 +277,81 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     const int r0 = rq * RPL;  // this lane's rows inside a chunk: [r0, r0 + RPL)
     const uint32_t lane_word0 = (uint32_t)unit0 * WORDS;
 
-    for (int kc = 0; kc < K; kc += KC) {
-        const int rows = K - kc < KC ? K - kc : KC;
-        // ---- stage (scale, zero) of rows [kc, kc+rows) x units [t0, t0+TU), and x ----
-        {
-            Half8 s8[NIT], z8[NIT];
+    auto load_batch = [&](Words<LW>(&w)[U], int kc, int b, bool full) {
+        const int kfirst = kc + r0 + b;
+        if (full) {
+            const uint32_t off0 = (uint32_t)kfirst * c_rs + lane_word0;
 #pragma unroll
-            for (int it = 0; it < NIT; it++) {
-                const int idx = it * kWave + lane;
-                const int row = idx / SEGS, seg = idx % SEGS;
-                const int rowc = kc + (row < rows ? row : rows - 1);
-                const uint32_t off = (uint32_t)rowc * s_rs + (uint32_t)(t0 + seg * 8);
-                s8[it] = *reinterpret_cast<const Half8 *>(sp + off);
-                z8[it] = *reinterpret_cast<const Half8 *>(zp + off);
-            }
-#pragma unroll
-            for (int it = 0; it < NIT; it++) {
-                const int idx = it * kWave + lane;
-                uint32_t pk[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) pk[e] = s8[it].v[e] | ((uint32_t)z8[it].v[e] << 16);
-                uint4 *dst = reinterpret_cast<uint4 *>(szw + (idx / SEGS) * TU + (idx % SEGS) * 8);
-                dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-                dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
-            }
-            for (int r = lane; r < KC; r += kWave) xw[r] = r < rows ? h16_to_f32(xp[kc + r]) : 0.f;
-        }
-        wave_lds_fence();
-
-        // ---- stream the codes ----
-        const bool full = rows == KC;
-#pragma unroll 1
-        for (int b = 0; b < RPL; b += U) {
-            Words<LW> w[U];
-            const int kfirst = kc + r0 + b;
-            if (full) {
-                const uint32_t off0 = (uint32_t)kfirst * c_rs + lane_word0;
-#pragma unroll
-                for (int u = 0; u < U; u++)
-                    w[u] = *reinterpret_cast<const Words<LW> *>(cp + (off0 + (uint32_t)u * c_rs));
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int k = kfirst + u < K ? kfirst + u : K - 1;
-                    w[u] = *reinterpret_cast<const Words<LW> *>(cp + ((uint32_t)k * c_rs + lane_word0));
-                }
-            }
+            for (int u = 0; u < U; u++)
+                w[u] = *reinterpret_cast<const Words<LW> *>(cp + (off0 + (uint32_t)u * c_rs));
+        } else {
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int r = r0 + b + u;
-                const float xv = xw[r];
-#pragma unroll
-                for (int j = 0; j < UPL; j++) {
-                    const half2_t sz = __builtin_bit_cast(half2_t, szw[r * TU + gl * UPL + j]);
-                    zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
-                    accumulate_unit<MODE>(w[u].v + j * WORDS, xv * (float)sz.x, acc[j]);
-                }
+                const int k = kfirst + u < K ? kfirst + u : K - 1;
+                w[u] = *reinterpret_cast<const Words<LW> *>(cp + ((uint32_t)k * c_rs + lane_word0));
             }
+        }
+    };
+    auto compute_batch = [&](const Words<LW>(&w)[U], int b) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int r = r0 + b + u;
+            const float xv = xw[r];
+#pragma unroll
+            for (int j = 0; j < UPL; j++) {
+                const half2_t sz = __builtin_bit_cast(half2_t, szw[r * TU + gl * UPL + j]);
+                zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
+                accumulate_unit<MODE>(w[u].v + j * WORDS, xv * (float)sz.x, acc[j]);
+            }
+        }
+    };
+
+    for (int kc = 0; kc < K; kc += KC) {
+        const int rows = K - kc < KC ? K - kc : KC;
+        const bool full = rows == KC;
+        // ---- loads of the chunk's (scale, zero) tile and x, then -- before waiting for
+        //      them -- the first batch of packed codes ----
+        Half8 s8[NIT], z8[NIT];
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int idx = it * kWave + lane;
+            const int row = idx / SEGS, seg = idx % SEGS;
+            const int rowc = kc + (row < rows ? row : rows - 1);
+            const uint32_t off = (uint32_t)rowc * s_rs + (uint32_t)(t0 + seg * 8);
+            s8[it] = *reinterpret_cast<const Half8 *>(sp + off);
+            z8[it] = *reinterpret_cast<const Half8 *>(zp + off);
+        }
+        uint16_t xh[(KC + kWave - 1) / kWave];
+#pragma unroll
+        for (int i = 0; i < (KC + kWave - 1) / kWave; i++) {
+            const int r = i * kWave + lane;
+            xh[i] = xp[kc + (r < rows ? r : rows - 1)];
+        }
+        Words<LW> w[U];
+        load_batch(w, kc, 0, full);
+        // ---- tile to LDS ----
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int idx = it * kWave + lane;
+            uint32_t pk[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) pk[e] = s8[it].v[e] | ((uint32_t)z8[it].v[e] << 16);
+            uint4 *dst = reinterpret_cast<uint4 *>(szw + (idx / SEGS) * TU + (idx % SEGS) * 8);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        }
+#pragma unroll
+        for (int i = 0; i < (KC + kWave - 1) / kWave; i++) {
+            const int r = i * kWave + lane;
+            if (r < KC) xw[r] = r < rows ? h16_to_f32(xh[i]) : 0.f;
+        }
+        wave_lds_fence();
+        // ---- stream the codes ----
+        compute_batch(w, 0);
+#pragma unroll 1
+        for (int b = U; b < RPL; b += U) {
+            load_batch(w, kc, b, full);
+            compute_batch(w, b);
         }
         wave_lds_fence();  // the next chunk overwrites the tile
     }
@@ -407,8 +425,10 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     float *red = lds + KW * (CH * LPR);                 // [KW][LPR*VALS] block reduction
     const int r = lane / LPR;
     const int j = lane % LPR;
+    // (measured: with one query head per kv head nothing is shared between blocks and the
+    // launch order is 3 us faster at B=16, T=8k; with GQA the heads of a kv head want one L2)
     int64_t split, sample;
-    xcd_swizzled_block(split, sample);
+    xcd_swizzled_block(split, sample, a.heads_per_kv > 1);
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
     const int64_t kbeg = split * a.rows_per_split;
@@ -429,40 +449,43 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     const int e0 = lane * 8;    // first element of the chunk's [CH][LPR] scale array this lane stages
     const int row0 = e0 / LPR;  // its 8 elements are RPS whole rows
 
+    // ---- rotating software pipeline over this wave's chunks -----------------------------
+    // Register sets: S (scale / zero / x of a chunk), X (codes of row tiles 0..3), Y (tiles
+    // 4..7).  Each set is refilled with the NEXT chunk's data right after its last use, so
+    // while a chunk is being consumed the next one's loads are in flight and nothing is held
+    // twice.  No load sits behind a branch (a conditional load makes the compiler drain the
+    // whole queue): rows past the end are redirected to the last valid row and meet
+    // x*scale == 0; a prefetch past the last chunk re-reads the current one.
+    constexpr int HT = TILES / 2;
     const uint32_t c_rs = (uint32_t)a.c_rs;
-    const int kb32 = (int)kbeg, ke32 = (int)kend;
-    for (int k0 = kb32 + wy * CH; k0 < ke32; k0 += KW * CH) {
-        const int rows = ke32 - k0 < CH ? ke32 - k0 : CH;
-        const bool full = rows == CH;
-        // ---- all loads of the chunk, none behind a branch that would drain the queue ----
-        // small operands first (so waiting for them leaves the code loads in flight); a lane
-        // whose staging rows are cut by the end of the range reads the last whole window (in
-        // bounds: the host routes K < 8 elsewhere) and is repaired below
-        int kr = k0 + row0;
-        kr = kr + RPS <= ke32 ? kr : ke32 - RPS;
+    const int ke32 = (int)kend;
+    const int stride = KW * CH;
+    const int kfirst = (int)kbeg + wy * CH;
+    Half8 s8, z8;
+    uint16_t xh[RPS];
+    Words<WORDS> wx[HT], wz[HT];
+
+    auto load_small = [&](int k0) {
+        int kr = k0 + row0;  // a window cut by the end of the range is read one window early
+        kr = kr + RPS <= ke32 ? kr : ke32 - RPS;  // (in bounds: the host routes K < 8 elsewhere)
         kr = kr < 0 ? 0 : kr;
-        Half8 s8 = *reinterpret_cast<const Half8 *>(sp + (uint32_t)kr * LPR);
-        Half8 z8 = *reinterpret_cast<const Half8 *>(zp + (uint32_t)kr * LPR);
-        uint16_t xh[RPS];
+        s8 = *reinterpret_cast<const Half8 *>(sp + (uint32_t)kr * LPR);
+        z8 = *reinterpret_cast<const Half8 *>(zp + (uint32_t)kr * LPR);
 #pragma unroll
         for (int q = 0; q < RPS; q++) xh[q] = xp[k0 + row0 + q < ke32 ? k0 + row0 + q : ke32 - 1];
-        Words<WORDS> w[TILES];
-        if (full) {
-            const uint32_t off0 = (uint32_t)(k0 + r) * c_rs;
+    };
+    auto load_codes = [&](Words<WORDS>(&w)[HT], int k0, int t0) {
 #pragma unroll
-            for (int t = 0; t < TILES; t++)
-                w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (off0 + (uint32_t)(t * RPW) * c_rs));
-        } else {
-#pragma unroll
-            for (int t = 0; t < TILES; t++) {
-                int row = t * RPW + r;
-                row = row < rows ? row : rows - 1;  // clamped rows meet x*scale == 0
-                w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (uint32_t)(k0 + row) * c_rs);
-            }
+        for (int t = 0; t < HT; t++) {
+            int k = k0 + (t0 + t) * RPW + r;
+            k = k < ke32 ? k : ke32 - 1;
+            w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (uint32_t)k * c_rs);
         }
-        // ---- x*scale to LDS, x*zero into the private sums ----
-        if (!full && row0 + RPS > rows) {
-            // edge lane of the last chunk: element loads for the rows that exist
+    };
+    auto stage = [&](int k0) {
+        const int rows = ke32 - k0;  // >= 1; >= CH for every chunk but the last
+        if (row0 < rows && row0 + RPS > rows) {
+            // the lane whose window is cut by the end of the range: element loads
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const bool ok = (e0 + e) / LPR < rows;
@@ -472,25 +495,41 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
                 z8.v[e] = ok ? z1 : (uint16_t)0;
             }
         }
-        {
-            float qv[8];
+        float qv[8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float xv = (full || row0 + e / LPR < rows) ? h16_to_f32(xh[e / LPR]) : 0.f;
-                qv[e] = xv * h16_to_f32(s8.v[e]);
-                zacc[e % LPR] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[e % LPR]);
-            }
-            float4 *dst = reinterpret_cast<float4 *>(qw + e0);
-            dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
-            dst[1] = make_float4(qv[4], qv[5], qv[6], qv[7]);
+        for (int e = 0; e < 8; e++) {
+            const float xv = row0 + e / LPR < rows ? h16_to_f32(xh[e / LPR]) : 0.f;
+            qv[e] = xv * h16_to_f32(s8.v[e]);
+            zacc[e % LPR] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[e % LPR]);
         }
-        wave_lds_fence();
+        float4 *dst = reinterpret_cast<float4 *>(qw + e0);
+        dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
+        dst[1] = make_float4(qv[4], qv[5], qv[6], qv[7]);
+    };
+    auto compute = [&](const Words<WORDS>(&w)[HT], int t0) {
 #pragma unroll
-        for (int t = 0; t < TILES; t++) {
-            const float qs = qw[(t * RPW + r) * LPR + j];
+        for (int t = 0; t < HT; t++) {
+            const float qs = qw[((t0 + t) * RPW + r) * LPR + j];
             accumulate_unit<MODE>(w[t].v, qs, acc);
         }
-        wave_lds_fence();
+    };
+
+    if (kfirst < ke32) {
+        load_small(kfirst);
+        load_codes(wx, kfirst, 0);
+        load_codes(wz, kfirst, HT);
+#pragma unroll 1
+        for (int k0 = kfirst; k0 < ke32; k0 += stride) {
+            const int kn = k0 + stride < ke32 ? k0 + stride : k0;
+            stage(k0);
+            wave_lds_fence();
+            load_small(kn);
+            compute(wx, 0);
+            load_codes(wx, kn, 0);
+            compute(wz, HT);
+            load_codes(wz, kn, HT);
+            wave_lds_fence();  // the next chunk overwrites the tile
+        }
     }
 
     // zero term: zacc[g] summed over all lanes of the wave (every lane staged other rows)
