@@ -233,3 +233,89 @@ def test_full_size_properties_b16_t8192(dev):
         ref = torch.matmul(pr.float(), deq)
         ab = torch.matmul(pr.float().abs(), deq.abs())
         assert ((out - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
+
+
+def _unpack_torch(code, bits):
+    """Reference-layout unpack on the GPU with torch integer ops (test-side checker)."""
+    dev = code.device
+    if bits == 3:
+        shifts = torch.tensor([3 * i for i in range(10)] + [30], device=dev, dtype=torch.int32)
+        masks = torch.tensor([7] * 10 + [3], device=dev, dtype=torch.int32)
+    else:
+        shifts = torch.arange(0, 32, bits, device=dev, dtype=torch.int32)
+        masks = torch.full((32 // bits,), (1 << bits) - 1, device=dev, dtype=torch.int32)
+    q = (code.unsqueeze(-1) >> shifts) & masks
+    return q.reshape(code.shape[:-1] + (code.shape[-1] * shifts.numel(),))
+
+
+def test_full_size_properties_gqa_32k(dev):
+    """BASELINE configs[2] shape: 32 query heads on 8 kv heads, head_dim 128, batch 16, 32768
+    tokens, reference 3-bit keys (32637 = 11 * 2967 quantized tokens) and 2-bit values (32640)."""
+    import KVmix
+
+    torch.manual_seed(2)
+    B, H, Hkv, D = 16, 32, 8, 128
+    Tqk, Tqv = 32637, 32640
+    kcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, D, Tqk // 11), dtype=torch.int64, device=dev).to(torch.int32)
+    ones = torch.ones(B, Hkv, D, Tqk // 11, dtype=torch.float16, device=dev)
+    x1 = torch.ones(B, H, 1, D, dtype=torch.float16, device=dev)
+    out = KVmix.quantized_gemm(11, x1, kcode, ones, torch.zeros_like(ones), 3)
+    assert out.shape == (B, H, 1, Tqk)
+    for b0 in range(0, B, 4):
+        sums = _unpack_torch(kcode[b0:b0 + 4], 3).sum(2)                       # [4, Hkv, Tqk] <= 128*7
+        got = out[b0:b0 + 4, :, 0].to(torch.int32).reshape(4, Hkv, H // Hkv, Tqk)
+        assert torch.equal(got, sums.unsqueeze(2).expand_as(got))              # every head of a group
+    # values: one-hot probabilities pick one dequantized row, per query head
+    vcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, Tqv, D // 16), dtype=torch.int64, device=dev).to(torch.int32)
+    vs = (torch.rand(B, Hkv, Tqv, D // 32, device=dev) + 0.5).half()
+    vz = torch.randn(B, Hkv, Tqv, D // 32, device=dev).half()
+    p = torch.zeros(B, H, 1, Tqv, dtype=torch.float16, device=dev)
+    rows = torch.randint(0, Tqv, (H,), device=dev)
+    for h in range(H):
+        p[:, h, 0, rows[h]] = 1
+    out = KVmix.quantized_gemm(32, p, vcode, vs, vz, 2)
+    for h in range(H):
+        r, kvh = int(rows[h]), h // (H // Hkv)
+        qv = _unpack_torch(vcode[:, kvh, r], 2).float()
+        want = (vs[:, kvh, r].float().repeat_interleave(32, -1) * qv + vz[:, kvh, r].float().repeat_interleave(32, -1)).half()
+        assert torch.equal(out[:, h, 0], want), h
+    # dense check of two batch entries against torch's fp32 matmul of the dequantized values
+    pr = torch.softmax(torch.randn(2, H, 1, Tqv, device=dev), -1).half()
+    out = KVmix.quantized_gemm(32, pr, vcode[:2], vs[:2], vz[:2], 2).float()
+    deq = vs[:2].float().repeat_interleave(32, -1) * _unpack_torch(vcode[:2], 2).float() + vz[:2].float().repeat_interleave(32, -1)
+    deq = deq.repeat_interleave(H // Hkv, dim=1)
+    ref = torch.matmul(pr.float(), deq)
+    ab = torch.matmul(pr.float().abs(), deq.abs())
+    assert ((out - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+def test_full_size_properties_batch128_t4096(dev, bits):
+    """BASELINE configs[3] at its largest batch: 128 x 32 heads, 4064 quantized tokens, 1/2 bits."""
+    import KVmix
+
+    torch.manual_seed(3)
+    B, H, D, Tq, g = 128, 32, 128, 4064, 32
+    vpw = 32 // bits
+    kcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq // vpw), dtype=torch.int64, device=dev).to(torch.int32)
+    ones = torch.ones(B, H, D, Tq // g, dtype=torch.float16, device=dev)
+    x1 = torch.ones(B, H, 1, D, dtype=torch.float16, device=dev)
+    out = KVmix.quantized_gemm(g, x1, kcode, ones, torch.zeros_like(ones), bits)
+    for b0 in range(0, B, 16):
+        assert torch.equal(out[b0:b0 + 16, :, 0].to(torch.int32), _unpack_torch(kcode[b0:b0 + 16], bits).sum(2))
+    del kcode, ones
+    vcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D // vpw), dtype=torch.int64, device=dev).to(torch.int32)
+    vs = (torch.rand(B, H, Tq, D // g, device=dev) + 0.5).half()
+    vz = torch.randn(B, H, Tq, D // g, device=dev).half()
+    p = torch.zeros(B, H, 1, Tq, dtype=torch.float16, device=dev)
+    p[..., 4063] = 1
+    out = KVmix.quantized_gemm(g, p, vcode, vs, vz, bits)
+    qv = _unpack_torch(vcode[:, :, 4063], bits).float()
+    want = (vs[:, :, 4063].float().repeat_interleave(g, -1) * qv + vz[:, :, 4063].float().repeat_interleave(g, -1)).half()
+    assert torch.equal(out[:, :, 0], want)
+    # all-ones probabilities with scale 1, zero 0: exact integer sums over tokens (<= 4064 * 3, exact in fp16 up to 2048)
+    if bits == 1:
+        one = torch.ones_like(vs)
+        out = KVmix.quantized_gemm(g, torch.ones_like(p)[..., :2016], vcode[:, :, :2016], one[:, :, :2016],
+                                   torch.zeros_like(one)[:, :, :2016], bits)
+        assert torch.equal(out[:, :, 0].to(torch.int32), _unpack_torch(vcode[:, :, :2016], bits).sum(2))
