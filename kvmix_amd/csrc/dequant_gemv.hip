@@ -181,6 +181,79 @@ __device__ __forceinline__ void accumulate_unit(const uint32_t *w, float qs, flo
     }
 }
 
+// The same unpack for NREP query heads that share one kv head (GQA): the field of a code is
+// isolated ONCE as an fp32 subnormal (`word & mask` is code * 2^(offset-149)) and each head
+// pays a single v_fmac_f32.  Shifted copies of the word keep the number of distinct field
+// offsets -- hence of per-head multipliers q * 2^(90-offset) -- at four (eight for 1 bit).
+// The sums come out scaled by 2^-59 (kHeadsOutScale undoes it), for every format.
+constexpr float kHeadsOutScale = 576460752303423488.0f;  // 2^59
+
+template <int MODE, int NREP>
+__device__ __forceinline__ void accumulate_heads(const uint32_t *w, const float *q,
+                                                 float (*acc)[Fmt<MODE>::VALS])
+{
+    constexpr int NM = MODE == 1 ? 8 : 4;                       // distinct field offsets
+    constexpr int STEP = MODE == 30 ? 3 : MODE;                 // bits between fields of a copy
+    constexpr float DOWN = MODE == 4 ? 0.0625f : (MODE == 2 ? 0.25f : (MODE == 1 ? 0.5f : 0.125f));
+    float mq[NREP][NM];
+#pragma unroll
+    for (int h = 0; h < NREP; h++) {
+        mq[h][0] = q[h] * 1237940039285380274899124224.0f;  // 2^90
+#pragma unroll
+        for (int s = 1; s < NM; s++) mq[h][s] = mq[h][s - 1] * DOWN;
+    }
+    // one masked field -> NREP fmacs
+    auto field = [&](uint32_t copy, uint32_t mask, int s, int code) {
+        const float f = __uint_as_float(copy & mask);
+#pragma unroll
+        for (int h = 0; h < NREP; h++) acc[h][code] = fmaf(mq[h][s], f, acc[h][code]);
+    };
+    if constexpr (MODE == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {  // nibble i at bit 4i: copies w and w >> 16, offsets 0,4,8,12
+            const uint32_t v0 = w[j], v1 = w[j] >> 16;
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                field(v0, 0xFu << (4 * s), s, 8 * j + s);
+                field(v1, 0xFu << (4 * s), s, 8 * j + 4 + s);
+            }
+        }
+    } else if constexpr (MODE == 2) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {  // code i at bit 2i: copies w >> 8k, offsets 0,2,4,6
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t v = w[j] >> (8 * k);
+#pragma unroll
+                for (int s = 0; s < 4; s++) field(v, 3u << (2 * s), s, 16 * j + 4 * k + s);
+            }
+        }
+    } else if constexpr (MODE == 1) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {  // bit i: copies w >> 8k, offsets 0..7
+            const uint32_t v = w[0] >> (8 * k);
+#pragma unroll
+            for (int s = 0; s < 8; s++) field(v, 1u << s, s, 8 * k + s);
+        }
+    } else if constexpr (MODE == 3) {
+        const uint32_t v[3] = {w[0], w[0] >> 12, w[0] >> 24};
+#pragma unroll
+        for (int i = 0; i < 11; i++) field(v[i / 4], (i == 10 ? 3u : 7u) << (3 * (i % 4)), i % 4, i);
+    } else {
+        uint32_t v[8];
+        v[0] = w[0];
+        v[1] = w[0] >> 12;
+        v[2] = __builtin_amdgcn_alignbit(w[1], w[0], 24);
+        v[3] = w[1] >> 4;
+        v[4] = w[1] >> 16;
+        v[5] = __builtin_amdgcn_alignbit(w[2], w[1], 28);
+        v[6] = w[2] >> 8;
+        v[7] = w[2] >> 20;
+#pragma unroll
+        for (int i = 0; i < 32; i++) field(v[i / 4], 7u << (3 * (i % 4)), i % 4, i);
+    }
+}
+
 // Workgroups are handed to the 8 XCDs (each with its own L2) round-robin in launch order, so
 // neighbours in launch order never share an L2.  This maps the launch-order index to a
 // logical index such that CONSECUTIVE logical indices run on the SAME XCD: column tiles of
@@ -393,6 +466,29 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     }
 }
 
+// Halving butterfly over lanes.  v[0..NV) of every lane are summed across the lanes whose
+// indices differ in the bits {FIRST, 2*FIRST, ...} (UP = 1: up to bit 32; UP = 0: FIRST, FIRST/2,
+// ... down to bit 1).  A step halves what a lane holds: the lane with the step's bit clear
+// keeps the lower half, its partner the upper half.  Returns the index (in the original
+// numbering) of the value left in v[0]; the lane's remaining values follow it in order.
+template <int NV, int FIRST, int UP>
+__device__ __forceinline__ int scatter_reduce(float *v, int lane)
+{
+    if constexpr (NV <= 1 || FIRST < 1 || FIRST >= kWave) {
+        return 0;
+    } else {
+        constexpr int H = NV / 2;
+        const bool up = (lane & FIRST) != 0;
+#pragma unroll
+        for (int i = 0; i < H; i++) {
+            const float keep = up ? v[H + i] : v[i];
+            const float send = up ? v[i] : v[H + i];
+            v[i] = keep + __shfl_xor(send, FIRST);
+        }
+        return (up ? H : 0) + scatter_reduce<H, UP ? FIRST * 2 : FIRST / 2, UP>(v, lane);
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // gemv_rows<MODE, LPR>
 //   LPR = N/32 lanes per row (one 32-code group each), RPW = 64/LPR rows per tile,
@@ -403,10 +499,15 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
 //   block = (64, KW); grid = (splits, samples, M); dynamic LDS = KW * (512 + N) floats.
 //   Requires scale/zero rows to be contiguous (row stride == LPR).
 // ---------------------------------------------------------------------------------------
-constexpr int kRowsMaxWaves = 16;
+constexpr int kRowsMaxWaves = 16;  // plain (one head per block) configuration
 
-template <int MODE, int LPR>
-__global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
+// NREP > 1 (GQA): one block serves NREP query heads of a kv head from one pass over the
+// packed data -- NREP x 32 accumulators per lane, so such a block has at most four waves and
+// the kernel is compiled for the larger register budget that goes with it.
+constexpr int kRowsHeadsWaves = 4;
+
+template <int MODE, int LPR, int NREP>
+__global__ void __launch_bounds__(NREP > 1 ? 64 * kRowsHeadsWaves : 64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
 {
     using F = Fmt<MODE>;
     constexpr int VALS = F::VALS, WORDS = F::WORDS;
@@ -416,35 +517,42 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     constexpr int TILES = 8;           // tiles per chunk, all in flight
     constexpr int CH = TILES * RPW;    // rows per chunk (= 512 / LPR)
     constexpr int RPS = 8 / LPR;       // rows covered by one staging lane's 8 halves
+    constexpr int QT = CH * LPR;       // floats of one head's x*scale tile (= 512)
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
     const int wy = threadIdx.y;
     const int KW = blockDim.y;
-    float *qw = lds + wy * (CH * LPR);                  // this wave's x*scale tile
-    float *red = lds + KW * (CH * LPR);                 // [KW][LPR*VALS] block reduction
+    float *qw = lds + wy * (NREP * QT);           // this wave's x*scale tiles, one per query head
+    float *red = lds + KW * (NREP * QT);          // [KW][NREP][LPR*VALS] block reduction
     const int r = lane / LPR;
     const int j = lane % LPR;
+    // grid.y counts head groups: NREP query heads that share one kv head (NREP divides
+    // heads_per_kv; NREP == 1 is the plain case)
     // (measured: with one query head per kv head nothing is shared between blocks and the
     // launch order is 3 us faster at B=16, T=8k; with GQA the heads of a kv head want one L2)
-    int64_t split, sample;
-    xcd_swizzled_block(split, sample, a.heads_per_kv > 1);
+    int64_t split, hg;
+    xcd_swizzled_block(split, hg, a.heads_per_kv > NREP);
+    const int64_t sample0 = hg * NREP;
     const int64_t m = blockIdx.z;
-    const int64_t kv = sample / a.heads_per_kv;
+    const int64_t kv = sample0 / a.heads_per_kv;
     const int64_t kbeg = split * a.rows_per_split;
     const int64_t kend = kbeg + a.rows_per_split < a.K ? kbeg + a.rows_per_split : a.K;
 
-    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
     const uint32_t *cp = a.code + kv * a.c_bs + j * WORDS;
     const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
     const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
 
-    float acc[VALS];
+    float acc[NREP][VALS];
+    float zacc[NREP][LPR];  // x*zero sums of the elements this lane staged, by head and group
 #pragma unroll
-    for (int i = 0; i < VALS; i++) acc[i] = 0.f;
-    float zacc[LPR];  // x*zero sums of the elements this lane staged, by group
+    for (int h = 0; h < NREP; h++) {
 #pragma unroll
-    for (int i = 0; i < LPR; i++) zacc[i] = 0.f;
+        for (int i = 0; i < VALS; i++) acc[h][i] = 0.f;
+#pragma unroll
+        for (int i = 0; i < LPR; i++) zacc[h][i] = 0.f;
+    }
 
     const int e0 = lane * 8;    // first element of the chunk's [CH][LPR] scale array this lane stages
     const int row0 = e0 / LPR;  // its 8 elements are RPS whole rows
@@ -456,13 +564,15 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
     // twice.  No load sits behind a branch (a conditional load makes the compiler drain the
     // whole queue): rows past the end are redirected to the last valid row and meet
     // x*scale == 0; a prefetch past the last chunk re-reads the current one.
+    // With NREP > 1 the packed codes, scales and zeros are loaded once and used for every
+    // query head of the group; the field masks of the unpack are shared as well.
     constexpr int HT = TILES / 2;
     const uint32_t c_rs = (uint32_t)a.c_rs;
     const int ke32 = (int)kend;
     const int stride = KW * CH;
     const int kfirst = (int)kbeg + wy * CH;
     Half8 s8, z8;
-    uint16_t xh[RPS];
+    uint16_t xh[NREP][RPS];
     Words<WORDS> wx[HT], wz[HT];
 
     auto load_small = [&](int k0) {
@@ -472,7 +582,11 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
         s8 = *reinterpret_cast<const Half8 *>(sp + (uint32_t)kr * LPR);
         z8 = *reinterpret_cast<const Half8 *>(zp + (uint32_t)kr * LPR);
 #pragma unroll
-        for (int q = 0; q < RPS; q++) xh[q] = xp[k0 + row0 + q < ke32 ? k0 + row0 + q : ke32 - 1];
+        for (int h = 0; h < NREP; h++) {
+#pragma unroll
+            for (int q = 0; q < RPS; q++)
+                xh[h][q] = xp[h * a.x_bs + (k0 + row0 + q < ke32 ? k0 + row0 + q : ke32 - 1)];
+        }
     };
     auto load_codes = [&](Words<WORDS>(&w)[HT], int k0, int t0) {
 #pragma unroll
@@ -495,22 +609,37 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
                 z8.v[e] = ok ? z1 : (uint16_t)0;
             }
         }
-        float qv[8];
+        float sf[8], zf[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float xv = row0 + e / LPR < rows ? h16_to_f32(xh[e / LPR]) : 0.f;
-            qv[e] = xv * h16_to_f32(s8.v[e]);
-            zacc[e % LPR] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[e % LPR]);
+            sf[e] = h16_to_f32(s8.v[e]);
+            zf[e] = h16_to_f32(z8.v[e]);
         }
-        float4 *dst = reinterpret_cast<float4 *>(qw + e0);
-        dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
-        dst[1] = make_float4(qv[4], qv[5], qv[6], qv[7]);
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+            float qv[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float xv = row0 + e / LPR < rows ? h16_to_f32(xh[h][e / LPR]) : 0.f;
+                qv[e] = xv * sf[e];
+                zacc[h][e % LPR] = fmaf(xv, zf[e], zacc[h][e % LPR]);
+            }
+            float4 *dst = reinterpret_cast<float4 *>(qw + h * QT + e0);
+            dst[0] = make_float4(qv[0], qv[1], qv[2], qv[3]);
+            dst[1] = make_float4(qv[4], qv[5], qv[6], qv[7]);
+        }
     };
     auto compute = [&](const Words<WORDS>(&w)[HT], int t0) {
 #pragma unroll
         for (int t = 0; t < HT; t++) {
-            const float qs = qw[((t0 + t) * RPW + r) * LPR + j];
-            accumulate_unit<MODE>(w[t].v, qs, acc);
+            if constexpr (NREP == 1) {
+                accumulate_unit<MODE>(w[t].v, qw[((t0 + t) * RPW + r) * LPR + j], acc[0]);
+            } else {
+                float qs[NREP];
+#pragma unroll
+                for (int h = 0; h < NREP; h++) qs[h] = qw[h * QT + ((t0 + t) * RPW + r) * LPR + j];
+                accumulate_heads<MODE, NREP>(w[t].v, qs, acc);
+            }
         }
     };
 
@@ -532,36 +661,46 @@ __global__ void __launch_bounds__(64 * kRowsMaxWaves) gemv_rows(GemvArgs a)
         }
     }
 
-    // zero term: zacc[g] summed over all lanes of the wave (every lane staged other rows)
+    // ---- reduce over the wave's rows ------------------------------------------------------
+    // Both sums use a halving butterfly: at every step a lane keeps one half of its values
+    // and hands the other half to its partner, so the exchange count halves per step.
+    // zero term: zacc[h][g] summed over all lanes; lane (r, j) ends with the sum for g == j
+    float zterm[NREP];
 #pragma unroll
-    for (int g = 0; g < LPR; g++) {
-        float v = zacc[g];
+    for (int h = 0; h < NREP; h++) {
+        float z[LPR];
 #pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-        zacc[g] = v;
+        for (int g = 0; g < LPR; g++) z[g] = zacc[h][g];
+        scatter_reduce<LPR, LPR / 2, 0>(z, lane);          // over j: the lane's own group remains
+#pragma unroll
+        for (int off = LPR; off < kWave; off <<= 1) z[0] += __shfl_xor(z[0], off);  // over rows
+        zterm[h] = z[0];
     }
-    float zterm = 0.f;
+    // code sums: NREP*32 values summed over the RPW rows, NREP*32/RPW of them left per lane
+    constexpr int NV = NREP * VALS;
+    constexpr int KEEP = NV / RPW;
+    static_assert(KEEP >= 1, "a lane keeps at least one sum");
+    float *flat = &acc[0][0];
+    const int first = scatter_reduce<NV, LPR, 1>(flat, lane);  // index (h*32 + i) of flat[0]
 #pragma unroll
-    for (int g = 0; g < LPR; g++) zterm = (j == g) ? zacc[g] : zterm;
+    for (int i = 0; i < KEEP; i++) {
+        const int f = first + i;
+        const int h = f / VALS;  // (KEEP divides 32: a lane's sums belong to one head)
+        float zt = zterm[0];
 #pragma unroll
-    for (int i = 0; i < VALS; i++) {
-        float v = acc[i];
-#pragma unroll
-        for (int off = LPR; off < kWave; off <<= 1) v += __shfl_xor(v, off);
-        acc[i] = fmaf(v, F::OUT_SCALE, zterm);
-    }
-    if (r == 0) {
-#pragma unroll
-        for (int i = 0; i < VALS; i++) red[wy * (LPR * VALS) + j * VALS + i] = acc[i];
+        for (int hh = 1; hh < NREP; hh++) zt = h == hh ? zterm[hh] : zt;
+        red[(wy * NREP + h) * (LPR * VALS) + j * VALS + f % VALS] =
+            fmaf(flat[i], NREP == 1 ? F::OUT_SCALE : kHeadsOutScale, zt);
     }
     __syncthreads();
-    for (int t = wy * kWave + lane; t < LPR * VALS; t += KW * kWave) {
+    for (int t = wy * kWave + lane; t < NREP * LPR * VALS; t += KW * kWave) {
+        const int h = t / (LPR * VALS), n = t % (LPR * VALS);
         float v = 0.f;
-        for (int w = 0; w < KW; w++) v += red[w * (LPR * VALS) + t];
+        for (int w = 0; w < KW; w++) v += red[(w * NREP + h) * (LPR * VALS) + n];
         if (a.splits == 1)
-            a.out[sample * a.o_bs + m * a.o_rs + t] = __float2half_rn(v);
+            a.out[(sample0 + h) * a.o_bs + m * a.o_rs + n] = __float2half_rn(v);
         else
-            a.partial[((sample * a.M + m) * a.splits + split) * a.N + t] = v;
+            a.partial[(((sample0 + h) * a.M + m) * a.splits + split) * a.N + n] = v;
     }
 }
 
@@ -638,7 +777,7 @@ struct RowsPlan {
 };
 
 // How gemv_rows covers K for `batch_rows` = samples*M independent outputs.
-static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N)
+static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_waves)
 {
     RowsPlan p{4, 1, K > 0 ? K : 1};
     if (!rows_shape_ok(N) || batch_rows <= 0 || K <= 0) return p;
@@ -647,7 +786,7 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N)
     int64_t want = (kTargetWaves + batch_rows - 1) / batch_rows;  // waves wanted per output row
     if (want > chunks) want = chunks;
     if (want < 1) want = 1;
-    int64_t waves = want < kRowsMaxWaves ? want : kRowsMaxWaves;
+    int64_t waves = want < max_waves ? want : max_waves;
     if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
     int64_t splits = (want + waves - 1) / waves;
     if (splits > 64) splits = 64;
@@ -660,23 +799,36 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N)
     return p;
 }
 
-template <int MODE>
-static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
+// query heads one block of gemv_rows / gemv_cols serves from a single pass over the packed data
+static int heads_per_block(int heads_per_kv) { return heads_per_kv % 4 == 0 ? 4 : 1; }
+
+template <int MODE, int NREP>
+static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
 {
-    const RowsPlan p = plan_rows(samples * a.M, a.K, a.N);
+    // (a block's LDS is waves * NREP * (512 + N) floats)
+    const RowsPlan p = plan_rows(samples / NREP * a.M, a.K, a.N, NREP > 1 ? kRowsHeadsWaves : kRowsMaxWaves);
     a.splits = p.splits;
     a.rows_per_split = p.rows_per_split;
-    const dim3 grid((unsigned)a.splits, (unsigned)samples, (unsigned)a.M), block(kWave, p.waves);
-    const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)(512 + a.N);
+    const dim3 grid((unsigned)a.splits, (unsigned)(samples / NREP), (unsigned)a.M), block(kWave, p.waves);
+    const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)NREP * (size_t)(512 + a.N);
     switch (a.N / 32) {
-    case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2>), grid, block, lds, st, a); break;
-    case 4: hipLaunchKernelGGL((gemv_rows<MODE, 4>), grid, block, lds, st, a); break;
-    default: hipLaunchKernelGGL((gemv_rows<MODE, 8>), grid, block, lds, st, a); break;
+    case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2, NREP>), grid, block, lds, st, a); break;
+    case 4: hipLaunchKernelGGL((gemv_rows<MODE, 4, NREP>), grid, block, lds, st, a); break;
+    default: hipLaunchKernelGGL((gemv_rows<MODE, 8, NREP>), grid, block, lds, st, a); break;
     }
     if (a.splits > 1) {
         const dim3 g2((unsigned)((a.N + 255) / 256), (unsigned)samples, (unsigned)a.M);
         hipLaunchKernelGGL(reduce_splits, g2, dim3(256), 0, st, a);
     }
+}
+
+template <int MODE>
+static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    if (heads_per_block(a.heads_per_kv) == 4)
+        launch_rows_n<MODE, 4>(a, samples, st);
+    else
+        launch_rows_n<MODE, 1>(a, samples, st);
 }
 
 #ifndef KVMIX_COLS_RQ
@@ -753,8 +905,12 @@ using namespace kvmix;
 extern "C" size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t K, int64_t N)
 {
     if (samples <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
-    const RowsPlan p = plan_rows(samples * M, K, N);
-    return p.splits > 1 ? (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float) : 0;
+    // the split count depends on how many query heads share a block (1 or 4, which this query
+    // does not know): size for the larger of the two plans
+    const RowsPlan p1 = plan_rows(samples * M, K, N, kRowsMaxWaves);
+    const RowsPlan p4 = plan_rows((samples + 3) / 4 * M, K, N, kRowsHeadsWaves);
+    const int splits = p1.splits > p4.splits ? p1.splits : p4.splits;
+    return splits > 1 ? (size_t)(samples * M) * (size_t)splits * (size_t)N * sizeof(float) : 0;
 }
 
 extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride,
@@ -835,7 +991,8 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     }
 
     if (use_rows) {
-        const RowsPlan p = plan_rows(samples * M, K, N);
+        const int nrep = heads_per_block(heads_per_kv);
+        const RowsPlan p = plan_rows(samples / nrep * M, K, N, nrep > 1 ? kRowsHeadsWaves : kRowsMaxWaves);
         if (p.splits > 1) {
             const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
             if (!workspace || workspace_bytes < need) return KVMIX_ERR_WORKSPACE;
