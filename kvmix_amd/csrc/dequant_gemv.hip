@@ -292,7 +292,7 @@ __device__ __forceinline__ void wave_lds_fence()
 //                with four 128-bit loads per array per lane; inside a chunk a lane walks
 //                KC/RQ = 32/UPL rows of its section, 8 rows of packed codes in flight.
 //   Rows past K (last chunk only) are read from row K-1 and meet x == 0.
-//   block = (64, 4) waves on neighbouring tiles; grid = (tiles/4, samples, M), XCD-swizzled.
+//   block = (64, 2..4) waves on neighbouring tiles; grid = (tiles/waves, samples, M), XCD-swizzled.
 // Offsets inside one (batch, kv-head) slice are 32-bit (the host checks the extents).
 // ---------------------------------------------------------------------------------------
 constexpr int kColsWaves = 4;
@@ -325,7 +325,7 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int K = (int)a.K;
     const int nunits = (int)(a.N / VALS);
-    int t0 = (int)(bx * kColsWaves + wy) * TU;  // first unit of this wave's tile
+    int t0 = (int)(bx * blockDim.y + wy) * TU;  // first unit of this wave's tile
     if (t0 >= nunits) return;                   // whole wave outside (no block barrier below)
     t0 = t0 + TU <= nunits ? t0 : nunits - TU;  // last tile: shifted left, still whole
     const int unit0 = t0 + gl * UPL;            // this lane's first unit
@@ -848,8 +848,19 @@ static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / VALS;
     const int64_t tiles = (units + TU - 1) / TU;
-    const dim3 grid((unsigned)((tiles + kColsWaves - 1) / kColsWaves), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, kColsWaves), 0, st, a);
+    // waves per block: the count (2..4) that leaves the fewest waves without a tile
+    int wpb = kColsWaves;
+    int64_t idle = (tiles + wpb - 1) / wpb * wpb - tiles;
+    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
+        const int64_t i = (tiles + w - 1) / w * w - tiles;
+        if (i < idle) {
+            idle = i;
+            wpb = w;
+        }
+    }
+    if (tiles < wpb) wpb = (int)tiles;
+    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
+    hipLaunchKernelGGL((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, wpb), 0, st, a);
 }
 
 // smallest tile (in units) any gemv_cols configuration of this mode needs
