@@ -33,6 +33,26 @@
 
 #include "kvmix_common.h"
 
+#ifndef KVMIX_ROWS_MFMA
+#define KVMIX_ROWS_MFMA 1  // 4-bit p.V on the matrix cores
+#endif
+
+#ifndef KVMIX_HEADS_WAVE_DIV
+#define KVMIX_HEADS_WAVE_DIV 2
+#endif
+#ifndef KVMIX_MFMA_HEADS_OCC
+#define KVMIX_MFMA_HEADS_OCC 2
+#endif
+#ifndef KVMIX_MFMA_DEPTH4
+#define KVMIX_MFMA_DEPTH4 1
+#endif
+#ifndef KVMIX_MFMA_DEPTH2
+#define KVMIX_MFMA_DEPTH2 1
+#endif
+#ifndef KVMIX_MFMA_DEPTH1
+#define KVMIX_MFMA_DEPTH1 1
+#endif
+
 #ifndef KVMIX_TARGET_WAVES
 #define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
 #endif
@@ -704,6 +724,296 @@ __global__ void __launch_bounds__(NREP > 1 ? 64 * kRowsHeadsWaves : 64 * kRowsMa
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// gemv_rows_mfma<BITS, NREP>   p.V shape, 1/2/4-bit codes, N = 128: the multiply-accumulate
+// runs on the matrix cores, the vector ALU only isolates the code fields.
+//
+// Instruction: v_mfma_f32_4x4x4 (bf16, 16 independent 4x4x4 blocks per wave).  Block b is
+// lanes 4b..4b+3; per block  D[i][j] += sum_k A[i][k] * B[k][j]  with lane 4b+j supplying
+// column j of B (four k values, two registers), lane 4b+i supplying row i of A, and lane
+// 4b+j receiving column j of D (four registers, i = 0..3).
+//
+// Mapping: a lane owns 8 consecutive codes of a row (BITS bytes: one dword, ushort or byte
+// load), 16 lanes cover a row, so one load instruction reads 4 cache rows (contiguous).
+// The four lanes of a block hold the 32 codes of ONE quantization group of one row, so they
+// share x*scale: that is the A operand.
+//   k   <-> the 4 rows a lane holds after four loads (rows rs, rs+4, rs+8, rs+12 of a
+//           16-row k-block, rs = lane/16);
+//   B   <-> codes: v_perm_b32 puts byte b of two rows' elements into the low bytes of the two
+//           halves of a register and one v_and_b32 isolates a field of both.  An 8-bit
+//           pattern p in the low byte of a bf16 IS the number p * 2^-133 (subnormals and the
+//           first binade share one ulp), so the masked register is a bf16 pair with no
+//           shift and no conversion; a field at bit offset o simply counts 2^o-fold.
+//   A   <-> x*scale*2^90 split into three bf16 (8 significant bits each: the product of two
+//           fp16 has at most 22, so the split is exact).  2^90 keeps every product far above
+//           the fp32 subnormals and below overflow for any fp16 x and scale.  The 3*NREP
+//           (head, part) rows are packed four to an MFMA; unused rows are zero.
+//   D   <-> lane l accumulates, for each of its 8 code positions p, partial sums of output
+//           column 8*(l%16)+p over its rows, one per A row; the parts are added at the end.
+// NREP query heads of one kv head reuse the B registers.
+// x*scale is formed once per (row, group) by the lane that loaded that scale (as in
+// gemv_rows) and parked, already split, in the wave's LDS tile in A-operand order.
+// block = (64, KW); grid = (splits, samples/NREP, M); dynamic LDS = KW * NM A tiles,
+// NM = ceil(3*NREP/4).
+// ---------------------------------------------------------------------------------------
+typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int BITS>
+struct CodeElem;
+template <>
+struct CodeElem<4> {
+    using type = uint32_t;
+};
+template <>
+struct CodeElem<2> {
+    using type = uint16_t;
+};
+template <>
+struct CodeElem<1> {
+    using type = uint8_t;
+};
+
+constexpr int rows_mfma_sets(int nrep) { return (3 * nrep + 3) / 4; }
+constexpr int kRowsMfmaTile = (32 * 17 + 1) * 4 + 4;  // bf16 elements of one A tile (32 skewed rows), 8-byte multiple
+
+constexpr int kRowsMfmaWaves = 16;  // waves per block at most (register budget of 128 per lane)
+
+template <int BITS, int NREP, int DEPTH>
+__global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWaves))
+    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_MFMA_HEADS_OCC : 4))) gemv_rows_mfma(GemvArgs a)
+{
+    using Elem = typename CodeElem<BITS>::type;
+    constexpr int LPR = 4;             // groups per row (N = 128)
+    constexpr int EPR = 16;            // lanes (8-code elements) per row
+    constexpr int RL = kWave / EPR;    // rows per load instruction (4)
+    constexpr int RKB = 4 * RL;        // rows per k-block (16)
+    constexpr int CH = 128;            // rows per chunk: 512 scales = one 128-bit load per lane
+    constexpr int KB = CH / RKB;       // k-blocks per chunk (8)
+    constexpr int AT = kRowsMfmaTile;  // bf16 elements of one A tile
+    constexpr int NM = rows_mfma_sets(NREP);  // MFMAs per B operand
+    constexpr int NPOS = 8;            // code positions per lane
+    constexpr int FPB = 8 / BITS;      // fields per byte
+
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x;
+    const int wy = threadIdx.y;
+    const int KW = blockDim.y;
+    uint16_t *atile = reinterpret_cast<uint16_t *>(lds) + wy * (NM * AT);
+    float *red = lds;  // [KW][NREP][128], reuses the A tiles after the streaming loop
+    const int rs = lane / EPR;
+    const int wi = lane % EPR;
+    int64_t split, hg;
+    xcd_swizzled_block(split, hg, a.heads_per_kv > NREP);
+    const int64_t sample0 = hg * NREP;
+    const int64_t m = blockIdx.z;
+    const int64_t kv = sample0 / a.heads_per_kv;
+    const int64_t kbeg = split * a.rows_per_split;
+    const int64_t kend = kbeg + a.rows_per_split < a.K ? kbeg + a.rows_per_split : a.K;
+
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
+    const Elem *cp = reinterpret_cast<const Elem *>(a.code + kv * a.c_bs) + wi;
+    const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
+    const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
+
+    f32x4_t acc[NM][NPOS];
+    float zacc[NREP][LPR];
+#pragma unroll
+    for (int q = 0; q < NM; q++) {
+#pragma unroll
+        for (int p = 0; p < NPOS; p++) acc[q][p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int h = 0; h < NREP; h++) {
+#pragma unroll
+        for (int g = 0; g < LPR; g++) zacc[h][g] = 0.f;
+    }
+    // some A rows are never written: clear the tiles once
+    for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+
+    // staging: this lane owns elements [8*lane, 8*lane+8) of the chunk's [128][4] scale array,
+    // i.e. rows 2*lane and 2*lane+1, all four groups.  Row r of a chunk is k-slot (r%16)/4 of
+    // A-lanes  (r%4)*16 + 4*g + i  in k-block r/16.
+    // A tile: one 8-byte cell (4 k-slots) per (k-block t, lane); the 16 cells of the lanes with
+    // the same (t, lane/16) form a row of 17 cells' pitch, and the rows of k-blocks 4..7 are
+    // shifted by one more cell.  With that skew the 2-byte staging stores of a wave (same
+    // cell column, 32 different rows) fall into 32 different LDS banks, and a wave's 8-byte
+    // operand reads stay conflict-free.
+    auto cell = [](int t, int l) { return ((4 * t + l / EPR) * 17 + (l % EPR)) * 4 + (t >> 2) * 4; };
+    const int row0 = 2 * lane;
+    int aoff[2];  // bf16 index of (row0 + e, g = 0, i = 0)
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const int r = row0 + e;
+        aoff[e] = cell(r / RKB, (r % RL) * EPR) + (r % RKB) / RL;
+    }
+
+    // Chunks: CH rows each, handed round-robin to the block's waves.  A chunk that would cross
+    // the end of the range is moved back to end exactly there (the host gives this kernel only
+    // K >= CH): every address is then base + constant with no clamping, no load sits behind
+    // a condition (which would make the compiler drain the load queue), and the rows such a
+    // chunk repeats meet x == 0.  A chunk wholly past the end is all zeros.
+    // The wave index is made scalar so that the loop is uniform control flow.
+    const int ke32 = (int)kend;
+    const int stride = KW * CH;
+    const int kfirst = (int)kbeg + __builtin_amdgcn_readfirstlane(wy) * CH;
+    struct __attribute__((packed, aligned(2))) Half2x {
+        uint16_t v[2];
+    };
+    // DEPTH chunks are in flight per wave: register set d holds chunk c with c % DEPTH == d
+    Half8 s8[DEPTH], z8[DEPTH];
+    Half2x xh[DEPTH][NREP];
+    Elem w[DEPTH][KB][4];
+
+    auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : ke32 - CH; };
+    auto load_small = [&](int d, int k0) {
+        const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
+        s8[d] = *reinterpret_cast<const Half8 *>(sp + kr * LPR);
+        z8[d] = *reinterpret_cast<const Half8 *>(zp + kr * LPR);
+#pragma unroll
+        for (int h = 0; h < NREP; h++) xh[d][h] = *reinterpret_cast<const Half2x *>(xp + h * a.x_bs + kr);
+    };
+    auto load_codes = [&](int d, int k0, int t) {
+        const Elem *base = cp + (uint32_t)(chunk_base(k0) + rs) * EPR;
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[d][t][k] = base[(t * RKB + RL * k) * EPR];
+    };
+    auto stage = [&](int d, int k0) {
+        const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int q = e / LPR, g = e % LPR;
+                const float xv = row0 + q >= skip ? h16_to_f32(xh[d][h].v[q]) : 0.f;
+                zacc[h][g] = fmaf(xv, h16_to_f32(z8[d].v[e]), zacc[h][g]);
+                // x * scale * 2^90, split into three bf16 by truncation (exact)
+                const float v0 = (xv * 1237940039285380274899124224.0f) * h16_to_f32(s8[d].v[e]);
+                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+                const float v1 = v0 - __uint_as_float(b0);
+                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+                const float v2 = v1 - __uint_as_float(b1);
+                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+                for (int pt = 0; pt < 3; pt++) {  // A row 3h+pt: MFMA (3h+pt)/4, lanes 4g + (3h+pt)%4
+                    const int ar = 3 * h + pt;
+                    atile[(ar / 4) * AT + aoff[q] + g * 16 + (ar % 4) * 4] = (uint16_t)(part[pt] >> 16);
+                }
+            }
+        }
+    };
+    auto compute = [&](int d, int t) {
+        bf16x4_t av[NM];
+#pragma unroll
+        for (int q = 0; q < NM; q++)
+            av[q] = *reinterpret_cast<const bf16x4_t *>(atile + q * AT + cell(t, lane));
+#pragma unroll
+        for (int b = 0; b < BITS; b++) {
+            // byte b of rows k and k+1 -> low bytes of the two halves
+            const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+            const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
+            const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+#pragma unroll
+            for (int f = 0; f < FPB; f++) {
+                const uint32_t mask = (((1u << BITS) - 1u) * 0x00010001u) << (BITS * f);
+                const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+#pragma unroll
+                for (int q = 0; q < NM; q++)
+                    acc[q][b * FPB + f] =
+                        __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[q], bv, acc[q][b * FPB + f], 0, 0, 0);
+            }
+        }
+    };
+
+    wave_lds_fence();
+    if (kfirst < ke32) {
+        // (the first loads are issued in the loop's own order, each pinned in place: the wait
+        // counts at the loop head must hold for the entry path too)
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            load_small(d, kfirst + d * stride);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < KB; t++) {
+                load_codes(d, kfirst + d * stride, t);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll 1
+        for (int k0 = kfirst; k0 < ke32; k0 += DEPTH * stride) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; d++) {
+                const int kc = k0 + d * stride, kn = kc + DEPTH * stride;
+                stage(d, kc);
+                wave_lds_fence();
+                load_small(d, kn);
+                // a k-block's registers are refilled right after use.  The scheduling barriers
+                // pin the loads where they are written: left alone, the scheduler sinks them to
+                // the end of the iteration and the next one starts by draining the queue.
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < KB; t++) {
+                    compute(d, t);
+                    load_codes(d, kn, t);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                wave_lds_fence();  // the next chunk overwrites the tile
+            }
+        }
+    }
+
+    // ---- reduce ---------------------------------------------------------------------------
+    // zero term: zacc[h][g] summed over all lanes; a lane needs the sum of its own group
+    float zterm[NREP];
+#pragma unroll
+    for (int h = 0; h < NREP; h++) {
+        float z[LPR];
+#pragma unroll
+        for (int g = 0; g < LPR; g++) z[g] = zacc[h][g];
+        scatter_reduce<LPR, 8, 0>(z, lane);  // lane bits 3, 2 = group of the lane's codes
+        z[0] += __shfl_xor(z[0], 1);
+        z[0] += __shfl_xor(z[0], 2);
+        z[0] += __shfl_xor(z[0], 16);
+        z[0] += __shfl_xor(z[0], 32);
+        zterm[h] = z[0];
+    }
+    // code sums: the three parts meet; the 2^-133 of the bf16 patterns, the 2^90 and the
+    // field's bit offset are undone; then the 4 row slots (lane bits 4, 5) are summed
+    constexpr int NV = NREP * NPOS;
+    float flat[NV];
+#pragma unroll
+    for (int h = 0; h < NREP; h++) {
+#pragma unroll
+        for (int p = 0; p < NPOS; p++) {
+            const float sum = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
+                              acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
+            flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23);
+        }
+    }
+    __syncthreads();  // every wave is done with its A tile: the space becomes `red`
+    constexpr int KEEP = NV / 4;
+    const int first = scatter_reduce<NV, 16, 1>(flat, lane);
+#pragma unroll
+    for (int i = 0; i < KEEP; i++) {
+        const int f = first + i;
+        const int h = f / NPOS;
+        float zt = zterm[0];
+#pragma unroll
+        for (int hh = 1; hh < NREP; hh++) zt = h == hh ? zterm[hh] : zt;
+        red[(wy * NREP + h) * 128 + wi * NPOS + f % NPOS] = flat[i] + zt;
+    }
+    __syncthreads();
+    for (int t = wy * kWave + lane; t < NREP * 128; t += KW * kWave) {
+        const int h = t / 128, n = t % 128;
+        float v = 0.f;
+        for (int ww = 0; ww < KW; ww++) v += red[(ww * NREP + h) * 128 + n];
+        if (a.splits == 1)
+            a.out[(sample0 + h) * a.o_bs + m * a.o_rs + n] = __float2half_rn(v);
+        else
+            a.partial[(((sample0 + h) * a.M + m) * a.splits + split) * a.N + n] = v;
+    }
+}
+
 __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
 {
     const int64_t sample = blockIdx.y;
@@ -777,13 +1087,16 @@ struct RowsPlan {
 };
 
 // How gemv_rows covers K for `batch_rows` = samples*M independent outputs.
+// (blocks of at most four waves are the multi-head kernels, which hold two waves per SIMD:
+// they get half as many waves, again one resident round)
 static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_waves)
 {
+    const int64_t target = max_waves <= kRowsHeadsWaves ? kTargetWaves / KVMIX_HEADS_WAVE_DIV : kTargetWaves;
     RowsPlan p{4, 1, K > 0 ? K : 1};
     if (!rows_shape_ok(N) || batch_rows <= 0 || K <= 0) return p;
     const int64_t chunk = 512 / (N / 32);            // rows one wave takes per step
     const int64_t chunks = (K + chunk - 1) / chunk;  // units of parallelism along K
-    int64_t want = (kTargetWaves + batch_rows - 1) / batch_rows;  // waves wanted per output row
+    int64_t want = (target + batch_rows - 1) / batch_rows;  // waves wanted per output row
     if (want > chunks) want = chunks;
     if (want < 1) want = 1;
     int64_t waves = want < max_waves ? want : max_waves;
@@ -802,14 +1115,50 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
 // query heads one block of gemv_rows / gemv_cols serves from a single pass over the packed data
 static int heads_per_block(int heads_per_kv) { return heads_per_kv % 4 == 0 ? 4 : 1; }
 
+// which p.V kernel a problem gets, and the most waves one of its blocks may have
+// (gemv_rows_mfma: N = 128, dense code rows, at least one whole 128-row chunk)
+static bool rows_use_mfma(int mode, int64_t N, int64_t K, int64_t c_rs)
+{
+    return KVMIX_ROWS_MFMA && (mode == 1 || mode == 2 || mode == 4) && N == 128 && K >= 128 &&
+           c_rs == N * mode / 32;
+}
+static int rows_max_waves(bool mfma, int nrep)
+{
+    return nrep > 1 ? kRowsHeadsWaves : (mfma ? kRowsMfmaWaves : kRowsMaxWaves);
+}
+
 template <int MODE, int NREP>
 static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
 {
     // (a block's LDS is waves * NREP * (512 + N) floats)
-    const RowsPlan p = plan_rows(samples / NREP * a.M, a.K, a.N, NREP > 1 ? kRowsHeadsWaves : kRowsMaxWaves);
+    const bool mfma = rows_use_mfma(MODE, a.N, a.K, a.c_rs);
+    const RowsPlan p = plan_rows(samples / NREP * a.M, a.K, a.N, rows_max_waves(mfma, NREP));
     a.splits = p.splits;
     a.rows_per_split = p.rows_per_split;
     const dim3 grid((unsigned)a.splits, (unsigned)(samples / NREP), (unsigned)a.M), block(kWave, p.waves);
+    if constexpr (MODE == 1 || MODE == 2 || MODE == 4) {
+      if (mfma) {
+        // one A tile per wave and MFMA set; the block reduction (waves*NREP*128 floats) reuses it
+        const size_t lds = (size_t)p.waves * rows_mfma_sets(NREP) * kRowsMfmaTile * sizeof(uint16_t);
+        constexpr int DEPTH = NREP == 1 ? (MODE == 4 ? KVMIX_MFMA_DEPTH4 : (MODE == 2 ? KVMIX_MFMA_DEPTH2 : KVMIX_MFMA_DEPTH1)) : 1;
+        if (lds > 64 * 1024) {
+            // above the default per-block limit: raise it for this kernel, once per device
+            static bool raised[64] = {};
+            int dev = 0;
+            if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !raised[dev]) {
+                (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_rows_mfma<MODE, NREP, DEPTH>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                raised[dev] = true;
+            }
+        }
+        hipLaunchKernelGGL((gemv_rows_mfma<MODE, NREP, DEPTH>), grid, block, lds, st, a);
+        if (a.splits > 1) {
+            const dim3 g2((unsigned)((a.N + 255) / 256), (unsigned)samples, (unsigned)a.M);
+            hipLaunchKernelGGL(reduce_splits, g2, dim3(256), 0, st, a);
+        }
+        return;
+      }
+    }
     const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)NREP * (size_t)(512 + a.N);
     switch (a.N / 32) {
     case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2, NREP>), grid, block, lds, st, a); break;
@@ -916,11 +1265,13 @@ using namespace kvmix;
 extern "C" size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t K, int64_t N)
 {
     if (samples <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
-    // the split count depends on how many query heads share a block (1 or 4, which this query
-    // does not know): size for the larger of the two plans
+    // the split count depends on the kernel and on how many query heads share a block (which
+    // this query does not know): size for the largest of the possible plans
     const RowsPlan p1 = plan_rows(samples * M, K, N, kRowsMaxWaves);
+    const RowsPlan p8 = plan_rows(samples * M, K, N, kRowsMfmaWaves);
     const RowsPlan p4 = plan_rows((samples + 3) / 4 * M, K, N, kRowsHeadsWaves);
-    const int splits = p1.splits > p4.splits ? p1.splits : p4.splits;
+    int splits = p1.splits > p4.splits ? p1.splits : p4.splits;
+    splits = p8.splits > splits ? p8.splits : splits;
     return splits > 1 ? (size_t)(samples * M) * (size_t)splits * (size_t)N * sizeof(float) : 0;
 }
 
@@ -1003,7 +1354,8 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
 
     if (use_rows) {
         const int nrep = heads_per_block(heads_per_kv);
-        const RowsPlan p = plan_rows(samples / nrep * M, K, N, nrep > 1 ? kRowsHeadsWaves : kRowsMaxWaves);
+        const RowsPlan p = plan_rows(samples / nrep * M, K, N,
+                                     rows_max_waves(rows_use_mfma(mode, N, K, code_row_stride), nrep));
         if (p.splits > 1) {
             const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
             if (!workspace || workspace_bytes < need) return KVMIX_ERR_WORKSPACE;
