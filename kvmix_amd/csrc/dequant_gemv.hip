@@ -510,6 +510,147 @@ __device__ __forceinline__ int scatter_reduce(float *v, int lane)
 }
 
 // ---------------------------------------------------------------------------------------
+// gemv_cols3<RQ>   q.K^T shape for the reference's 3-bit format (11 codes per word, one
+// (scale, zero) pair per word, so half of the bytes are scales and zeros).
+//   A lane owns 4 consecutive words of N for one of RQ sections of the K rows: per row it
+//   loads 16 bytes of codes, 8 of scales and 8 of zeros straight into registers -- no LDS
+//   staging, no barriers in the stream.  U rows are in flight per lane: a row's registers
+//   are refilled with row k+U right after row k is consumed, every load unconditional
+//   (rows past the section are redirected to the last row and meet x == 0) and pinned in
+//   place with scheduling barriers, so the load queue never drains.
+//   x is converted once per block into LDS (fp32, with a zero in slot K for the redirected
+//   rows).  Tiles as in gemv_cols: TU = (64/RQ)*4 words per wave, last tile shifted left.
+//   block = (64, 2..4); grid = (tiles/waves, samples, M), XCD-swizzled; dynamic LDS = (K+1)*4.
+// ---------------------------------------------------------------------------------------
+template <int RQ, int UPL, int U>
+__global__ void __launch_bounds__(64 * kColsWaves) gemv_cols3(GemvArgs a)
+{
+    constexpr int VALS = 11;
+    constexpr int GL = kWave / RQ;
+    constexpr int TU = GL * UPL;
+    extern __shared__ float xs[];  // [K + 1]
+
+    const int lane = threadIdx.x;
+    const int wy = threadIdx.y;
+    const int rq = lane / GL;
+    const int gl = lane % GL;
+    int64_t bx, sample;
+    xcd_swizzled_block(bx, sample, true);
+    const int64_t m = blockIdx.z;
+    const int64_t kv = sample / a.heads_per_kv;
+    const int K = (int)a.K;
+    const int nunits = (int)(a.N / VALS);
+
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
+    for (int i = wy * kWave + lane; i <= K; i += blockDim.y * kWave) xs[i] = i < K ? h16_to_f32(xp[i]) : 0.f;
+    __syncthreads();
+
+    int t0 = (int)(bx * blockDim.y + wy) * TU;
+    if (t0 >= nunits) return;  // (after the only block barrier)
+    t0 = t0 + TU <= nunits ? t0 : nunits - TU;
+    const int unit0 = t0 + gl * UPL;
+    const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
+    const uint32_t *cp = a.code + kv * a.c_bs + unit0;
+    const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs + unit0;
+    const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs + unit0;
+
+    float acc[UPL][VALS];
+    float zsum[UPL];
+#pragma unroll
+    for (int j = 0; j < UPL; j++) {
+        zsum[j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < VALS; i++) acc[j][i] = 0.f;
+    }
+
+    // this lane's rows: [kbeg, kend), walked in steps of U
+    const int kq = (K + RQ - 1) / RQ;
+    const int kbeg = rq * kq;
+    const int kend = kbeg + kq < K ? kbeg + kq : K;
+    const int steps = (kq + U - 1) / U;  // the same for every section: uniform control flow
+
+    struct __attribute__((packed, aligned(2))) HalfN {
+        uint16_t v[UPL];
+    };
+    Words<UPL> cw[U];
+    HalfN sw[U], zw[U];
+    auto load_row = [&](int u, int k) {
+        const uint32_t kc = (uint32_t)(k < kend ? k : K - 1);
+        cw[u] = *reinterpret_cast<const Words<UPL> *>(cp + kc * c_rs);
+        sw[u] = *reinterpret_cast<const HalfN *>(sp + kc * s_rs);
+        zw[u] = *reinterpret_cast<const HalfN *>(zp + kc * s_rs);
+    };
+    auto compute_row = [&](int u, int k) {
+        const float xv = xs[k < kend ? k : K];
+        const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90, see accumulate_unit
+#pragma unroll
+        for (int j = 0; j < UPL; j++) {
+            const half2_t sz = __builtin_bit_cast(half2_t, (uint32_t)sw[u].v[j] | ((uint32_t)zw[u].v[j] << 16));
+            zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
+            float mq[4];
+            mq[0] = x2 * (float)sz.x;
+#pragma unroll
+            for (int t = 1; t < 4; t++) mq[t] = mq[t - 1] * 0.125f;
+            const uint32_t w = cw[u].v[j];
+            const uint32_t v[3] = {w, w >> 12, w >> 24};
+#pragma unroll
+            for (int i = 0; i < VALS; i++) {
+                const uint32_t mask = (i == 10 ? 3u : 7u) << (3 * (i % 4));
+                acc[j][i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & mask), acc[j][i]);
+            }
+        }
+    };
+
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        load_row(u, kbeg + u);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll 1
+    for (int st = 0; st < steps; st++) {
+        const int k0 = kbeg + st * U;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            compute_row(u, k0 + u);
+            load_row(u, k0 + U + u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- combine the RQ row sections, store fp16 ----
+    constexpr int TOT = UPL * VALS;  // consecutive outputs of this lane
+    float *flat = &acc[0][0];
+#pragma unroll
+    for (int j = 0; j < UPL; j++) {
+#pragma unroll
+        for (int i = 0; i < VALS; i++) acc[j][i] = fmaf(acc[j][i], Fmt<3>::OUT_SCALE, zsum[j]);
+    }
+    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
+    if constexpr (RQ == 1) {
+#pragma unroll
+        for (int e = 0; e < TOT; e += 2) {
+            const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
+            __builtin_memcpy(op + e, &pk, 4);
+        }
+    } else {
+        // halving butterfly: each section ends with its share of the sums (TOT / RQ each)
+        static_assert(RQ == 2 && TOT % 2 == 0, "two sections, equal shares");
+        const int first = scatter_reduce<TOT, GL, 1>(flat, lane);
+        constexpr int PER = TOT / RQ;
+        if constexpr (PER % 2 == 0) {
+#pragma unroll
+            for (int e = 0; e < PER; e += 2) {
+                const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
+                __builtin_memcpy(op + first + e, &pk, 4);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < PER; e++) op[first + e] = f32_to_h16(flat[e]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // gemv_rows<MODE, LPR>
 //   LPR = N/32 lanes per row (one 32-code group each), RPW = 64/LPR rows per tile,
 //   chunk = 8 tiles = 512/LPR rows: its scale array is 512 halves = one 128-bit load per lane.
@@ -1216,14 +1357,53 @@ static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
 template <int MODE>
 static int64_t cols_min_units()
 {
-    // (the reference 3-bit format is not instantiated with four row sections: with four
-    // units per lane that configuration needs more registers than a wave may have)
-    return (MODE == 3 ? 32 : 16) * ColsUpl<MODE>::value;
+    // (reference 3-bit format: gemv_cols3 with two words per lane and two row sections)
+    return MODE == 3 ? 64 : 16 * ColsUpl<MODE>::value;
+}
+
+#ifndef KVMIX_COLS3_MIN_WAVES
+#define KVMIX_COLS3_MIN_WAVES 2048
+#endif
+#ifndef KVMIX_COLS3_U
+#define KVMIX_COLS3_U 8
+#endif
+
+template <int RQ, int UPL>
+static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    constexpr int TU = (kWave / RQ) * UPL;
+    const int64_t units = a.N / 11;
+    const int64_t tiles = (units + TU - 1) / TU;
+    int wpb = kColsWaves;  // waves per block: the count (2..4) that leaves the fewest waves idle
+    int64_t idle = (tiles + wpb - 1) / wpb * wpb - tiles;
+    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
+        const int64_t i = (tiles + w - 1) / w * w - tiles;
+        if (i < idle) {
+            idle = i;
+            wpb = w;
+        }
+    }
+    if (tiles < wpb) wpb = (int)tiles;
+    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
+    hipLaunchKernelGGL((gemv_cols3<RQ, UPL, KVMIX_COLS3_U>), grid, dim3(kWave, wpb),
+                       sizeof(float) * (size_t)(a.K + 1), st, a);
 }
 
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
+    if constexpr (MODE == 3) {
+        // reference 3-bit format: register-streaming kernel; the widest tile (256, 128 or 64
+        // words per wave) that still gives the chip enough waves and fits into N
+        const int64_t units = a.N / 11, batch = samples * a.M;
+        auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
+        if (units >= 256 && waves(256) >= kTargetWaves)
+            launch_cols3_cfg<1, 4>(a, samples, st);
+        else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
+            launch_cols3_cfg<2, 4>(a, samples, st);
+        else
+            launch_cols3_cfg<2, 2>(a, samples, st);
+    } else {
     // more row sections per wave = more, narrower waves: take the widest tile that still
     // gives the chip enough waves and fits into N
     constexpr int VALS = Fmt<MODE>::VALS;
@@ -1240,13 +1420,13 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
             rq = 4;
     }
     while (rq < 4 && units < (64 / rq) * UPL) rq *= 2;  // the tile must fit into N
-    if constexpr (MODE == 3) rq = rq > 2 ? 2 : rq;
-    if (rq == 4) {
-        if constexpr (MODE != 3) launch_cols_cfg<MODE, 4, UPL>(a, samples, st);
-    } else if (rq == 2)
+    if (rq == 4)
+        launch_cols_cfg<MODE, 4, UPL>(a, samples, st);
+    else if (rq == 2)
         launch_cols_cfg<MODE, 2, UPL>(a, samples, st);
     else
         launch_cols_cfg<MODE, 1, UPL>(a, samples, st);
+    }
 }
 
 template <int MODE>
@@ -1339,7 +1519,8 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     const bool rows_ok = fast_group && !ref3 && rows_shape_ok(N) && sz_row_stride == N / 32 && K >= 8;
     // gemv_cols needs one whole wave tile of group units along N
     const int64_t min_units = mode == 3 ? cols_min_units<3>() : cols_min_units<4>();
-    const bool cols_ok = fast_group && K > 0 && N / (ref3 ? 11 : 32) >= min_units;
+    // (gemv_cols3 keeps x for all K rows in LDS)
+    const bool cols_ok = fast_group && K > 0 && N / (ref3 ? 11 : 32) >= min_units && (!ref3 || K <= 8192);
     // p.V shape: few columns, many rows.  q.K^T shape: the opposite.
     const bool use_rows = rows_ok && (K >= 2 * N || !cols_ok);
 
