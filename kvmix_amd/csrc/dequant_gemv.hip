@@ -33,6 +33,9 @@
 
 #include "kvmix_common.h"
 
+#ifndef KVMIX_COLS_MFMA
+#define KVMIX_COLS_MFMA 1  // 1/2/4-bit q.K^T on the matrix cores
+#endif
 #ifndef KVMIX_ROWS_MFMA
 #define KVMIX_ROWS_MFMA 1  // 4-bit p.V on the matrix cores
 #endif
@@ -1155,6 +1158,223 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// gemv_cols_mfma<BITS, NREP>   q.K^T shape, 1/2/4-bit codes: the matrix-core scheme of
+// gemv_rows_mfma turned by 90 degrees.
+//   A lane owns 8 consecutive codes (BITS bytes) of N in every row; a wave's tile is 512
+//   codes = 16 quantization groups, the four lanes of an MFMA block are one group.  One load
+//   instruction reads 64*BITS contiguous bytes of one row; the k-slots of an MFMA are four
+//   consecutive rows.  All K rows are reduced inside the lane's accumulators, so nothing is
+//   exchanged between lanes or waves except the zero term, and a lane stores its 8 outputs
+//   with one 16-byte store.
+//   Rows are walked in chunks of 32 (8 MFMA k-steps): the chunk's [32][16] scales and zeros
+//   are one 128-bit load per lane each; the lane that loads a scale forms x*scale*2^90, splits
+//   it into three bf16 and parks them in the wave's LDS tile in A-operand order (rows of 32
+//   eight-byte cells at a pitch of 33: staging stores and operand reads are bank-conflict
+//   free).  A chunk that would cross K is moved back to end at K and its repeated rows meet
+//   x == 0 (the host gives this kernel K >= 32).  Loads rotate as in gemv_rows_mfma.
+//   The last tile of a row is shifted left to end at N (N >= 512, a multiple of 32).
+//   A wave walks `splits` tiles one after the other with the load pipeline running across
+//   them.  block = (64, 2..4) waves on neighbouring tiles; grid = (tiles/(waves*splits),
+//   samples/NREP, M), XCD-swizzled; dynamic LDS = waves * (NM tiles of kColsMfmaTile bf16 +
+//   NREP*16 floats).
+// ---------------------------------------------------------------------------------------
+constexpr int kColsMfmaTile = 16 * 33 * 4;  // bf16 elements: 16 rows of 33 four-element cells
+
+template <int BITS, int NREP>
+__global__ void __launch_bounds__(64 * kColsWaves)
+    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_MFMA_HEADS_OCC : 4))) gemv_cols_mfma(GemvArgs a)
+{
+    using Elem = typename CodeElem<BITS>::type;
+    constexpr int CH = 32;             // rows per chunk
+    constexpr int KB = CH / 4;         // MFMA k-steps per chunk
+    constexpr int AT = kColsMfmaTile;
+    constexpr int NM = rows_mfma_sets(NREP);
+    constexpr int NPOS = 8;
+    constexpr int FPB = 8 / BITS;
+    constexpr int TG = 16;             // groups per tile
+
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x;
+    const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int nw = (int)blockDim.y;
+    uint16_t *atile = reinterpret_cast<uint16_t *>(lds) + wy * (NM * AT + NREP * TG * 2);
+    float *zl = reinterpret_cast<float *>(atile + NM * AT);  // [NREP][16] zero terms of a tile
+    int64_t bx, hg;
+    xcd_swizzled_block(bx, hg, true);
+    const int64_t sample0 = hg * NREP;
+    const int64_t m = blockIdx.z;
+    const int64_t kv = sample0 / a.heads_per_kv;
+    const int K = (int)a.K;
+    const int ngroups = (int)(a.N / 32);
+    // a.splits tiles per wave: tiles (bx*splits + j)*nw + wy, j = 0..splits-1 -- the block's
+    // waves sit on neighbouring tiles at any time.  A tile past N is redirected to the last
+    // one (recomputed, stored twice with identical values): uniform control flow, no branches.
+    const int tpw = a.splits;
+    const int tile0 = (int)bx * tpw * nw + wy;
+    if (tile0 * TG >= ngroups) return;  // (no block barrier below)
+    const int nch = (K + CH - 1) / CH;
+    const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
+
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
+    const Elem *cbase = reinterpret_cast<const Elem *>(a.code + kv * a.c_bs) + lane;
+    const uint32_t c_re = (uint32_t)a.c_rs * (4 / BITS);  // row stride in elements
+    const uint32_t s_rs = (uint32_t)a.s_rs;
+    const int par = lane % 2;   // staging: row lane/2 of the chunk, groups 8*par .. 8*par+7
+    const int srow = lane / 2;
+    const uint16_t *sbase = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs + 8 * par;
+    const uint16_t *zbase = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs + 8 * par;
+
+    f32x4_t acc[NM][NPOS];
+    float zacc[NREP][8];
+    auto clear = [&]() {
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) acc[q][p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) zacc[h][j] = 0.f;
+        }
+    };
+    clear();
+    for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+
+    // cell of (k-step t, operand lane l): four bf16 k-slots
+    auto cell = [](int t, int l) { return ((2 * t + l / 32) * 33 + l % 32) * 4; };
+    // staged row srow is k-slot srow%4 of k-step srow/4; its group 8*par+j feeds lanes 4*(8*par+j)+i
+    const int aoff = cell(srow / 4, 32 * par) + srow % 4;
+
+    Half8 s8, z8;
+    uint16_t xh[NREP];
+    Elem w[KB][4];
+
+    // item -> first group of its tile, first row of its chunk (moved back to end at K)
+    auto tile_g0 = [&](int it) {
+        const int g = (tile0 + (it / nch) * nw) * TG;
+        return g + TG <= ngroups ? g : ngroups - TG;
+    };
+    auto chunk_k0 = [&](int it) { return (it % nch) * CH; };
+    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
+    auto load_small = [&](int it) {
+        const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
+        const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
+        s8 = *reinterpret_cast<const Half8 *>(sbase + off);
+        z8 = *reinterpret_cast<const Half8 *>(zbase + off);
+#pragma unroll
+        for (int h = 0; h < NREP; h++) xh[h] = xp[h * a.x_bs + d];
+    };
+    auto load_codes = [&](int it, int t) {
+        const Elem *base = cbase + ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_re + (uint32_t)tile_g0(it) * 4);
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[t][k] = base[(uint32_t)k * c_re];
+    };
+    auto stage = [&](int it) {
+        const int k0 = chunk_k0(it);
+        const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+            const float xv = srow >= skip ? h16_to_f32(xh[h]) : 0.f;
+            const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                zacc[h][j] = fmaf(xv, h16_to_f32(z8.v[j]), zacc[h][j]);
+                const float v0 = x2 * h16_to_f32(s8.v[j]);  // split into three bf16 by truncation (exact)
+                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+                const float v1 = v0 - __uint_as_float(b0);
+                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+                const float v2 = v1 - __uint_as_float(b1);
+                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+                for (int pt = 0; pt < 3; pt++) {  // A row 3h+pt: MFMA (3h+pt)/4, lanes 4g + (3h+pt)%4
+                    const int ar = 3 * h + pt;
+                    atile[(ar / 4) * AT + aoff + (4 * j + ar % 4) * 4] = (uint16_t)(part[pt] >> 16);
+                }
+            }
+        }
+    };
+    auto compute = [&](int t) {
+        bf16x4_t av[NM];
+#pragma unroll
+        for (int q = 0; q < NM; q++) av[q] = *reinterpret_cast<const bf16x4_t *>(atile + q * AT + cell(t, lane));
+#pragma unroll
+        for (int b = 0; b < BITS; b++) {
+            const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+            const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[t][1], (uint32_t)w[t][0], sel);
+            const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[t][3], (uint32_t)w[t][2], sel);
+#pragma unroll
+            for (int f = 0; f < FPB; f++) {
+                const uint32_t mask = (((1u << BITS) - 1u) * 0x00010001u) << (BITS * f);
+                const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+#pragma unroll
+                for (int q = 0; q < NM; q++)
+                    acc[q][b * FPB + f] =
+                        __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[q], bv, acc[q][b * FPB + f], 0, 0, 0);
+            }
+        }
+    };
+    struct __attribute__((packed, aligned(2))) Out8 {
+        uint16_t v[8];
+    };
+    // a tile's K rows are done: zero terms through LDS, 8 outputs per lane and head, clear
+    auto finish_tile = [&](int it) {
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+            float z[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) z[j] = zacc[h][j];
+            const int first = scatter_reduce<8, 2, 1>(z, lane);  // lane bits 1..3
+            z[0] += __shfl_xor(z[0], 16);
+            z[0] += __shfl_xor(z[0], 32);
+            zl[h * TG + 8 * par + first] = z[0];  // group 8*par+first (same value from 4 lanes)
+        }
+        wave_lds_fence();
+        const int64_t col = (int64_t)tile_g0(it) * 32 + lane * 8;
+#pragma unroll
+        for (int h = 0; h < NREP; h++) {
+            const float zt = zl[h * TG + lane / 4];
+            Out8 o;
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) {
+                const float sum = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
+                                  acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
+                o.v[p] = f32_to_h16(fmaf(sum, __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
+            }
+            uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + (sample0 + h) * a.o_bs + m * a.o_rs + col;
+            *reinterpret_cast<Out8 *>(op) = o;
+        }
+        wave_lds_fence();
+        clear();
+    };
+
+    wave_lds_fence();
+    load_small(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < KB; t++) {
+        load_codes(0, t);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll 1
+    for (int it = 0; it < items; it++) {
+        const int nx = it + 1 < items ? it + 1 : it;  // (past the end: the same item again)
+        stage(it);
+        wave_lds_fence();
+        load_small(nx);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < KB; t++) {
+            compute(t);
+            load_codes(nx, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wave_lds_fence();  // the next chunk overwrites the tile
+        if (it % nch == nch - 1) finish_tile(it);
+    }
+}
+
 __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
 {
     const int64_t sample = blockIdx.y;
@@ -1389,9 +1609,59 @@ static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
                        sizeof(float) * (size_t)(a.K + 1), st, a);
 }
 
+// (gemv_cols_mfma: whole 512-code tiles, at least one whole 32-row chunk)
+static bool cols_use_mfma(int mode, int64_t N, int64_t K)
+{
+    return KVMIX_COLS_MFMA && (mode == 1 || mode == 2 || mode == 4) && N >= 512 && K >= 32;
+}
+
+template <int BITS, int NREP>
+static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    const int64_t tiles = (a.N / 32 + 15) / 16;
+    const int64_t batch = samples / NREP * a.M;
+    // tiles per wave: as many as still leave one resident round of waves (4 per SIMD, 2 for
+    // the multi-head kernel); a wave that walks several tiles pays its start-up once
+    const int64_t target = NREP > 1 ? kTargetWaves / 2 : kTargetWaves;
+    int64_t tpw = batch * tiles / target;
+    tpw = tpw < 1 ? 1 : (tpw > 8 ? 8 : tpw);
+    const int64_t slots = (tiles + tpw - 1) / tpw;  // waves per output row
+    int wpb = kColsWaves;
+    int64_t idle = (slots + wpb - 1) / wpb * wpb - slots;
+    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
+        const int64_t i = (slots + w - 1) / w * w - slots;
+        if (i < idle) {
+            idle = i;
+            wpb = w;
+        }
+    }
+    if (slots < wpb) wpb = (int)slots;
+    a.splits = (int)tpw;
+    const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
+    const size_t lds = (size_t)wpb * (rows_mfma_sets(NREP) * kColsMfmaTile * sizeof(uint16_t) + NREP * 16 * sizeof(float));
+    hipLaunchKernelGGL((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a);
+}
+
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
+    if constexpr (MODE == 1 || MODE == 2 || MODE == 4) {
+        // Matrix-core kernel: always for GQA (the query heads of a kv head share one pass over
+        // the codes); for one head per kv head only when the problem is small enough that
+        // gemv_cols would have to cut its tiles down to 256-byte row pieces anyway -- measured,
+        // gemv_cols with 512-byte pieces streams faster than either kernel with 256-byte ones.
+        if (cols_use_mfma(MODE, a.N, a.K)) {
+            const int64_t units = a.N / 32, batch = samples * a.M;
+            if (heads_per_block(a.heads_per_kv) == 4) {
+                launch_cols_mfma<MODE, 4>(a, samples, st);
+                return;
+            }
+            if (batch * ((units + 31) / 32) < kTargetWaves) {
+                launch_cols_mfma<MODE, 1>(a, samples, st);
+                return;
+            }
+        }
+    }
     if constexpr (MODE == 3) {
         // reference 3-bit format: register-streaming kernel; the widest tile (256, 128 or 64
         // words per wave) that still gives the chip enough waves and fits into N
