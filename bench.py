@@ -17,6 +17,7 @@ the launch stream.  `cpu_baseline` times the CPU oracle on a bounded sample of t
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -118,17 +119,18 @@ def make_calls(torch, _lib, lib, layers, B, H, D, stream):
         kfmt = _lib.FMT_REF
         vfmt = _lib.FMT_DENSE3 if L.vb == 3 else _lib.FMT_REF
 
-        def fk(L=L):
-            return lib.kvmix_quant_pack_key_tokens(
-                L.ktail.data_ptr(), B * H, L.nk, D, L.ktail.stride(1), L.ktail.stride(2), L.kg, L.kb, kfmt,
-                _lib.SCALE_RECIPROCAL, L.fk_code.data_ptr(), L.fk_code.stride(1), L.fk_code.stride(2),
-                L.fk_s.data_ptr(), L.fk_z.data_ptr(), L.fk_s.stride(1), L.fk_s.stride(2), stream)
+        # both flushes of the layer in one launch (kvmix_quant_pack_kv_flush)
+        L.kflush = _lib.KeyFlush(L.ktail.data_ptr(), B * H, L.nk, D, L.ktail.stride(1), L.ktail.stride(2), L.kg, L.kb,
+                                 kfmt, _lib.SCALE_RECIPROCAL, L.fk_code.data_ptr(), L.fk_code.stride(1),
+                                 L.fk_code.stride(2), L.fk_s.data_ptr(), L.fk_z.data_ptr(), L.fk_s.stride(1),
+                                 L.fk_s.stride(2))
+        L.vflush = _lib.ValueFlush(L.vtail.data_ptr(), B * H, L.nv, D, L.vtail.stride(1), L.vtail.stride(2), 32, L.vb,
+                                   vfmt, _lib.SCALE_RECIPROCAL, L.fv_code.data_ptr(), L.fv_code.stride(1),
+                                   L.fv_code.stride(2), L.fv_s.data_ptr(), L.fv_z.data_ptr(), L.fv_s.stride(1),
+                                   L.fv_s.stride(2))
 
-        def fv(L=L, vfmt=vfmt):
-            return lib.kvmix_quant_pack_last_dim(
-                L.vtail.data_ptr(), _lib.F16, B * H, L.nv, D, L.vtail.stride(1), L.vtail.stride(2), 32, L.vb, vfmt,
-                _lib.SCALE_RECIPROCAL, L.fv_code.data_ptr(), L.fv_code.stride(1), L.fv_code.stride(2),
-                L.fv_s.data_ptr(), L.fv_z.data_ptr(), L.fv_s.stride(1), L.fv_s.stride(2), stream)
+        def fl(L=L):
+            return lib.kvmix_quant_pack_kv_flush(ctypes.byref(L.kflush), ctypes.byref(L.vflush), stream)
 
         def qk(L=L):
             return lib.kvmix_quantized_gemv(
@@ -142,7 +144,7 @@ def make_calls(torch, _lib, lib, layers, B, H, D, stream):
                 L.vz.data_ptr(), L.vs.stride(1), L.vs.stride(2), L.vb, vfmt, B * H, 1, 1, L.Tqv, D,
                 L.out.data_ptr(), D, D, L.ws.data_ptr(), L.wsb, stream)
 
-        calls += [(f"quant_key_tokens[{L.kfmt}]", L.bytes_fk, fk), (f"quant_rows[{L.vfmt}]", L.bytes_fv, fv),
+        calls += [(f"quant_kv_flush[{L.kfmt},{L.vfmt}]", L.bytes_fk + L.bytes_fv, fl),
                   (f"gemv_cols[{L.kfmt}]", L.bytes_qk, qk), (f"gemv_rows[{L.vfmt}]", L.bytes_pv, pv)]
     return calls
 

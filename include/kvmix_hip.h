@@ -109,6 +109,40 @@ int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t n, int64_t
                                 int64_t sz_outer_stride, int64_t sz_inner_stride, kvmix_stream_t stream);
 
 /*
+ * Both flushes of one decode step in a single launch: the key tail through
+ * kvmix_quant_pack_key_tokens and the value tail through kvmix_quant_pack_last_dim
+ * (fp16 input), same arguments, same results bit for bit.  The reference issues the two
+ * quantizers back to back from models/modeling_llama_KVmix.py:119-160; each is a small,
+ * latency-bound launch, so one launch for both costs about what either costs alone.
+ * Both halves are validated before anything is launched.  When a half is empty or the
+ * value half is not the group-32 fp16 case, the call falls back to separate launches.
+ */
+typedef struct kvmix_key_flush {
+    const void *k;              /* [outer, n, D] fp16 */
+    int64_t outer, n, D;
+    int64_t k_outer_stride, k_token_stride;
+    int group, bits, fmt, scale_mode;
+    uint32_t *code;             /* [outer, D, n/vpw] */
+    int64_t code_outer_stride, code_inner_stride;
+    void *scale, *zero;         /* [outer, D, n/group] fp16 */
+    int64_t sz_outer_stride, sz_inner_stride;
+} kvmix_key_flush_t;
+
+typedef struct kvmix_value_flush {
+    const void *x;              /* [outer, inner, steps] fp16 */
+    int64_t outer, inner, steps;
+    int64_t x_outer_stride, x_inner_stride;
+    int group, bits, fmt, scale_mode;
+    uint32_t *code;             /* [outer, inner, steps/vpw] */
+    int64_t code_outer_stride, code_inner_stride;
+    void *scale, *zero;         /* [outer, inner, steps/group] fp16 */
+    int64_t sz_outer_stride, sz_inner_stride;
+} kvmix_value_flush_t;
+
+int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *key, const kvmix_value_flush_t *value,
+                              kvmix_stream_t stream);
+
+/*
  * Fused dequantize + matrix-vector product over the packed cache.
  * Replaces quantized_gemm (quant_cuda/csrc/dequantization_gemv_cuda.h:22-29,
  * dequantization_gemv_cuda.cu:7-248):

@@ -20,11 +20,32 @@ EXPORTS = (
     "kvmix_strerror",
     "kvmix_quant_pack_last_dim",
     "kvmix_quant_pack_key_tokens",
+    "kvmix_quant_pack_kv_flush",
     "kvmix_gemv_workspace_bytes",
     "kvmix_quantized_gemv",
 )
 
 _lib = None
+
+
+class KeyFlush(ctypes.Structure):
+    """kvmix_key_flush_t"""
+    _fields_ = [("k", ctypes.c_void_p), ("outer", ctypes.c_int64), ("n", ctypes.c_int64), ("D", ctypes.c_int64),
+                ("k_outer_stride", ctypes.c_int64), ("k_token_stride", ctypes.c_int64),
+                ("group", ctypes.c_int), ("bits", ctypes.c_int), ("fmt", ctypes.c_int), ("scale_mode", ctypes.c_int),
+                ("code", ctypes.c_void_p), ("code_outer_stride", ctypes.c_int64), ("code_inner_stride", ctypes.c_int64),
+                ("scale", ctypes.c_void_p), ("zero", ctypes.c_void_p),
+                ("sz_outer_stride", ctypes.c_int64), ("sz_inner_stride", ctypes.c_int64)]
+
+
+class ValueFlush(ctypes.Structure):
+    """kvmix_value_flush_t"""
+    _fields_ = [("x", ctypes.c_void_p), ("outer", ctypes.c_int64), ("inner", ctypes.c_int64), ("steps", ctypes.c_int64),
+                ("x_outer_stride", ctypes.c_int64), ("x_inner_stride", ctypes.c_int64),
+                ("group", ctypes.c_int), ("bits", ctypes.c_int), ("fmt", ctypes.c_int), ("scale_mode", ctypes.c_int),
+                ("code", ctypes.c_void_p), ("code_outer_stride", ctypes.c_int64), ("code_inner_stride", ctypes.c_int64),
+                ("scale", ctypes.c_void_p), ("zero", ctypes.c_void_p),
+                ("sz_outer_stride", ctypes.c_int64), ("sz_inner_stride", ctypes.c_int64)]
 
 
 class KVmixLibraryMissing(ImportError):
@@ -51,6 +72,8 @@ def load() -> ctypes.CDLL:
     L.kvmix_quant_pack_key_tokens.restype = i32
     L.kvmix_quant_pack_key_tokens.argtypes = [vp, i64, i64, i64, i64, i64, i32, i32, i32, i32,
                                               vp, i64, i64, vp, vp, i64, i64, vp]
+    L.kvmix_quant_pack_kv_flush.restype = i32
+    L.kvmix_quant_pack_kv_flush.argtypes = [ctypes.POINTER(KeyFlush), ctypes.POINTER(ValueFlush), vp]
     L.kvmix_gemv_workspace_bytes.restype = sz
     L.kvmix_gemv_workspace_bytes.argtypes = [i64, i64, i64, i64]
     L.kvmix_quantized_gemv.restype = i32

@@ -95,23 +95,29 @@ class KVmixAttention:
         self.residual_length = residual_length
 
     # -- flush helpers ---------------------------------------------------------------------
-    def _flush_keys(self, k_tail, code, scale, mn, prompt=False):
-        n = flush_length(k_tail.shape[-2], self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
-        if n > 0:
-            chunk = k_tail[:, :, :n, :]
-            k_tail = k_tail[:, :, n:, :]
-            c, s, m = ops.quantize_pack_last_dim_cuda(chunk.transpose(2, 3).contiguous(), self.Kgroup_size, self.k_bits)
-            code, scale, mn = _cat(code, c, 3), _cat(scale, s, 3), _cat(mn, m, 3)
-        return k_tail, code, scale, mn
-
-    def _flush_values(self, v_tail, code, scale, mn, prompt=False):
-        n = flush_length(v_tail.shape[-2], self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
-        if n > 0:
-            chunk = v_tail[:, :, :n, :]
-            v_tail = v_tail[:, :, n:, :]
-            c, s, m = ops.quantize_pack_last_dim_cuda(chunk.contiguous(), self.Vgroup_size, self.v_bits)
-            code, scale, mn = _cat(code, c, 2), _cat(scale, s, 2), _cat(mn, m, 2)
-        return v_tail, code, scale, mn
+    def _flush(self, k_tail, kq, v_tail, vq, prompt=False):
+        """Quantize the oldest tokens of both tails.  kq / vq = (code, scale, min) so far (or Nones).
+        When both tails flush in the same step the two quantizers run as one launch."""
+        nk = flush_length(k_tail.shape[-2], self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
+        nv = flush_length(v_tail.shape[-2], self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
+        kc = vc = None
+        if nk > 0 and nv > 0 and k_tail.dtype == torch.float16 and v_tail.shape[-1] % self.Vgroup_size == 0:
+            kc, ks, km, vc, vs, vm = ops.quantize_kv_flush(k_tail[:, :, :nk, :], self.Kgroup_size, self.k_bits,
+                                                           v_tail[:, :, :nv, :], self.Vgroup_size, self.v_bits)
+        else:
+            if nk > 0:
+                kc, ks, km = ops.quantize_pack_last_dim_cuda(k_tail[:, :, :nk, :].transpose(2, 3).contiguous(),
+                                                             self.Kgroup_size, self.k_bits)
+            if nv > 0:
+                vc, vs, vm = ops.quantize_pack_last_dim_cuda(v_tail[:, :, :nv, :].contiguous(), self.Vgroup_size,
+                                                             self.v_bits)
+        if kc is not None:
+            k_tail = k_tail[:, :, nk:, :]
+            kq = (_cat(kq[0], kc, 3), _cat(kq[1], ks, 3), _cat(kq[2], km, 3))
+        if vc is not None:
+            v_tail = v_tail[:, :, nv:, :]
+            vq = (_cat(vq[0], vc, 2), _cat(vq[1], vs, 2), _cat(vq[2], vm, 2))
+        return k_tail, kq, v_tail, vq
 
     # -- the step --------------------------------------------------------------------------
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
@@ -127,8 +133,7 @@ class KVmixAttention:
             kc, k_tail, ks, km, vc, v_tail, vs, vm, _ = past_key_value
             k_tail = key_states if k_tail is None else torch.cat([k_tail, key_states], dim=2)
             v_tail = value_states if v_tail is None else torch.cat([v_tail, value_states], dim=2)
-            k_tail, kc, ks, km = self._flush_keys(k_tail, kc, ks, km)
-            v_tail, vc, vs, vm = self._flush_values(v_tail, vc, vs, vm)
+            k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(k_tail, (kc, ks, km), v_tail, (vc, vs, vm))
 
             att_full = _grouped_matmul_qk(query_states, k_tail, n_rep)
             if kc is not None:
@@ -156,8 +161,8 @@ class KVmixAttention:
         else:
             # prompt: dense fp16 attention; the cache keeps the oldest tokens quantized
             # (models/modeling_llama_KVmix.py:213-266)
-            k_tail, kc, ks, km = self._flush_keys(key_states, None, None, None, prompt=True)
-            v_tail, vc, vs, vm = self._flush_values(value_states, None, None, None, prompt=True)
+            k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(key_states, (None,) * 3, value_states,
+                                                                     (None,) * 3, prompt=True)
             k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
             attn_weights = _grouped_matmul_qk(query_states, key_states, n_rep) / math.sqrt(D)
             if attention_mask is not None:

@@ -134,10 +134,9 @@ __global__ void __launch_bounds__(256) quant_rows_generic(QuantArgs a, int unit,
 // BITS = 1, 2, 4 (reference layout) or 3 with DENSE3 = true (bit-stream extension).
 // ---------------------------------------------------------------------------------------
 template <int BITS>
-__global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t groups_per_row,
-                                                          int64_t total_groups)
+__device__ __forceinline__ void rows_g32_f16_body(const QuantArgs &a, int64_t groups_per_row,
+                                                  int64_t total_groups, int64_t tid)
 {
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int64_t g = tid >> 2;
     const int j = (int)(tid & 3);
     const bool active = g < total_groups;
@@ -208,6 +207,13 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t g
     }
 }
 
+template <int BITS>
+__global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t groups_per_row,
+                                                          int64_t total_groups)
+{
+    rows_g32_f16_body<BITS>(a, groups_per_row, total_groups, (int64_t)blockIdx.x * blockDim.x + threadIdx.x);
+}
+
 // ---------------------------------------------------------------------------------------
 // keys from the token-major tail: k [outer, n, D] -> code [outer, D, n/vpw], groups of G
 // tokens per channel.  One thread per channel, one block row per (group, outer).
@@ -227,15 +233,11 @@ struct KeyTokArgs {
 };
 
 template <int G, int MODE>
-__global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
+__device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi, int64_t o, int64_t d)
 {
     constexpr int BITS = MODE == 30 ? 3 : MODE;
     constexpr int qmax = (1 << BITS) - 1;
     constexpr int WORDS = MODE == 3 ? 1 : (G * BITS) / 32;  // words per group
-    const int64_t d = (int64_t)blockIdx.z * blockDim.x + threadIdx.x;
-    if (d >= a.D) return;
-    const int64_t gi = blockIdx.x;
-    const int64_t o = blockIdx.y;
     const __half *src = a.k + o * a.k_os + gi * G * a.k_ts + d;
     float v[G];
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
@@ -268,6 +270,47 @@ __global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
     a.scale[o * a.s_os + d * a.s_is + gi] =
         __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
     a.zero[o * a.s_os + d * a.s_is + gi] = __float2half_rn(mn);
+}
+
+template <int G, int MODE>
+__global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
+{
+    const int64_t d = (int64_t)blockIdx.z * blockDim.x + threadIdx.x;
+    if (d >= a.D) return;
+    key_tokens_body<G, MODE>(a, blockIdx.x, blockIdx.y, d);
+}
+
+// ---------------------------------------------------------------------------------------
+// both flushes of a decode step in one launch: blocks [0, k_blocks) run the key-token
+// quantizer (one thread per (group, outer, channel)), the rest the group-32 value quantizer.
+// The two parts touch disjoint tensors; a launch of this size is latency-bound, so one
+// launch costs about what either part costs alone.
+// ---------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, int64_t k_groups,
+                                                      int64_t k_threads, unsigned k_blocks, QuantArgs va,
+                                                      int64_t v_groups_per_row, int64_t v_total_groups)
+{
+    if (blockIdx.x < k_blocks) {
+        const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (id >= k_threads) return;
+        const int64_t d = id % ka.D, pair = id / ka.D;
+        const int64_t gi = pair % k_groups, o = pair / k_groups;
+        switch (kmode) {
+        case 1: key_tokens_body<32, 1>(ka, gi, o, d); break;
+        case 2: key_tokens_body<32, 2>(ka, gi, o, d); break;
+        case 3: key_tokens_body<11, 3>(ka, gi, o, d); break;
+        case 4: key_tokens_body<32, 4>(ka, gi, o, d); break;
+        default: key_tokens_body<32, 30>(ka, gi, o, d); break;
+        }
+    } else {
+        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * 256 + threadIdx.x;
+        switch (va.bits) {
+        case 1: rows_g32_f16_body<1>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3>(va, v_groups_per_row, v_total_groups, tid); break;
+        default: rows_g32_f16_body<4>(va, v_groups_per_row, v_total_groups, tid); break;
+        }
+    }
 }
 
 static int64_t gcd64(int64_t a, int64_t b)
@@ -304,24 +347,26 @@ static int check_format(int group, int bits, int fmt, int64_t steps, int *vpw)
     return KVMIX_OK;
 }
 
-}  // namespace kvmix
-
-using namespace kvmix;
-
-extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t outer, int64_t inner,
-                                         int64_t steps, int64_t x_outer_stride, int64_t x_inner_stride,
-                                         int group, int bits, int fmt, int scale_mode, uint32_t *code,
-                                         int64_t code_outer_stride, int64_t code_inner_stride,
-                                         void *scale, void *zero, int64_t sz_outer_stride,
-                                         int64_t sz_inner_stride, kvmix_stream_t stream)
+// Validation and argument set-up shared by the separate and the fused entry points.
+// *empty is set when there is nothing to do; *fast when the group-32 fp16 kernel applies.
+static int setup_last_dim(const void *x, int x_dtype, int64_t outer, int64_t inner, int64_t steps,
+                          int64_t x_outer_stride, int64_t x_inner_stride, int group, int bits, int fmt,
+                          int scale_mode, uint32_t *code, int64_t code_outer_stride,
+                          int64_t code_inner_stride, void *scale, void *zero, int64_t sz_outer_stride,
+                          int64_t sz_inner_stride, QuantArgs &a, int &vpw, bool &empty, bool &fast)
 {
-    int vpw = 0;
+    vpw = 0;
+    empty = false;
+    fast = false;
     if (x_dtype != KVMIX_F16 && x_dtype != KVMIX_F32) return KVMIX_ERR_DTYPE;
     if (outer < 0 || inner < 0 || steps < 0) return KVMIX_ERR_SHAPE;
     int rc = check_format(group, bits, fmt, steps, &vpw);
     if (rc != KVMIX_OK) return rc;
     if (scale_mode != KVMIX_SCALE_RECIPROCAL && scale_mode != KVMIX_SCALE_DIVIDE) return KVMIX_ERR_FORMAT;
-    if (outer == 0 || inner == 0 || steps == 0) return KVMIX_OK;
+    if (outer == 0 || inner == 0 || steps == 0) {
+        empty = true;
+        return KVMIX_OK;
+    }
     if (!x || !code || !scale || !zero) return KVMIX_ERR_NULL;
     const int64_t words = vpw ? steps / vpw : steps * 3 / 32;
     const int64_t groups = steps / group;
@@ -330,7 +375,6 @@ extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t out
                       sz_outer_stride < sz_inner_stride))
         return KVMIX_ERR_SHAPE;
 
-    QuantArgs a;
     a.x = x;
     a.code = code;
     a.scale = scale;
@@ -349,15 +393,20 @@ extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t out
     a.fmt = fmt;
     a.scale_mode = scale_mode;
     a.inv_qmax = 1.0f / (float)((1 << bits) - 1);
-    hipStream_t st = (hipStream_t)stream;
-
     const bool ref3 = bits == 3 && fmt != KVMIX_FMT_DENSE3;
     const bool aligned16 = ((uintptr_t)x % 16 == 0) && (x_outer_stride % 8 == 0) && (x_inner_stride % 8 == 0);
-    if (x_dtype == KVMIX_F16 && group == 32 && !ref3 && aligned16) {
-        const int64_t total_groups = outer * inner * groups;
+    fast = x_dtype == KVMIX_F16 && group == 32 && !ref3 && aligned16;
+    return KVMIX_OK;
+}
+
+static int launch_last_dim(const QuantArgs &a, int x_dtype, int vpw, bool fast, hipStream_t st)
+{
+    const int64_t groups = a.steps / a.group;
+    if (fast) {
+        const int64_t total_groups = a.outer * a.inner * groups;
         const int64_t threads = total_groups * 4;
         const unsigned blocks = (unsigned)((threads + 255) / 256);
-        switch (bits) {
+        switch (a.bits) {
         case 1: hipLaunchKernelGGL(quant_rows_g32_f16<1>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
         case 2: hipLaunchKernelGGL(quant_rows_g32_f16<2>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
         case 3: hipLaunchKernelGGL(quant_rows_g32_f16<3>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
@@ -367,10 +416,10 @@ extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t out
     }
     // generic path: a thread owns lcm(group, codes per word) values, i.e. whole groups and whole words
     const int64_t word_span = vpw ? vpw : 32;
-    const int64_t unit = (int64_t)group / gcd64(group, word_span) * word_span;
-    if (steps % unit != 0 || unit > (1 << 20)) return KVMIX_ERR_UNSUPPORTED;
-    const int64_t units_per_row = steps / unit;
-    const int64_t total_units = outer * inner * units_per_row;
+    const int64_t unit = (int64_t)a.group / gcd64(a.group, word_span) * word_span;
+    if (a.steps % unit != 0 || unit > (1 << 20)) return KVMIX_ERR_UNSUPPORTED;
+    const int64_t units_per_row = a.steps / unit;
+    const int64_t total_units = a.outer * a.inner * units_per_row;
     const unsigned blocks = (unsigned)((total_units + 255) / 256);
     if (x_dtype == KVMIX_F16)
         hipLaunchKernelGGL(quant_rows_generic<__half>, dim3(blocks), dim3(256), 0, st, a, (int)unit,
@@ -381,14 +430,15 @@ extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t out
     return launch_status();
 }
 
-extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D,
-                                           int64_t k_outer_stride, int64_t k_token_stride, int group,
-                                           int bits, int fmt, int scale_mode, uint32_t *code,
-                                           int64_t code_outer_stride, int64_t code_inner_stride,
-                                           void *scale, void *zero, int64_t sz_outer_stride,
-                                           int64_t sz_inner_stride, kvmix_stream_t stream)
+// *mode: 1, 2, 4 (reference layout), 3 (reference 3-bit), 30 (dense 3-bit)
+static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, int64_t k_outer_stride,
+                            int64_t k_token_stride, int group, int bits, int fmt, int scale_mode,
+                            uint32_t *code, int64_t code_outer_stride, int64_t code_inner_stride,
+                            void *scale, void *zero, int64_t sz_outer_stride, int64_t sz_inner_stride,
+                            KeyTokArgs &a, int &mode, int64_t &groups, bool &empty)
 {
     int vpw = 0;
+    empty = false;
     if (outer < 0 || n < 0 || D < 0) return KVMIX_ERR_SHAPE;
     if (fmt == KVMIX_FMT_REF3_WRAP) return KVMIX_ERR_FORMAT;
     int rc = check_format(group, bits, fmt, n, &vpw);
@@ -396,14 +446,15 @@ extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t
     const bool ref3 = bits == 3 && fmt == KVMIX_FMT_REF;
     if (!ref3 && group != 32) return KVMIX_ERR_UNSUPPORTED;
     if (scale_mode != KVMIX_SCALE_RECIPROCAL && scale_mode != KVMIX_SCALE_DIVIDE) return KVMIX_ERR_FORMAT;
-    if (outer == 0 || n == 0 || D == 0) return KVMIX_OK;
+    if (outer == 0 || n == 0 || D == 0) {
+        empty = true;
+        return KVMIX_OK;
+    }
     if (!k || !code || !scale || !zero) return KVMIX_ERR_NULL;
     const int64_t words = vpw ? n / vpw : n * 3 / 32;
-    const int64_t groups = n / group;
+    groups = n / group;
     if (k_token_stride < D || code_inner_stride < words || sz_inner_stride < groups) return KVMIX_ERR_SHAPE;
     if (outer > 65535 || groups > 0x7fffffff) return KVMIX_ERR_SHAPE;
-
-    KeyTokArgs a;
     a.k = (const __half *)k;
     a.code = code;
     a.scale = (__half *)scale;
@@ -418,18 +469,97 @@ extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t
     a.s_is = sz_inner_stride;
     a.scale_mode = scale_mode;
     a.inv_qmax = 1.0f / (float)((1 << bits) - 1);
+    mode = ref3 ? 3 : (bits == 3 ? 30 : bits);
+    return KVMIX_OK;
+}
+
+static int launch_key_tokens(const KeyTokArgs &a, int mode, int64_t groups, int64_t outer, hipStream_t st)
+{
+    const int block = a.D >= 128 ? 128 : 64;
+    const dim3 grid((unsigned)groups, (unsigned)outer, (unsigned)((a.D + block - 1) / block));
+    switch (mode) {
+    case 3: hipLaunchKernelGGL((quant_key_tokens<11, 3>), grid, dim3(block), 0, st, a); break;
+    case 30: hipLaunchKernelGGL((quant_key_tokens<32, 30>), grid, dim3(block), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((quant_key_tokens<32, 4>), grid, dim3(block), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((quant_key_tokens<32, 2>), grid, dim3(block), 0, st, a); break;
+    default: hipLaunchKernelGGL((quant_key_tokens<32, 1>), grid, dim3(block), 0, st, a); break;
+    }
+    return launch_status();
+}
+
+}  // namespace kvmix
+
+using namespace kvmix;
+
+extern "C" int kvmix_quant_pack_last_dim(const void *x, int x_dtype, int64_t outer, int64_t inner,
+                                         int64_t steps, int64_t x_outer_stride, int64_t x_inner_stride,
+                                         int group, int bits, int fmt, int scale_mode, uint32_t *code,
+                                         int64_t code_outer_stride, int64_t code_inner_stride,
+                                         void *scale, void *zero, int64_t sz_outer_stride,
+                                         int64_t sz_inner_stride, kvmix_stream_t stream)
+{
+    QuantArgs a;
+    int vpw;
+    bool empty, fast;
+    const int rc = setup_last_dim(x, x_dtype, outer, inner, steps, x_outer_stride, x_inner_stride, group, bits, fmt,
+                                  scale_mode, code, code_outer_stride, code_inner_stride, scale, zero,
+                                  sz_outer_stride, sz_inner_stride, a, vpw, empty, fast);
+    if (rc != KVMIX_OK || empty) return rc;
+    return launch_last_dim(a, x_dtype, vpw, fast, (hipStream_t)stream);
+}
+
+extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D,
+                                           int64_t k_outer_stride, int64_t k_token_stride, int group,
+                                           int bits, int fmt, int scale_mode, uint32_t *code,
+                                           int64_t code_outer_stride, int64_t code_inner_stride,
+                                           void *scale, void *zero, int64_t sz_outer_stride,
+                                           int64_t sz_inner_stride, kvmix_stream_t stream)
+{
+    KeyTokArgs a;
+    int mode = 0;
+    int64_t groups = 0;
+    bool empty;
+    const int rc = setup_key_tokens(k, outer, n, D, k_outer_stride, k_token_stride, group, bits, fmt, scale_mode, code,
+                                    code_outer_stride, code_inner_stride, scale, zero, sz_outer_stride,
+                                    sz_inner_stride, a, mode, groups, empty);
+    if (rc != KVMIX_OK || empty) return rc;
+    return launch_key_tokens(a, mode, groups, outer, (hipStream_t)stream);
+}
+
+extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf,
+                                         kvmix_stream_t stream)
+{
+    if (!kf || !vf) return KVMIX_ERR_NULL;
+    KeyTokArgs ka;
+    QuantArgs va;
+    int kmode = 0, vpw = 0;
+    int64_t kgroups = 0;
+    bool kempty, vempty, vfast;
+    int rc = setup_key_tokens(kf->k, kf->outer, kf->n, kf->D, kf->k_outer_stride, kf->k_token_stride, kf->group,
+                              kf->bits, kf->fmt, kf->scale_mode, kf->code, kf->code_outer_stride,
+                              kf->code_inner_stride, kf->scale, kf->zero, kf->sz_outer_stride, kf->sz_inner_stride,
+                              ka, kmode, kgroups, kempty);
+    if (rc != KVMIX_OK) return rc;
+    rc = setup_last_dim(vf->x, KVMIX_F16, vf->outer, vf->inner, vf->steps, vf->x_outer_stride, vf->x_inner_stride,
+                        vf->group, vf->bits, vf->fmt, vf->scale_mode, vf->code, vf->code_outer_stride,
+                        vf->code_inner_stride, vf->scale, vf->zero, vf->sz_outer_stride, vf->sz_inner_stride, va, vpw,
+                        vempty, vfast);
+    if (rc != KVMIX_OK) return rc;  // (nothing was launched: both halves are checked first)
     hipStream_t st = (hipStream_t)stream;
-    const int block = D >= 128 ? 128 : 64;
-    const dim3 grid((unsigned)groups, (unsigned)outer, (unsigned)((D + block - 1) / block));
-    if (ref3)
-        hipLaunchKernelGGL((quant_key_tokens<11, 3>), grid, dim3(block), 0, st, a);
-    else if (bits == 3)
-        hipLaunchKernelGGL((quant_key_tokens<32, 30>), grid, dim3(block), 0, st, a);
-    else if (bits == 4)
-        hipLaunchKernelGGL((quant_key_tokens<32, 4>), grid, dim3(block), 0, st, a);
-    else if (bits == 2)
-        hipLaunchKernelGGL((quant_key_tokens<32, 2>), grid, dim3(block), 0, st, a);
-    else
-        hipLaunchKernelGGL((quant_key_tokens<32, 1>), grid, dim3(block), 0, st, a);
+    if (kempty || vempty || !vfast) {
+        // one half is empty or the value half needs the generic quantizer: separate launches
+        if (!kempty) {
+            rc = launch_key_tokens(ka, kmode, kgroups, kf->outer, st);
+            if (rc != KVMIX_OK) return rc;
+        }
+        return vempty ? KVMIX_OK : launch_last_dim(va, KVMIX_F16, vpw, vfast, st);
+    }
+    const int64_t k_threads = kgroups * kf->outer * kf->D;
+    const int64_t k_blocks = (k_threads + 255) / 256;
+    const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
+    const int64_t v_blocks = (v_total * 4 + 255) / 256;
+    if (k_blocks + v_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    hipLaunchKernelGGL(quant_kv_flush, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, ka, kmode, kgroups,
+                       k_threads, (unsigned)k_blocks, va, v_groups, v_total);
     return launch_status();
 }

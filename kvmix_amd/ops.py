@@ -124,6 +124,53 @@ FMT_REF = _lib.FMT_REF
 FMT_DENSE3 = _lib.FMT_DENSE3
 
 
+def quantize_kv_flush(k_chunk: torch.Tensor, k_group: int, k_bits: int, v_chunk: torch.Tensor, v_group: int,
+                      v_bits: int, k_fmt: int = _lib.FMT_REF, v_fmt: int = _lib.FMT_REF):
+    """Extension (no reference counterpart): both flushes of a decode step in ONE launch.
+
+    k_chunk [B,H,n,D] fp16 are the oldest n tokens of the key tail, token-major as the tail is
+    stored; the result is what quantize_pack_last_dim_cuda(k_chunk.transpose(2, 3).contiguous(),
+    k_group, k_bits) returns (models/modeling_llama_KVmix.py:131-133), without the transpose copy.
+    v_chunk [B,H,nv,D] fp16 is quantized along D as quantize_pack_last_dim_cuda(v_chunk, v_group,
+    v_bits) does (:157-159).  Bit-identical to the two separate operators.
+    Returns (k_code [B,H,D,n/vpw], k_scale, k_min [B,H,D,n/g], v_code [B,H,nv,D/vpw], v_scale, v_min)."""
+    for t in (k_chunk, v_chunk):
+        if t.dim() != 4:
+            raise RuntimeError("input_tensor must be a 4D tensor")
+        if t.dtype != torch.float16:
+            raise RuntimeError(f"expected scalar type Half but found {t.dtype}")
+    _check_bits(k_bits)
+    _check_bits(v_bits)
+    _need_gpu(k_chunk, v_chunk)
+    L = _lib.load()
+    B, H, n, D = k_chunk.shape
+    Bv, Hv, nv, Dv = v_chunk.shape
+    dev = k_chunk.device
+
+    def words(steps, bits, fmt):
+        return steps * 3 // 32 if (bits == 3 and fmt == _lib.FMT_DENSE3) else steps // _values_per_word(bits)
+
+    if k_chunk.stride(3) != 1 or (B > 1 and k_chunk.stride(0) != H * k_chunk.stride(1)):
+        k_chunk = k_chunk.contiguous()
+    v_chunk, vo, vi = _rows3(v_chunk)
+    kc = torch.empty((B, H, D, words(n, k_bits, k_fmt)), dtype=torch.int32, device=dev)
+    ks = torch.empty((B, H, D, n // k_group if k_group > 0 else 0), dtype=torch.float16, device=dev)
+    km = torch.empty_like(ks)
+    vc = torch.empty((Bv, Hv, nv, words(Dv, v_bits, v_fmt)), dtype=torch.int32, device=dev)
+    vs = torch.empty((Bv, Hv, nv, Dv // v_group if v_group > 0 else 0), dtype=torch.float16, device=dev)
+    vm = torch.empty_like(vs)
+    kf = _lib.KeyFlush(k_chunk.data_ptr(), B * H, n, D, k_chunk.stride(1), k_chunk.stride(2), k_group, k_bits, k_fmt,
+                       _lib.SCALE_RECIPROCAL, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(), km.data_ptr(),
+                       ks.stride(1), ks.stride(2))
+    vf = _lib.ValueFlush(v_chunk.data_ptr(), Bv * Hv, nv, Dv, vo, vi, v_group, v_bits, v_fmt, _lib.SCALE_RECIPROCAL,
+                         vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(), vm.data_ptr(), vs.stride(1),
+                         vs.stride(2))
+    import ctypes
+    with torch.cuda.device(dev):
+        _lib.check(L.kvmix_quant_pack_kv_flush(ctypes.byref(kf), ctypes.byref(vf), _stream(k_chunk)))
+    return kc, ks, km, vc, vs, vm
+
+
 def _batched3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:
     """[B, H, R, S] -> (tensor, batch stride, row stride) with (B, H) collapsible, unit last stride."""
     B, H, R, S = t.shape
