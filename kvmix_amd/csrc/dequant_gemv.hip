@@ -46,15 +46,6 @@
 #ifndef KVMIX_MFMA_HEADS_OCC
 #define KVMIX_MFMA_HEADS_OCC 2
 #endif
-#ifndef KVMIX_MFMA_DEPTH4
-#define KVMIX_MFMA_DEPTH4 1
-#endif
-#ifndef KVMIX_MFMA_DEPTH2
-#define KVMIX_MFMA_DEPTH2 1
-#endif
-#ifndef KVMIX_MFMA_DEPTH1
-#define KVMIX_MFMA_DEPTH1 1
-#endif
 
 #ifndef KVMIX_TARGET_WAVES
 #define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
@@ -917,6 +908,10 @@ template <>
 struct CodeElem<1> {
     using type = uint8_t;
 };
+template <>
+struct CodeElem<30> {
+    using type = uint32_t;
+};
 
 constexpr int rows_mfma_sets(int nrep) { return (3 * nrep + 3) / 4; }
 constexpr int kRowsMfmaTile = (32 * 17 + 1) * 4 + 4;  // bf16 elements of one A tile (32 skewed rows), 8-byte multiple
@@ -927,7 +922,10 @@ template <int BITS, int NREP, int DEPTH>
 __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWaves))
     __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_MFMA_HEADS_OCC : 4))) gemv_rows_mfma(GemvArgs a)
 {
+    // BITS = 30: dense 3-bit stream, a lane's 8 codes are 3 bytes
     using Elem = typename CodeElem<BITS>::type;
+    constexpr int EB = BITS == 30 ? 3 : BITS;   // bytes of a lane's 8 codes
+    constexpr int FB = BITS == 30 ? 3 : BITS;   // bits of a code
     constexpr int LPR = 4;             // groups per row (N = 128)
     constexpr int EPR = 16;            // lanes (8-code elements) per row
     constexpr int RL = kWave / EPR;    // rows per load instruction (4)
@@ -937,7 +935,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     constexpr int AT = kRowsMfmaTile;  // bf16 elements of one A tile
     constexpr int NM = rows_mfma_sets(NREP);  // MFMAs per B operand
     constexpr int NPOS = 8;            // code positions per lane
-    constexpr int FPB = 8 / BITS;      // fields per byte
+    constexpr int FPB = 8 / FB;        // whole fields per byte window
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
@@ -956,7 +954,11 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     const int64_t kend = kbeg + a.rows_per_split < a.K ? kbeg + a.rows_per_split : a.K;
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
-    const Elem *cp = reinterpret_cast<const Elem *>(a.code + kv * a.c_bs) + wi;
+    // dense 3-bit: a group is three aligned words; lane j of the group's four loads word
+    // min(j, 2), and its 24 bits [24j, 24j+24) are cut out of two neighbours' words in compute()
+    const uint8_t *cp = reinterpret_cast<const uint8_t *>(a.code + kv * a.c_bs) +
+                        (BITS == 30 ? (wi / 4) * 12 + (wi % 4 < 2 ? wi % 4 : 2) * 4 : wi * EB);
+    [[maybe_unused]] const uint32_t sh3 = (uint32_t)(24 * (wi % 4)) % 32u;
     const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs;
     const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs;
 
@@ -1018,9 +1020,10 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         for (int h = 0; h < NREP; h++) xh[d][h] = *reinterpret_cast<const Half2x *>(xp + h * a.x_bs + kr);
     };
     auto load_codes = [&](int d, int k0, int t) {
-        const Elem *base = cp + (uint32_t)(chunk_base(k0) + rs) * EPR;
+        const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
 #pragma unroll
-        for (int k = 0; k < 4; k++) w[d][t][k] = base[(t * RKB + RL * k) * EPR];
+        for (int k = 0; k < 4; k++)
+            w[d][t][k] = *reinterpret_cast<const Elem *>(base + (t * RKB + RL * k) * (EPR * EB));
     };
     auto stage = [&](int d, int k0) {
         const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
@@ -1051,20 +1054,46 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
 #pragma unroll
         for (int q = 0; q < NM; q++)
             av[q] = *reinterpret_cast<const bf16x4_t *>(atile + q * AT + cell(t, lane));
+        if constexpr (BITS == 30) {
+            // 24-bit stream per row: codes (2m, 2m+1) lie in the 8-bit window at bit 6m
+            uint32_t v[4];
 #pragma unroll
-        for (int b = 0; b < BITS; b++) {
-            // byte b of rows k and k+1 -> low bytes of the two halves
-            const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-            const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
-            const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+            for (int k = 0; k < 4; k++) {
+                // words (0,0,1,2) and (0,1,2,2) of the group for lanes 0..3, funnel-shifted
+                const uint32_t lo = __builtin_amdgcn_mov_dpp(w[d][t][k], 0x90, 0xf, 0xf, false);
+                const uint32_t hi = __builtin_amdgcn_mov_dpp(w[d][t][k], 0xA4, 0xf, 0xf, false);
+                v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
+            }
 #pragma unroll
-            for (int f = 0; f < FPB; f++) {
-                const uint32_t mask = (((1u << BITS) - 1u) * 0x00010001u) << (BITS * f);
-                const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+            for (int mm = 0; mm < 4; mm++) {
+                const uint32_t t01 = __builtin_amdgcn_perm(v[1] >> (6 * mm), v[0] >> (6 * mm), 0x0c040c00u);
+                const uint32_t t23 = __builtin_amdgcn_perm(v[3] >> (6 * mm), v[2] >> (6 * mm), 0x0c040c00u);
 #pragma unroll
-                for (int q = 0; q < NM; q++)
-                    acc[q][b * FPB + f] =
-                        __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[q], bv, acc[q][b * FPB + f], 0, 0, 0);
+                for (int f = 0; f < 2; f++) {
+                    const uint32_t mask = 0x00070007u << (3 * f);
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+#pragma unroll
+                    for (int q = 0; q < NM; q++)
+                        acc[q][mm * 2 + f] =
+                            __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[q], bv, acc[q][mm * 2 + f], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < EB; b++) {
+                // byte b of rows k and k+1 -> low bytes of the two halves
+                const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+#pragma unroll
+                for (int f = 0; f < FPB; f++) {
+                    const uint32_t mask = (((1u << FB) - 1u) * 0x00010001u) << (FB * f);
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+#pragma unroll
+                    for (int q = 0; q < NM; q++)
+                        acc[q][b * FPB + f] =
+                            __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[q], bv, acc[q][b * FPB + f], 0, 0, 0);
+                }
             }
         }
     };
@@ -1131,7 +1160,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         for (int p = 0; p < NPOS; p++) {
             const float sum = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
                               acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
-            flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23);
+            flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - FB * (p % FPB)) << 23);
         }
     }
     __syncthreads();  // every wave is done with its A tile: the space becomes `red`
@@ -1480,8 +1509,8 @@ static int heads_per_block(int heads_per_kv) { return heads_per_kv % 4 == 0 ? 4 
 // (gemv_rows_mfma: N = 128, dense code rows, at least one whole 128-row chunk)
 static bool rows_use_mfma(int mode, int64_t N, int64_t K, int64_t c_rs)
 {
-    return KVMIX_ROWS_MFMA && (mode == 1 || mode == 2 || mode == 4) && N == 128 && K >= 128 &&
-           c_rs == N * mode / 32;
+    return KVMIX_ROWS_MFMA && (mode == 1 || mode == 2 || mode == 4 || mode == 30) && N == 128 && K >= 128 &&
+           c_rs == N * (mode == 30 ? 3 : mode) / 32;
 }
 static int rows_max_waves(bool mfma, int nrep)
 {
@@ -1497,11 +1526,11 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
     a.splits = p.splits;
     a.rows_per_split = p.rows_per_split;
     const dim3 grid((unsigned)a.splits, (unsigned)(samples / NREP), (unsigned)a.M), block(kWave, p.waves);
-    if constexpr (MODE == 1 || MODE == 2 || MODE == 4) {
+    {
       if (mfma) {
         // one A tile per wave and MFMA set; the block reduction (waves*NREP*128 floats) reuses it
         const size_t lds = (size_t)p.waves * rows_mfma_sets(NREP) * kRowsMfmaTile * sizeof(uint16_t);
-        constexpr int DEPTH = NREP == 1 ? (MODE == 4 ? KVMIX_MFMA_DEPTH4 : (MODE == 2 ? KVMIX_MFMA_DEPTH2 : KVMIX_MFMA_DEPTH1)) : 1;
+        constexpr int DEPTH = 1;  // chunks in flight per wave (deeper costs occupancy and was slower)
         if (lds > 64 * 1024) {
             // above the default per-block limit: raise it for this kernel, once per device
             static bool raised[64] = {};
