@@ -31,6 +31,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
+# device kernel behind each tag at this workload (the names the rocprofv3 summaries list)
+DEVICE_KERNEL = {
+    "gemv_cols[ref3]": "kvmix::gemv_cols3<2, 2, 8>", "gemv_cols[b4]": "kvmix::gemv_cols_mfma<4, 1>",
+    "gemv_cols[b2]": "kvmix::gemv_cols_mfma<2, 1>", "gemv_rows[b4]": "kvmix::gemv_rows_mfma<4, 1, 1>",
+    "gemv_rows[b2]": "kvmix::gemv_rows_mfma<2, 1, 1>", "gemv_rows[dense3]": "kvmix::gemv_rows_mfma<30, 1, 1>",
+}
+
+
 def layer_bits(num_layers: int = 32, seed: int = 1):
     rng = np.random.default_rng(seed)
     base = np.array([4] * (num_layers // 4) + [3] * (num_layers // 2) + [2] * (num_layers // 4))
@@ -402,7 +410,8 @@ def main():
                            "GBps": round(quant_bytes / quant_us / 1e3, 1)},
         "kernels": {k: {"launches_per_step": v["launches_per_step"], "avg_us": round(v["avg_us"], 2),
                         "GBps": round(v["bytes_per_launch"] / v["avg_us"] / 1e3, 1)} for k, v in per_kernel.items()},
-        "roofline": {"kernel": dname, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"kernel": dname, "device_kernel": DEVICE_KERNEL.get(dname.split("[")[0] + "[" + dname.split("[")[1], ""),
+                     "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "bytes_per_launch": int(d["bytes_per_launch"]), "avg_launch_us": round(d["avg_us"], 2)},
     }
