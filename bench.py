@@ -410,7 +410,7 @@ def main():
                            "GBps": round(quant_bytes / quant_us / 1e3, 1)},
         "kernels": {k: {"launches_per_step": v["launches_per_step"], "avg_us": round(v["avg_us"], 2),
                         "GBps": round(v["bytes_per_launch"] / v["avg_us"] / 1e3, 1)} for k, v in per_kernel.items()},
-        "roofline": {"kernel": dname, "device_kernel": DEVICE_KERNEL.get(dname.split("[")[0] + "[" + dname.split("[")[1], ""),
+        "roofline": {"kernel": dname, "device_kernel": DEVICE_KERNEL.get(dname, ""),
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "bytes_per_launch": int(d["bytes_per_launch"]), "avg_launch_us": round(d["avg_us"], 2)},

@@ -59,6 +59,24 @@ def test_gqa_head_mapping(oracle, dev, bits, g):
         run_case(oracle, dev, bits, g, B=2, nh=8, nkv=2, K=200, N=128, seed=22)
 
 
+@pytest.mark.parametrize("bits,g", [(4, 32), (2, 32), (1, 32)])
+def test_matrix_core_kernel_edges(oracle, dev, bits, g):
+    """Shapes that exercise the edges of the matrix-core kernels: a last row chunk moved back to
+    end at K (K not a multiple of the chunk), a last tile shifted to end at N, several tiles per
+    wave, GQA head groups with ragged tiles, GQA split-K, and a query-row count M > 1."""
+    # q.K^T: K below / between / above chunk multiples, N ragged against the 512-code tile
+    for K, N in ((32, 512), (40, 544), (96, 1024 + 32), (200, 512 * 5 + 96)):
+        run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=K, N=N, seed=K + N)
+    run_case(oracle, dev, bits, g, B=1, nh=8, nkv=2, K=128, N=32 * 41, seed=41)      # GQA, 4 heads per block
+    run_case(oracle, dev, bits, g, B=1, nh=6, nkv=2, K=128, N=32 * 20, seed=42)      # GQA, 3 heads per kv head
+    run_case(oracle, dev, bits, g, B=4, nh=16, nkv=16, K=64, N=512 * 9, seed=43)     # many tiles
+    # p.V: chunks of 128 rows, K ragged; GQA with split-K; M = 2
+    for K in (128, 129, 255, 1000):
+        run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=K, N=128, seed=K)
+    run_case(oracle, dev, bits, g, B=1, nh=8, nkv=2, K=5000, N=128, seed=44)
+    run_case(oracle, dev, bits, g, B=1, nh=4, nkv=4, K=777, N=128, seed=45, M=2)
+
+
 @pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
 def test_generic_shapes(oracle, dev, bits, g):
     """Group sizes and shapes outside the fast kernels (including a 3-bit p.V shape)."""
