@@ -283,6 +283,58 @@ def target_shape_extra(torch, _lib, lib, dev, stream):
     return res
 
 
+def gqa_shape_extra(torch, _lib, lib, dev, stream):
+    """BASELINE configs[2]: GQA 32 query / 8 kv heads, B=16, T=32768, reference 3-bit keys (group 11,
+    32637 quantized tokens), 2-bit values (32640).  The bytes are the packed cache's, counted once:
+    the four query heads of a kv head are served from one pass (p.V) or from one L2 (q.K^T)."""
+    B, H, Hkv, D = 16, 32, 8, 128
+    Tk, Tv = 32637, 32640
+    sets = []
+    for _ in range(2):
+        kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, D, Tk // 11), dtype=torch.int64, device=dev).to(torch.int32)
+        ks = torch.rand(B, Hkv, D, Tk // 11, device=dev).half()
+        kz = torch.randn(B, Hkv, D, Tk // 11, device=dev).half()
+        vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, Tv, D * 2 // 32), dtype=torch.int64, device=dev).to(torch.int32)
+        vs = torch.rand(B, Hkv, Tv, D // 32, device=dev).half()
+        vz = torch.randn(B, Hkv, Tv, D // 32, device=dev).half()
+        sets.append((kc, ks, kz, vc, vs, vz))
+    q = torch.randn(B, H, 1, D, device=dev).half()
+    p = torch.softmax(torch.randn(B, H, 1, Tv, device=dev), -1).half()
+    lo = torch.empty(B, H, 1, Tk, device=dev, dtype=torch.float16)
+    o = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+    wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, Tv, D)
+    ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+
+    def qk(i):
+        kc, ks, kz = sets[i % 2][:3]
+        return lib.kvmix_quantized_gemv(11, q.data_ptr(), D, D, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(),
+                                        kz.data_ptr(), ks.stride(1), ks.stride(2), 3, _lib.FMT_REF, B * H, H // Hkv, 1, D, Tk,
+                                        lo.data_ptr(), Tk, Tk, None, 0, stream)
+
+    def pv(i):
+        vc, vs, vz = sets[i % 2][3:]
+        return lib.kvmix_quantized_gemv(32, p.data_ptr(), Tv, Tv, vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(),
+                                        vz.data_ptr(), vs.stride(1), vs.stride(2), 2, _lib.FMT_REF, B * H, H // Hkv, 1, Tv, D,
+                                        o.data_ptr(), D, D, ws.data_ptr(), wsb, stream)
+
+    res = {}
+    for name, fn, nbytes in (("qk_ref3", qk, B * Hkv * Tk * bytes_per_token(3, "ref3")),
+                             ("pv_2bit", pv, B * Hkv * Tv * bytes_per_token(2, ""))):
+        for i in range(4):
+            assert fn(i) == 0
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(20):
+            fn(i)
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) * 1e3 / 20
+        res[name] = {"us": round(us, 2), "packed_MB": round(nbytes / 1e6, 1), "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -428,6 +480,9 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
         torch.cuda.empty_cache()
         result["target_shape_B16_T8192"] = target_shape_extra(torch, _lib, lib, dev,
                                                               torch.cuda.current_stream().cuda_stream)
+        torch.cuda.empty_cache()
+        result["gqa_config2_B16_T32768"] = gqa_shape_extra(torch, _lib, lib, dev,
+                                                           torch.cuda.current_stream().cuda_stream)
     print(json.dumps(result))
 
 

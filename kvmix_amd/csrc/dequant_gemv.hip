@@ -33,6 +33,12 @@
 
 #include "kvmix_common.h"
 
+#ifndef KVMIX_COLS3_HEADS_U
+#define KVMIX_COLS3_HEADS_U 4
+#endif
+#ifndef KVMIX_COLS3_HEADS_OCC
+#define KVMIX_COLS3_HEADS_OCC 2
+#endif
 #ifndef KVMIX_COLS_MFMA
 #define KVMIX_COLS_MFMA 1  // 1/2/4-bit q.K^T on the matrix cores
 #endif
@@ -516,27 +522,33 @@ __device__ __forceinline__ int scatter_reduce(float *v, int lane)
 //   rows).  Tiles as in gemv_cols: TU = (64/RQ)*4 words per wave, last tile shifted left.
 //   block = (64, 2..4); grid = (tiles/waves, samples, M), XCD-swizzled; dynamic LDS = (K+1)*4.
 // ---------------------------------------------------------------------------------------
-template <int RQ, int UPL, int U>
-__global__ void __launch_bounds__(64 * kColsWaves) gemv_cols3(GemvArgs a)
+template <int RQ, int UPL, int U, int NREP>
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_COLS3_HEADS_OCC : 3)))
+gemv_cols3(GemvArgs a)
 {
     constexpr int VALS = 11;
     constexpr int GL = kWave / RQ;
     constexpr int TU = GL * UPL;
-    extern __shared__ float xs[];  // [K + 1]
+    extern __shared__ float xs[];  // [NREP][K + 1]
 
     const int lane = threadIdx.x;
     const int wy = threadIdx.y;
     const int rq = lane / GL;
     const int gl = lane % GL;
-    int64_t bx, sample;
-    xcd_swizzled_block(bx, sample, true);
+    // grid.y counts head groups: NREP query heads that share one kv head (NREP == 1: plain)
+    int64_t bx, hg;
+    xcd_swizzled_block(bx, hg, true);
+    const int64_t sample0 = hg * NREP;
     const int64_t m = blockIdx.z;
-    const int64_t kv = sample / a.heads_per_kv;
+    const int64_t kv = sample0 / a.heads_per_kv;
     const int K = (int)a.K;
     const int nunits = (int)(a.N / VALS);
 
-    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
-    for (int i = wy * kWave + lane; i <= K; i += blockDim.y * kWave) xs[i] = i < K ? h16_to_f32(xp[i]) : 0.f;
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
+    for (int i = wy * kWave + lane; i < NREP * (K + 1); i += blockDim.y * kWave) {
+        const int h = i / (K + 1), k = i % (K + 1);
+        xs[i] = k < K ? h16_to_f32(xp[h * a.x_bs + k]) : 0.f;
+    }
     __syncthreads();
 
     int t0 = (int)(bx * blockDim.y + wy) * TU;
@@ -548,13 +560,16 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols3(GemvArgs a)
     const uint16_t *sp = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs + unit0;
     const uint16_t *zp = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs + unit0;
 
-    float acc[UPL][VALS];
-    float zsum[UPL];
+    float acc[UPL][NREP][VALS];
+    float zsum[NREP][UPL];
 #pragma unroll
     for (int j = 0; j < UPL; j++) {
-        zsum[j] = 0.f;
 #pragma unroll
-        for (int i = 0; i < VALS; i++) acc[j][i] = 0.f;
+        for (int h = 0; h < NREP; h++) {
+            zsum[h][j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < VALS; i++) acc[j][h][i] = 0.f;
+        }
     }
 
     // this lane's rows: [kbeg, kend), walked in steps of U
@@ -575,22 +590,35 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols3(GemvArgs a)
         zw[u] = *reinterpret_cast<const HalfN *>(zp + kc * s_rs);
     };
     auto compute_row = [&](int u, int k) {
-        const float xv = xs[k < kend ? k : K];
-        const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90, see accumulate_unit
+        const int kx = k < kend ? k : K;
+        float xv[NREP];
+#pragma unroll
+        for (int h = 0; h < NREP; h++) xv[h] = xs[h * (K + 1) + kx];
 #pragma unroll
         for (int j = 0; j < UPL; j++) {
             const half2_t sz = __builtin_bit_cast(half2_t, (uint32_t)sw[u].v[j] | ((uint32_t)zw[u].v[j] << 16));
-            zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
-            float mq[4];
-            mq[0] = x2 * (float)sz.x;
+            if constexpr (NREP == 1) {
+                zsum[0][j] = fmaf(xv[0], (float)sz.y, zsum[0][j]);
+                float mq[4];
+                mq[0] = (xv[0] * 1237940039285380274899124224.0f) * (float)sz.x;  // 2^90, see accumulate_unit
 #pragma unroll
-            for (int t = 1; t < 4; t++) mq[t] = mq[t - 1] * 0.125f;
-            const uint32_t w = cw[u].v[j];
-            const uint32_t v[3] = {w, w >> 12, w >> 24};
+                for (int t = 1; t < 4; t++) mq[t] = mq[t - 1] * 0.125f;
+                const uint32_t w = cw[u].v[j];
+                const uint32_t v[3] = {w, w >> 12, w >> 24};
 #pragma unroll
-            for (int i = 0; i < VALS; i++) {
-                const uint32_t mask = (i == 10 ? 3u : 7u) << (3 * (i % 4));
-                acc[j][i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & mask), acc[j][i]);
+                for (int i = 0; i < VALS; i++) {
+                    const uint32_t mask = (i == 10 ? 3u : 7u) << (3 * (i % 4));
+                    acc[j][0][i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & mask), acc[j][0][i]);
+                }
+            } else {
+                // the field masks are shared by the heads: one v_and_b32 + NREP v_fmac_f32 per code
+                float qs[NREP];
+#pragma unroll
+                for (int h = 0; h < NREP; h++) {
+                    zsum[h][j] = fmaf(xv[h], (float)sz.y, zsum[h][j]);
+                    qs[h] = xv[h] * (float)sz.x;
+                }
+                accumulate_heads<3, NREP>(&cw[u].v[j], qs, acc[j]);
             }
         }
     };
@@ -611,35 +639,38 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols3(GemvArgs a)
         }
     }
 
-    // ---- combine the RQ row sections, store fp16 ----
+    // ---- combine the RQ row sections, store fp16 (2^59 undoes the fp32-subnormal scaling) ----
     constexpr int TOT = UPL * VALS;  // consecutive outputs of this lane
-    float *flat = &acc[0][0];
 #pragma unroll
-    for (int j = 0; j < UPL; j++) {
+    for (int h = 0; h < NREP; h++) {
+        float flat[TOT];
 #pragma unroll
-        for (int i = 0; i < VALS; i++) acc[j][i] = fmaf(acc[j][i], Fmt<3>::OUT_SCALE, zsum[j]);
-    }
-    uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
-    if constexpr (RQ == 1) {
+        for (int j = 0; j < UPL; j++) {
 #pragma unroll
-        for (int e = 0; e < TOT; e += 2) {
-            const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
-            __builtin_memcpy(op + e, &pk, 4);
+            for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], kHeadsOutScale, zsum[h][j]);
         }
-    } else {
-        // halving butterfly: each section ends with its share of the sums (TOT / RQ each)
-        static_assert(RQ == 2 && TOT % 2 == 0, "two sections, equal shares");
-        const int first = scatter_reduce<TOT, GL, 1>(flat, lane);
-        constexpr int PER = TOT / RQ;
-        if constexpr (PER % 2 == 0) {
+        uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + (sample0 + h) * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
+        if constexpr (RQ == 1) {
 #pragma unroll
-            for (int e = 0; e < PER; e += 2) {
+            for (int e = 0; e < TOT; e += 2) {
                 const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
-                __builtin_memcpy(op + first + e, &pk, 4);
+                __builtin_memcpy(op + e, &pk, 4);
             }
         } else {
+            // halving butterfly: each section ends with its share of the sums (TOT / RQ each)
+            static_assert(RQ == 2 && TOT % 2 == 0, "two sections, equal shares");
+            const int first = scatter_reduce<TOT, GL, 1>(flat, lane);
+            constexpr int PER = TOT / RQ;
+            if constexpr (PER % 2 == 0) {
 #pragma unroll
-            for (int e = 0; e < PER; e++) op[first + e] = f32_to_h16(flat[e]);
+                for (int e = 0; e < PER; e += 2) {
+                    const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
+                    __builtin_memcpy(op + first + e, &pk, 4);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < PER; e++) op[first + e] = f32_to_h16(flat[e]);
+            }
         }
     }
 }
@@ -1617,7 +1648,7 @@ static int64_t cols_min_units()
 #define KVMIX_COLS3_U 8
 #endif
 
-template <int RQ, int UPL>
+template <int RQ, int UPL, int NREP>
 static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
 {
     constexpr int TU = (kWave / RQ) * UPL;
@@ -1633,9 +1664,10 @@ static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
         }
     }
     if (tiles < wpb) wpb = (int)tiles;
-    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL((gemv_cols3<RQ, UPL, KVMIX_COLS3_U>), grid, dim3(kWave, wpb),
-                       sizeof(float) * (size_t)(a.K + 1), st, a);
+    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
+    constexpr int U = NREP > 1 ? KVMIX_COLS3_HEADS_U : KVMIX_COLS3_U;  // rows in flight per lane
+    hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, wpb),
+                       sizeof(float) * (size_t)NREP * (size_t)(a.K + 1), st, a);
 }
 
 // (gemv_cols_mfma: whole 512-code tiles, at least one whole 32-row chunk)
@@ -1696,12 +1728,14 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // words per wave) that still gives the chip enough waves and fits into N
         const int64_t units = a.N / 11, batch = samples * a.M;
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
-        if (units >= 256 && waves(256) >= kTargetWaves)
-            launch_cols3_cfg<1, 4>(a, samples, st);
+        if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
+            launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
+        else if (units >= 256 && waves(256) >= kTargetWaves)
+            launch_cols3_cfg<1, 4, 1>(a, samples, st);
         else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
-            launch_cols3_cfg<2, 4>(a, samples, st);
+            launch_cols3_cfg<2, 4, 1>(a, samples, st);
         else
-            launch_cols3_cfg<2, 2>(a, samples, st);
+            launch_cols3_cfg<2, 2, 1>(a, samples, st);
     } else {
     // more row sections per wave = more, narrower waves: take the widest tile that still
     // gives the chip enough waves and fits into N

@@ -77,6 +77,17 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
     run_case(oracle, dev, bits, g, B=1, nh=4, nkv=4, K=777, N=128, seed=45, M=2)
 
 
+def test_reference_3bit_kernel_edges(oracle, dev):
+    """gemv_cols3: four and two words per lane, GQA head groups (four query heads per pass), K ragged
+    against the 8-row rotation, N ragged against the tile, M = 2."""
+    run_case(oracle, dev, 3, 11, B=1, nh=8, nkv=2, K=128, N=11 * 150, seed=51)   # GQA, 4 heads per block
+    run_case(oracle, dev, 3, 11, B=1, nh=6, nkv=2, K=128, N=11 * 70, seed=52)    # GQA, heads one by one
+    run_case(oracle, dev, 3, 11, B=2, nh=2, nkv=2, K=77, N=11 * 300, seed=53)    # K = 77: ragged sections
+    run_case(oracle, dev, 3, 11, B=1, nh=8, nkv=2, K=50, N=11 * 64, seed=54)     # smallest fast tile, GQA
+    run_case(oracle, dev, 3, 11, B=1, nh=2, nkv=2, K=128, N=11 * 131, seed=55, M=2)
+    run_case(oracle, dev, 3, 11, B=8, nh=8, nkv=8, K=128, N=11 * 733, seed=56)   # wide tiles (4 words per lane)
+
+
 @pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
 def test_generic_shapes(oracle, dev, bits, g):
     """Group sizes and shapes outside the fast kernels (including a 3-bit p.V shape)."""
