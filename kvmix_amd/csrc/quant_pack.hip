@@ -133,85 +133,109 @@ __global__ void __launch_bounds__(256) quant_rows_generic(QuantArgs a, int unit,
 // fast path: fp16, group 32, 4 lanes per group, 8 halves (one 128-bit load) per lane.
 // BITS = 1, 2, 4 (reference layout) or 3 with DENSE3 = true (bit-stream extension).
 // ---------------------------------------------------------------------------------------
-template <int BITS>
+// A thread handles P pieces (P*256 threads apart, so every load instruction of a wave is one
+// contiguous kilobyte): the P loads are issued first, then the pieces are processed one by one.
+// With one piece per thread the kernel is bound by wave turnover (one load latency per wave
+// lifetime); with several it streams.  IDX32: the group index fits 32 bits (no 64-bit divisions).
+template <int BITS, int P, bool IDX32>
 __device__ __forceinline__ void rows_g32_f16_body(const QuantArgs &a, int64_t groups_per_row,
-                                                  int64_t total_groups, int64_t tid)
+                                                  int64_t total_groups, int64_t first_tid)
 {
-    int64_t g = tid >> 2;
-    const int j = (int)(tid & 3);
-    const bool active = g < total_groups;
-    if (!active) g = total_groups - 1;  // keep the quad's shuffles convergent
-    const int64_t row = g / groups_per_row;
-    const int64_t gr = g - row * groups_per_row;
-    const int64_t o = row / a.inner;
-    const int64_t i = row - o * a.inner;
-    const __half *x = (const __half *)a.x + o * a.x_os + i * a.x_is + gr * 32 + j * 8;
-
-    const uint4 raw = *reinterpret_cast<const uint4 *>(x);
-    float v[8];
-    {
-        const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+    const int j = (int)(first_tid & 3);
+    bool active[P];
+    int64_t o[P], i[P], gr[P];
+    uint4 raw[P];
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            v[2 * t] = h16_to_f32((uint16_t)(r[t] & 0xffffu));
-            v[2 * t + 1] = h16_to_f32((uint16_t)(r[t] >> 16));
+    for (int p = 0; p < P; p++) {
+        int64_t g = (first_tid + (int64_t)p * 256) >> 2;
+        active[p] = g < total_groups;
+        if (!active[p]) g = total_groups - 1;  // keep the quad's shuffles convergent
+        if constexpr (IDX32) {
+            const uint32_t g32 = (uint32_t)g, gpr = (uint32_t)groups_per_row, inner = (uint32_t)a.inner;
+            const uint32_t row = g32 / gpr;
+            gr[p] = g32 - row * gpr;
+            o[p] = row / inner;
+            i[p] = row - (uint32_t)o[p] * inner;
+        } else {
+            const int64_t row = g / groups_per_row;
+            gr[p] = g - row * groups_per_row;
+            o[p] = row / a.inner;
+            i[p] = row - o[p] * a.inner;
         }
+        const __half *x = (const __half *)a.x + o[p] * a.x_os + i[p] * a.x_is + gr[p] * 32 + j * 8;
+        raw[p] = *reinterpret_cast<const uint4 *>(x);
     }
-    float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-        mn = fminf(mn, v[t]);
-        mx = fmaxf(mx, v[t]);
-    }
-    mn = fminf(mn, __shfl_xor(mn, 1));
-    mx = fmaxf(mx, __shfl_xor(mx, 1));
-    mn = fminf(mn, __shfl_xor(mn, 2));
-    mx = fmaxf(mx, __shfl_xor(mx, 2));
-
-    constexpr int qmax = (1 << BITS) - 1;
-    const float range = mx - mn;
-    const float scale = range / (float)qmax;
-    uint32_t piece = 0;  // this lane's 8 codes, 8*BITS bits
+    for (int p = 0; p < P; p++) {
+        float v[8];
+        {
+            const uint32_t r[4] = {raw[p].x, raw[p].y, raw[p].z, raw[p].w};
 #pragma unroll
-    for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, qmax) << (t * BITS);
+            for (int t = 0; t < 4; t++) {
+                v[2 * t] = h16_to_f32((uint16_t)(r[t] & 0xffffu));
+                v[2 * t + 1] = h16_to_f32((uint16_t)(r[t] >> 16));
+            }
+        }
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            mn = fminf(mn, v[t]);
+            mx = fmaxf(mx, v[t]);
+        }
+        mn = fminf(mn, __shfl_xor(mn, 1));
+        mx = fmaxf(mx, __shfl_xor(mx, 1));
+        mn = fminf(mn, __shfl_xor(mn, 2));
+        mx = fmaxf(mx, __shfl_xor(mx, 2));
 
-    uint32_t *cw = a.code + o * a.c_os + i * a.c_is + gr * BITS;  // BITS words per group of 32
-    if (BITS == 4) {
-        if (active) cw[j] = piece;
-    } else if (BITS == 2) {
-        const uint32_t other = __shfl_xor(piece, 1);
-        if (active && (j & 1) == 0) cw[j >> 1] = piece | (other << 16);
-    } else if (BITS == 1) {
-        uint32_t w = piece << (8 * j);
-        w |= __shfl_xor(w, 1);
-        w |= __shfl_xor(w, 2);
-        if (active && j == 0) cw[0] = w;
-    } else {  // BITS == 3, bit stream: lane j holds stream bits [24j, 24j+24)
-        const uint32_t next = __shfl_down(piece, 1);  // lane j+1's piece (unused for j == 3)
-        uint32_t w;
-        if (j == 0)
-            w = piece | (next << 24);
-        else if (j == 1)
-            w = (piece >> 8) | (next << 16);
-        else
-            w = (piece >> 16) | (next << 8);
-        if (active && j < 3) cw[j] = w;
-    }
-    if (active && j == 0) {
-        __half *sc = (__half *)a.scale + o * a.s_os + i * a.s_is + gr;
-        *sc = __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
-    }
-    if (active && j == 1) {
-        __half *zr = (__half *)a.zero + o * a.s_os + i * a.s_is + gr;
-        *zr = __float2half_rn(mn);
+        constexpr int qmax = (1 << BITS) - 1;
+        const float range = mx - mn;
+        const float scale = range / (float)qmax;
+        uint32_t piece = 0;  // this lane's 8 codes, 8*BITS bits
+#pragma unroll
+        for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, qmax) << (t * BITS);
+
+        const bool act = active[p];
+        uint32_t *cw = a.code + o[p] * a.c_os + i[p] * a.c_is + gr[p] * BITS;  // BITS words per group of 32
+        if (BITS == 4) {
+            if (act) cw[j] = piece;
+        } else if (BITS == 2) {
+            const uint32_t other = __shfl_xor(piece, 1);
+            if (act && (j & 1) == 0) cw[j >> 1] = piece | (other << 16);
+        } else if (BITS == 1) {
+            uint32_t w = piece << (8 * j);
+            w |= __shfl_xor(w, 1);
+            w |= __shfl_xor(w, 2);
+            if (act && j == 0) cw[0] = w;
+        } else {  // BITS == 3, bit stream: lane j holds stream bits [24j, 24j+24)
+            const uint32_t next = __shfl_down(piece, 1);  // lane j+1's piece (unused for j == 3)
+            uint32_t w;
+            if (j == 0)
+                w = piece | (next << 24);
+            else if (j == 1)
+                w = (piece >> 8) | (next << 16);
+            else
+                w = (piece >> 16) | (next << 8);
+            if (act && j < 3) cw[j] = w;
+        }
+        if (act && j == 0) {
+            __half *sc = (__half *)a.scale + o[p] * a.s_os + i[p] * a.s_is + gr[p];
+            *sc = __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+        }
+        if (act && j == 1) {
+            __half *zr = (__half *)a.zero + o[p] * a.s_os + i[p] * a.s_is + gr[p];
+            *zr = __float2half_rn(mn);
+        }
     }
 }
 
-template <int BITS>
+constexpr int kRowsPieces = 4;  // pieces per thread in the streaming configuration
+
+template <int BITS, int P, bool IDX32>
 __global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t groups_per_row,
                                                           int64_t total_groups)
 {
-    rows_g32_f16_body<BITS>(a, groups_per_row, total_groups, (int64_t)blockIdx.x * blockDim.x + threadIdx.x);
+    rows_g32_f16_body<BITS, P, IDX32>(a, groups_per_row, total_groups,
+                                      (int64_t)blockIdx.x * (256 * P) + threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -305,10 +329,10 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
     } else {
         const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * 256 + threadIdx.x;
         switch (va.bits) {
-        case 1: rows_g32_f16_body<1>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3>(va, v_groups_per_row, v_total_groups, tid); break;
-        default: rows_g32_f16_body<4>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 1: rows_g32_f16_body<1, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        default: rows_g32_f16_body<4, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
         }
     }
 }
@@ -405,13 +429,33 @@ static int launch_last_dim(const QuantArgs &a, int x_dtype, int vpw, bool fast, 
     if (fast) {
         const int64_t total_groups = a.outer * a.inner * groups;
         const int64_t threads = total_groups * 4;
-        const unsigned blocks = (unsigned)((threads + 255) / 256);
+        // large inputs stream with several pieces per thread; small ones keep one (more waves)
+        const bool many = threads >= (int64_t)256 * kRowsPieces * 2048;
+        const bool idx32 = total_groups < (1ll << 30);
+        const int64_t per_block = 256 * (many ? kRowsPieces : 1);
+        const unsigned blocks = (unsigned)((threads + per_block - 1) / per_block);
+#define KVMIX_ROWS_LAUNCH(B_)                                                                                         \
+    do {                                                                                                              \
+        if (many && idx32)                                                                                            \
+            hipLaunchKernelGGL((quant_rows_g32_f16<B_, kRowsPieces, true>), dim3(blocks), dim3(256), 0, st, a, groups, \
+                               total_groups);                                                                         \
+        else if (many)                                                                                                \
+            hipLaunchKernelGGL((quant_rows_g32_f16<B_, kRowsPieces, false>), dim3(blocks), dim3(256), 0, st, a,       \
+                               groups, total_groups);                                                                 \
+        else if (idx32)                                                                                               \
+            hipLaunchKernelGGL((quant_rows_g32_f16<B_, 1, true>), dim3(blocks), dim3(256), 0, st, a, groups,          \
+                               total_groups);                                                                         \
+        else                                                                                                          \
+            hipLaunchKernelGGL((quant_rows_g32_f16<B_, 1, false>), dim3(blocks), dim3(256), 0, st, a, groups,         \
+                               total_groups);                                                                         \
+    } while (0)
         switch (a.bits) {
-        case 1: hipLaunchKernelGGL(quant_rows_g32_f16<1>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
-        case 2: hipLaunchKernelGGL(quant_rows_g32_f16<2>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
-        case 3: hipLaunchKernelGGL(quant_rows_g32_f16<3>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
-        default: hipLaunchKernelGGL(quant_rows_g32_f16<4>, dim3(blocks), dim3(256), 0, st, a, groups, total_groups); break;
+        case 1: KVMIX_ROWS_LAUNCH(1); break;
+        case 2: KVMIX_ROWS_LAUNCH(2); break;
+        case 3: KVMIX_ROWS_LAUNCH(3); break;
+        default: KVMIX_ROWS_LAUNCH(4); break;
         }
+#undef KVMIX_ROWS_LAUNCH
         return launch_status();
     }
     // generic path: a thread owns lcm(group, codes per word) values, i.e. whole groups and whole words
