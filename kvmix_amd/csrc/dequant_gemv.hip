@@ -1641,6 +1641,9 @@ static int64_t cols_min_units()
     return MODE == 3 ? 64 : 16 * ColsUpl<MODE>::value;
 }
 
+#ifndef KVMIX_COLS3_WIDE_WAVES
+#define KVMIX_COLS3_WIDE_WAVES 4096
+#endif
 #ifndef KVMIX_COLS3_MIN_WAVES
 #define KVMIX_COLS3_MIN_WAVES 2048
 #endif
@@ -1730,7 +1733,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
         if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
-        else if (units >= 256 && waves(256) >= kTargetWaves)
+        else if (units >= 256 && waves(256) >= KVMIX_COLS3_WIDE_WAVES)
             launch_cols3_cfg<1, 4, 1>(a, samples, st);
         else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
             launch_cols3_cfg<2, 4, 1>(a, samples, st);
