@@ -11,25 +11,22 @@
 // term is one fma per (k, group) instead of one per element, and the first needs no
 // int->float conversion (see mix2 below).  All accumulation is fp32.
 //
-// Memory plan (the kernels are HBM-bound; measured on MI355X, 2-byte loads of scale/zero
-// issued per lane cost a third of the run time, so they never happen):
-//   * packed codes: one 128/64/32-bit load per lane and row, straight to registers;
-//   * scale, zero and x: fetched with 128-bit loads by whichever lane the address falls to,
-//     combined (x*scale, or (scale, zero) pairs) and parked in a wave-private LDS tile, from
-//     which the consuming lane reads one dword per row.  Wave-private means no block barrier
-//     in the streaming loop.
+// Kernels (each documented where it is defined)
+//   gemv_rows_mfma  p.V (K = tokens large, N = 128), 1/2/4-bit and dense 3-bit: matrix cores.
+//   gemv_cols_mfma  q.K^T (K = head_dim small, N = tokens large), 1/2/4-bit: matrix cores; used
+//                   for GQA and for problems too small for gemv_cols' wide tiles.
+//   gemv_cols3      q.K^T, the reference's 3-bit format: register streaming, vector ALU.
+//   gemv_cols       q.K^T, 1/2/4-bit and dense 3-bit: vector ALU, (scale, zero) staged in LDS.
+//   gemv_rows       p.V for N = 64 / 256 or strided code rows: vector ALU.
+//   gemv_generic    any shape/group: one thread per packed word, serial over K.
+//   reduce_splits   sums the split-K partials of the p.V kernels and stores fp16.
 //
-// Kernels
-//   gemv_cols   q.K^T shape (K = head_dim small, N = tokens large).  A lane owns one
-//               quantization group of N (32 codes, or one 11-code word of the reference's
-//               3-bit format) for a quarter / half / all of the K rows (RQ = 4 / 2 / 1 row
-//               sections per wave); the sections meet in a butterfly over lanes at the end.
-//   gemv_rows   p.V shape (K = tokens large, N = head_dim small).  A lane owns one group of
-//               one row; a wave walks a contiguous chunk of rows, 8 row tiles in flight.
-//               Butterfly across the row lanes, LDS across waves, optional split-K across
-//               blocks with fp32 partials in the caller's workspace.
-//   gemv_generic  any shape/group: one thread per packed word, serial over K.
-//   reduce_splits sums the split-K partials and stores fp16.
+// Common rules of the streaming kernels (measured on MI355X): scale/zero never by 2-byte loads
+// per lane (they cost a third of the run time) but by 128-bit loads of whichever lane the
+// address falls to, handed on through a wave-private LDS tile (no block barrier in the stream);
+// every load unconditional, in one fixed order from the first iteration on, and pinned with
+// scheduling barriers -- otherwise the compiler sinks the prefetch loads to the end of the loop
+// body and every iteration starts by draining the load queue.
 
 #include "kvmix_common.h"
 
@@ -43,7 +40,7 @@
 #define KVMIX_COLS_MFMA 1  // 1/2/4-bit q.K^T on the matrix cores
 #endif
 #ifndef KVMIX_ROWS_MFMA
-#define KVMIX_ROWS_MFMA 1  // 4-bit p.V on the matrix cores
+#define KVMIX_ROWS_MFMA 1  // 1/2/4-bit and dense 3-bit p.V on the matrix cores
 #endif
 
 #ifndef KVMIX_HEADS_WAVE_DIV
@@ -1557,8 +1554,7 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
     a.splits = p.splits;
     a.rows_per_split = p.rows_per_split;
     const dim3 grid((unsigned)a.splits, (unsigned)(samples / NREP), (unsigned)a.M), block(kWave, p.waves);
-    {
-      if (mfma) {
+    if (mfma) {
         // one A tile per wave and MFMA set; the block reduction (waves*NREP*128 floats) reuses it
         const size_t lds = (size_t)p.waves * rows_mfma_sets(NREP) * kRowsMfmaTile * sizeof(uint16_t);
         constexpr int DEPTH = 1;  // chunks in flight per wave (deeper costs occupancy and was slower)
@@ -1578,7 +1574,6 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
             hipLaunchKernelGGL(reduce_splits, g2, dim3(256), 0, st, a);
         }
         return;
-      }
     }
     const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)NREP * (size_t)(512 + a.N);
     switch (a.N / 32) {
@@ -1605,6 +1600,23 @@ static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
 #define KVMIX_COLS_RQ 0  // 0 = choose by problem size
 #endif
 
+// waves per block for a kernel whose waves each take one of `slots` tiles of an output row:
+// the count (2..4) that leaves the fewest launched waves without a tile
+static int pick_waves_per_block(int64_t slots)
+{
+    int wpb = kColsWaves;
+    int64_t idle = (slots + wpb - 1) / wpb * wpb - slots;
+    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
+        const int64_t i = (slots + w - 1) / w * w - slots;
+        if (i < idle) {
+            idle = i;
+            wpb = w;
+        }
+    }
+    return slots < wpb ? (int)slots : wpb;
+}
+
+
 // units one lane owns in gemv_cols: enough for a 128-bit code load per lane and row
 template <int MODE>
 struct ColsUpl {
@@ -1618,17 +1630,7 @@ static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / VALS;
     const int64_t tiles = (units + TU - 1) / TU;
-    // waves per block: the count (2..4) that leaves the fewest waves without a tile
-    int wpb = kColsWaves;
-    int64_t idle = (tiles + wpb - 1) / wpb * wpb - tiles;
-    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
-        const int64_t i = (tiles + w - 1) / w * w - tiles;
-        if (i < idle) {
-            idle = i;
-            wpb = w;
-        }
-    }
-    if (tiles < wpb) wpb = (int)tiles;
+    const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
     hipLaunchKernelGGL((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, wpb), 0, st, a);
 }
@@ -1657,16 +1659,7 @@ static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / 11;
     const int64_t tiles = (units + TU - 1) / TU;
-    int wpb = kColsWaves;  // waves per block: the count (2..4) that leaves the fewest waves idle
-    int64_t idle = (tiles + wpb - 1) / wpb * wpb - tiles;
-    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
-        const int64_t i = (tiles + w - 1) / w * w - tiles;
-        if (i < idle) {
-            idle = i;
-            wpb = w;
-        }
-    }
-    if (tiles < wpb) wpb = (int)tiles;
+    const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
     constexpr int U = NREP > 1 ? KVMIX_COLS3_HEADS_U : KVMIX_COLS3_U;  // rows in flight per lane
     hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, wpb),
@@ -1690,16 +1683,7 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     int64_t tpw = batch * tiles / target;
     tpw = tpw < 1 ? 1 : (tpw > 8 ? 8 : tpw);
     const int64_t slots = (tiles + tpw - 1) / tpw;  // waves per output row
-    int wpb = kColsWaves;
-    int64_t idle = (slots + wpb - 1) / wpb * wpb - slots;
-    for (int w = kColsWaves - 1; w >= 2 && idle > 0; w--) {
-        const int64_t i = (slots + w - 1) / w * w - slots;
-        if (i < idle) {
-            idle = i;
-            wpb = w;
-        }
-    }
-    if (slots < wpb) wpb = (int)slots;
+    const int wpb = pick_waves_per_block(slots);
     a.splits = (int)tpw;
     const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
     const size_t lds = (size_t)wpb * (rows_mfma_sets(NREP) * kColsMfmaTile * sizeof(uint16_t) + NREP * 16 * sizeof(float));
