@@ -346,6 +346,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-target-shape", action="store_true")
+    ap.add_argument("--shapes-only", action="store_true",
+                    help="skip the step: only the B=16/T=8192 target shape and the GQA configuration (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 1 GiB device copies (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
@@ -362,6 +364,18 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, D, T, R = args.batch, 32, 128, args.context, 128
+    if args.shapes_only:
+        if args.copy_calibration:
+            src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
+        st = torch.cuda.current_stream().cuda_stream
+        print(json.dumps({"target_shape_B16_T8192": target_shape_extra(torch, _lib, lib, dev, st),
+                          "gqa_config2_B16_T32768": gqa_shape_extra(torch, _lib, lib, dev, st)}))
+        return
     kbits, vbits = layer_bits(args.layers)
     layers = build_layers(torch, ops, lib, B, H, D, T, R, kbits, vbits, dev)
     torch.cuda.synchronize()
