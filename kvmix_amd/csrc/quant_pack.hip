@@ -239,6 +239,61 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t g
 }
 
 // ---------------------------------------------------------------------------------------
+// reference 3-bit format, fp16 rows: one thread per 11-code word (= one group of 11 values,
+// 22 bytes at 2-byte alignment, fetched with three vector loads), P words per thread with the
+// loads issued first.  WRAP: the append-V "placeholder" packing (11th code quantized to 0..7,
+// low two bits kept).
+// ---------------------------------------------------------------------------------------
+struct __attribute__((packed, aligned(2))) Half11 {
+    uint16_t v[11];
+};
+
+template <int P, bool WRAP>
+__global__ void __launch_bounds__(256) quant_rows_ref3_f16(QuantArgs a, uint32_t words_per_row, int64_t total_words)
+{
+    const int64_t first = (int64_t)blockIdx.x * (256 * P) + threadIdx.x;
+    Half11 raw[P];
+    int64_t o[P], i[P];
+    uint32_t wr[P];
+    bool active[P];
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        int64_t w = first + (int64_t)p * 256;
+        active[p] = w < total_words;
+        if (!active[p]) w = total_words - 1;
+        const int64_t row = w / words_per_row;  // (64-bit: the word count may exceed 2^32)
+        wr[p] = (uint32_t)(w - row * words_per_row);
+        o[p] = row / a.inner;
+        i[p] = row - o[p] * a.inner;
+        const __half *x = (const __half *)a.x + o[p] * a.x_os + i[p] * a.x_is + (int64_t)wr[p] * 11;
+        raw[p] = *reinterpret_cast<const Half11 *>(x);
+    }
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        float v[11];
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+#pragma unroll
+        for (int t = 0; t < 11; t++) {
+            v[t] = h16_to_f32(raw[p].v[t]);
+            mn = fminf(mn, v[t]);
+            mx = fmaxf(mx, v[t]);
+        }
+        const float range = mx - mn;
+        const float scale = range / 7.0f;
+        uint32_t word = 0;
+#pragma unroll
+        for (int t = 0; t < 10; t++) word |= quantize_code(v[t], mn, scale, 7) << (3 * t);
+        word |= (quantize_code(v[10], mn, scale, WRAP ? 7 : 3) & 3u) << 30;
+        if (active[p]) {
+            a.code[o[p] * a.c_os + i[p] * a.c_is + wr[p]] = word;
+            ((__half *)a.scale)[o[p] * a.s_os + i[p] * a.s_is + wr[p]] =
+                __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+            ((__half *)a.zero)[o[p] * a.s_os + i[p] * a.s_is + wr[p]] = __float2half_rn(mn);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // keys from the token-major tail: k [outer, n, D] -> code [outer, D, n/vpw], groups of G
 // tokens per channel.  One thread per channel, one block row per (group, outer).
 // MODE: 1, 2, 4 = reference layout bits; 3 = reference 3-bit (G must be 11); 30 = dense 3-bit.
@@ -457,6 +512,17 @@ static int launch_last_dim(const QuantArgs &a, int x_dtype, int vpw, bool fast, 
         }
 #undef KVMIX_ROWS_LAUNCH
         return launch_status();
+    }
+    if (x_dtype == KVMIX_F16 && a.bits == 3 && a.fmt != KVMIX_FMT_DENSE3 && a.group == 11) {
+        const int64_t wpr = a.steps / 11, total = a.outer * a.inner * wpr;
+        if (wpr < (1ll << 31)) {
+            const unsigned blocks = (unsigned)((total + 256 * 2 - 1) / (256 * 2));
+            if (a.fmt == KVMIX_FMT_REF3_WRAP)
+                hipLaunchKernelGGL((quant_rows_ref3_f16<2, true>), dim3(blocks), dim3(256), 0, st, a, (uint32_t)wpr, total);
+            else
+                hipLaunchKernelGGL((quant_rows_ref3_f16<2, false>), dim3(blocks), dim3(256), 0, st, a, (uint32_t)wpr, total);
+            return launch_status();
+        }
     }
     // generic path: a thread owns lcm(group, codes per word) values, i.e. whole groups and whole words
     const int64_t word_span = vpw ? vpw : 32;
