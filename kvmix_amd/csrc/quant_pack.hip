@@ -20,6 +20,10 @@
 
 #include "kvmix_common.h"
 
+#ifndef KVMIX_QUANT_STREAM
+#define KVMIX_QUANT_STREAM 1
+#endif
+
 namespace kvmix {
 
 struct QuantArgs {
@@ -236,6 +240,74 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t g
 {
     rows_g32_f16_body<BITS, P, IDX32>(a, groups_per_row, total_groups,
                                       (int64_t)blockIdx.x * (256 * P) + threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------------------
+// large inputs, fp16, group 32: one thread per group (four 128-bit loads, no lane exchange),
+// P groups per thread with the loads issued first; codes leave as one vector store per group.
+// ---------------------------------------------------------------------------------------
+template <int BITS, int P>
+__global__ void __launch_bounds__(256) quant_rows_g32_f16_stream(QuantArgs a, uint32_t groups_per_row,
+                                                                 int64_t total_groups)
+{
+    const int64_t first = (int64_t)blockIdx.x * (256 * P) + threadIdx.x;
+    uint4 raw[P][4];
+    int64_t o[P], i[P];
+    uint32_t gr[P];
+    bool active[P];
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        int64_t g = first + (int64_t)p * 256;
+        active[p] = g < total_groups;
+        if (!active[p]) g = total_groups - 1;
+        const int64_t row = g / groups_per_row;
+        gr[p] = (uint32_t)(g - row * groups_per_row);
+        o[p] = row / a.inner;
+        i[p] = row - o[p] * a.inner;
+        const uint4 *x = reinterpret_cast<const uint4 *>((const __half *)a.x + o[p] * a.x_os + i[p] * a.x_is + (int64_t)gr[p] * 32);
+#pragma unroll
+        for (int q = 0; q < 4; q++) raw[p][q] = x[q];
+    }
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        float v[32];
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t r[4] = {raw[p][q].x, raw[p][q].y, raw[p][q].z, raw[p][q].w};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                v[8 * q + 2 * t] = h16_to_f32((uint16_t)(r[t] & 0xffffu));
+                v[8 * q + 2 * t + 1] = h16_to_f32((uint16_t)(r[t] >> 16));
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 32; t++) {
+            mn = fminf(mn, v[t]);
+            mx = fmaxf(mx, v[t]);
+        }
+        constexpr int qmax = (1 << BITS) - 1;
+        const float range = mx - mn;
+        const float scale = range / (float)qmax;
+        uint32_t w[BITS];
+#pragma unroll
+        for (int t = 0; t < BITS; t++) w[t] = 0;
+#pragma unroll
+        for (int t = 0; t < 32; t++) {
+            const uint32_t q = quantize_code(v[t], mn, scale, qmax);
+            const int bit = t * BITS;
+            w[bit >> 5] |= q << (bit & 31);
+            if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+        }
+        if (active[p]) {
+            uint32_t *cw = a.code + o[p] * a.c_os + i[p] * a.c_is + (int64_t)gr[p] * BITS;
+#pragma unroll
+            for (int t = 0; t < BITS; t++) cw[t] = w[t];
+            ((__half *)a.scale)[o[p] * a.s_os + i[p] * a.s_is + gr[p]] =
+                __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+            ((__half *)a.zero)[o[p] * a.s_os + i[p] * a.s_is + gr[p]] = __float2half_rn(mn);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -483,6 +555,16 @@ static int launch_last_dim(const QuantArgs &a, int x_dtype, int vpw, bool fast, 
     const int64_t groups = a.steps / a.group;
     if (fast) {
         const int64_t total_groups = a.outer * a.inner * groups;
+        if (KVMIX_QUANT_STREAM && total_groups >= (int64_t)256 * 2 * 4096 && groups < (1ll << 31)) {
+            const unsigned nb = (unsigned)((total_groups + 511) / 512);
+            switch (a.bits) {
+            case 1: hipLaunchKernelGGL((quant_rows_g32_f16_stream<1, 2>), dim3(nb), dim3(256), 0, st, a, (uint32_t)groups, total_groups); break;
+            case 2: hipLaunchKernelGGL((quant_rows_g32_f16_stream<2, 2>), dim3(nb), dim3(256), 0, st, a, (uint32_t)groups, total_groups); break;
+            case 3: hipLaunchKernelGGL((quant_rows_g32_f16_stream<3, 2>), dim3(nb), dim3(256), 0, st, a, (uint32_t)groups, total_groups); break;
+            default: hipLaunchKernelGGL((quant_rows_g32_f16_stream<4, 2>), dim3(nb), dim3(256), 0, st, a, (uint32_t)groups, total_groups); break;
+            }
+            return launch_status();
+        }
         const int64_t threads = total_groups * 4;
         // large inputs stream with several pieces per thread; small ones keep one (more waves)
         const bool many = threads >= (int64_t)256 * kRowsPieces * 2048;

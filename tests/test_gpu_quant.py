@@ -226,3 +226,27 @@ def test_full_size_flush_properties(dev):
         deq = scale.float().unsqueeze(-1) * q + mn.float().unsqueeze(-1)
         bound = scale.float().unsqueeze(-1) * 0.5 + 2.0 ** -10 * (mn.float().abs().unsqueeze(-1) + qmax * scale.float().unsqueeze(-1))
         assert ((deq - xg).abs() <= bound).all()
+
+
+@pytest.mark.parametrize("bits", [4, 2, 1, 3])
+def test_prompt_size_inputs_take_the_streaming_kernels(oracle, dev, bits):
+    """Inputs of prompt size (2 M groups and more) go through the one-thread-per-group kernels;
+    bits = 3 covers both the dense stream (group 32) and the reference format (group 11, fp16)."""
+    import KVmix
+    from kvmix_amd import ops
+
+    rng = np.random.default_rng(bits)
+    x = kv_like(rng, (4, 8, 2048 * 4 + 3, 256)).astype(np.float16)  # 2 098 944 groups of 32, rows not a block multiple
+    xt = torch.from_numpy(x).to(dev)
+    if bits == 3:
+        code, scale, mn = ops.quantize_pack_dense3(xt, 32)
+        oc, osc, omn = oracle.quantize_pack_dense3(x, 32)
+    else:
+        code, scale, mn = KVmix.quantize_pack_last_dim_cuda(xt, 32, bits)
+        oc, osc, omn = oracle.quantize_pack_last_dim(x, 32, bits)
+    assert same_bits(code.cpu().numpy(), oc) and same_bits(scale.cpu().numpy(), osc) and same_bits(mn.cpu().numpy(), omn)
+    if bits == 3:
+        x11 = np.ascontiguousarray(x[..., :253])  # 23 words per row: odd row length, 2-byte aligned rows
+        code, scale, mn = KVmix.quantize_pack_last_dim_cuda(torch.from_numpy(x11).to(dev), 11, 3)
+        oc, osc, omn = oracle.quantize_pack_last_dim(x11, 11, 3)
+        assert same_bits(code.cpu().numpy(), oc) and same_bits(scale.cpu().numpy(), osc) and same_bits(mn.cpu().numpy(), omn)
