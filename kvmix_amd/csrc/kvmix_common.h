@@ -36,6 +36,31 @@ __device__ __forceinline__ uint32_t quantize_code(float x, float mn, float scale
     return (uint32_t)q;
 }
 
+// The same code without a division per element.  rcp approximates 1/scale (v_rcp_f32, 1 ulp), so
+// t = (x - mn) * rcp is within a few ulp of the true quotient -- for quotients up to 15 that is
+// below 1e-5 -- and the IEEE quotient rounds to the same integer as t unless t lies within that
+// distance of a tie k + 0.5.  Only then (margin 2^-12), or when t is not an ordinary number
+// (constant group: 0 * inf), the exact path runs.  Bit-identical to quantize_code.
+// rcp for the division-free quantize_code below; NaN (= always take the exact path) when the
+// scale is so small or large that the reciprocal leaves the range where v_rcp_f32 is 1 ulp
+__device__ __forceinline__ float quantize_rcp(float scale)
+{
+    return (scale > 1e-30f && scale < 1e30f) ? __builtin_amdgcn_rcpf(scale) : __builtin_nanf("");
+}
+
+__device__ __forceinline__ uint32_t quantize_code(float x, float mn, float scale, float rcp, int hi)
+{
+    const float t = (x - mn) * rcp;
+    const float fl = floorf(t);
+    const float fr = t - fl;
+    if (__builtin_expect(!(fabsf(fr - 0.5f) >= 0.000244140625f) || !(fabsf(t) < 1024.0f), 0))
+        return quantize_code(x, mn, scale, hi);
+    int q = (int)fl + (fr > 0.5f ? 1 : 0);
+    q = q > hi ? hi : q;
+    q = q < 0 ? 0 : q;
+    return (uint32_t)q;
+}
+
 // scale returned to the caller; the codes always use the true division.
 __device__ __forceinline__ float scale_for_output(float range, float scale_div, float inv_qmax, int scale_mode)
 {

@@ -20,6 +20,12 @@
 
 #include "kvmix_common.h"
 
+#ifndef KVMIX_FLUSH_K_TILED
+#define KVMIX_FLUSH_K_TILED 1
+#endif
+#ifndef KVMIX_FLUSH_V_PIECES
+#define KVMIX_FLUSH_V_PIECES 1
+#endif
 #ifndef KVMIX_QUANT_STREAM
 #define KVMIX_QUANT_STREAM 1
 #endif
@@ -106,12 +112,13 @@ __global__ void __launch_bounds__(256) quant_rows_generic(QuantArgs a, int unit,
         }
         const float range = mx - mn;
         const float scale = range / (float)qmax;
+        const float rcp = quantize_rcp(scale);
         store_from_float<T>(sc + g, scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
         store_from_float<T>(zr + g, mn);
         for (int j = 0; j < a.group; j++) {
             float v = load_as_float<T>(xg + j);
             if (ref3) {
-                uint32_t q = quantize_code(v, mn, scale, (pos3 < 10 || wrap11) ? 7 : 3);
+                uint32_t q = quantize_code(v, mn, scale, rcp, (pos3 < 10 || wrap11) ? 7 : 3);
                 if (pos3 == 10) q &= 3u;  // only two bits of the word are left
                 buf |= (uint64_t)q << (pos3 < 10 ? 3 * pos3 : 30);
                 if (++pos3 == 11) {
@@ -120,7 +127,7 @@ __global__ void __launch_bounds__(256) quant_rows_generic(QuantArgs a, int unit,
                     pos3 = 0;
                 }
             } else {
-                uint32_t q = quantize_code(v, mn, scale, qmax);
+                uint32_t q = quantize_code(v, mn, scale, rcp, qmax);
                 buf |= (uint64_t)q << filled;
                 filled += a.bits;
                 if (filled >= 32) {
@@ -194,9 +201,10 @@ __device__ __forceinline__ void rows_g32_f16_body(const QuantArgs &a, int64_t gr
         constexpr int qmax = (1 << BITS) - 1;
         const float range = mx - mn;
         const float scale = range / (float)qmax;
+        const float rcp = quantize_rcp(scale);
         uint32_t piece = 0;  // this lane's 8 codes, 8*BITS bits
 #pragma unroll
-        for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, qmax) << (t * BITS);
+        for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, rcp, qmax) << (t * BITS);
 
         const bool act = active[p];
         uint32_t *cw = a.code + o[p] * a.c_os + i[p] * a.c_is + gr[p] * BITS;  // BITS words per group of 32
@@ -247,10 +255,9 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16(QuantArgs a, int64_t g
 // P groups per thread with the loads issued first; codes leave as one vector store per group.
 // ---------------------------------------------------------------------------------------
 template <int BITS, int P>
-__global__ void __launch_bounds__(256) quant_rows_g32_f16_stream(QuantArgs a, uint32_t groups_per_row,
-                                                                 int64_t total_groups)
+__device__ __forceinline__ void rows_g32_f16_stream_body(const QuantArgs &a, uint32_t groups_per_row,
+                                                         int64_t total_groups, int64_t first)
 {
-    const int64_t first = (int64_t)blockIdx.x * (256 * P) + threadIdx.x;
     uint4 raw[P][4];
     int64_t o[P], i[P];
     uint32_t gr[P];
@@ -289,12 +296,13 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16_stream(QuantArgs a, ui
         constexpr int qmax = (1 << BITS) - 1;
         const float range = mx - mn;
         const float scale = range / (float)qmax;
+        const float rcp = quantize_rcp(scale);
         uint32_t w[BITS];
 #pragma unroll
         for (int t = 0; t < BITS; t++) w[t] = 0;
 #pragma unroll
         for (int t = 0; t < 32; t++) {
-            const uint32_t q = quantize_code(v[t], mn, scale, qmax);
+            const uint32_t q = quantize_code(v[t], mn, scale, rcp, qmax);
             const int bit = t * BITS;
             w[bit >> 5] |= q << (bit & 31);
             if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
@@ -308,6 +316,13 @@ __global__ void __launch_bounds__(256) quant_rows_g32_f16_stream(QuantArgs a, ui
             ((__half *)a.zero)[o[p] * a.s_os + i[p] * a.s_is + gr[p]] = __float2half_rn(mn);
         }
     }
+}
+
+template <int BITS, int P>
+__global__ void __launch_bounds__(256) quant_rows_g32_f16_stream(QuantArgs a, uint32_t groups_per_row,
+                                                                 int64_t total_groups)
+{
+    rows_g32_f16_stream_body<BITS, P>(a, groups_per_row, total_groups, (int64_t)blockIdx.x * (256 * P) + threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -352,10 +367,11 @@ __global__ void __launch_bounds__(256) quant_rows_ref3_f16(QuantArgs a, uint32_t
         }
         const float range = mx - mn;
         const float scale = range / 7.0f;
+        const float rcp = quantize_rcp(scale);
         uint32_t word = 0;
 #pragma unroll
-        for (int t = 0; t < 10; t++) word |= quantize_code(v[t], mn, scale, 7) << (3 * t);
-        word |= (quantize_code(v[10], mn, scale, WRAP ? 7 : 3) & 3u) << 30;
+        for (int t = 0; t < 10; t++) word |= quantize_code(v[t], mn, scale, rcp, 7) << (3 * t);
+        word |= (quantize_code(v[10], mn, scale, rcp, WRAP ? 7 : 3) & 3u) << 30;
         if (active[p]) {
             a.code[o[p] * a.c_os + i[p] * a.c_is + wr[p]] = word;
             ((__half *)a.scale)[o[p] * a.s_os + i[p] * a.s_is + wr[p]] =
@@ -383,33 +399,33 @@ struct KeyTokArgs {
     float inv_qmax;
 };
 
+// G values of one channel -> packed words, scale, zero, stored at group gi of channel d
 template <int G, int MODE>
-__device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi, int64_t o, int64_t d)
+__device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float (&v)[G], int64_t gi, int64_t o,
+                                                int64_t d)
 {
     constexpr int BITS = MODE == 30 ? 3 : MODE;
     constexpr int qmax = (1 << BITS) - 1;
     constexpr int WORDS = MODE == 3 ? 1 : (G * BITS) / 32;  // words per group
-    const __half *src = a.k + o * a.k_os + gi * G * a.k_ts + d;
-    float v[G];
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
 #pragma unroll
     for (int t = 0; t < G; t++) {
-        v[t] = __half2float(src[t * a.k_ts]);
         mn = fminf(mn, v[t]);
         mx = fmaxf(mx, v[t]);
     }
     const float range = mx - mn;
     const float scale = range / (float)qmax;
+    const float rcp = quantize_rcp(scale);
     uint32_t w[WORDS];
 #pragma unroll
     for (int t = 0; t < WORDS; t++) w[t] = 0;
 #pragma unroll
     for (int t = 0; t < G; t++) {
         if (MODE == 3) {
-            uint32_t q = quantize_code(v[t], mn, scale, t < 10 ? 7 : 3);
+            uint32_t q = quantize_code(v[t], mn, scale, rcp, t < 10 ? 7 : 3);
             w[0] |= q << (t < 10 ? 3 * t : 30);
         } else {
-            uint32_t q = quantize_code(v[t], mn, scale, qmax);
+            uint32_t q = quantize_code(v[t], mn, scale, rcp, qmax);
             const int bit = t * BITS;
             w[bit >> 5] |= q << (bit & 31);
             if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
@@ -421,6 +437,50 @@ __device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi,
     a.scale[o * a.s_os + d * a.s_is + gi] =
         __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
     a.zero[o * a.s_os + d * a.s_is + gi] = __float2half_rn(mn);
+}
+
+template <int G, int MODE>
+__device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi, int64_t o, int64_t d)
+{
+    const __half *src = a.k + o * a.k_os + gi * G * a.k_ts + d;
+    float v[G];
+#pragma unroll
+    for (int t = 0; t < G; t++) v[t] = __half2float(src[t * a.k_ts]);
+    key_group_store<G, MODE>(a, v, gi, o, d);
+}
+
+// The same for D = 128 with 16-byte-aligned token rows, 256 threads = two (group, outer) pairs:
+// the pair's [G tokens][128 channels] tile is fetched with 128-bit loads (a thread: 8 channels of
+// one token) into LDS and each thread then reads its channel's column -- 4 wide loads per
+// thread instead of 32 two-byte ones.  Every thread of the block must call it (block barrier).
+template <int G, int MODE>
+__device__ __forceinline__ void key_tokens_tile_body(const KeyTokArgs &a, int64_t k_groups, int64_t pairs,
+                                                     int64_t first_pair, uint16_t (*tile)[32][128])
+{
+    const int half = threadIdx.x / 128, t = threadIdx.x % 128;
+    const int64_t pair = first_pair + half;
+    const bool valid = pair < pairs;
+    const int64_t pc = valid ? pair : pairs - 1;
+    const int64_t gi = pc % k_groups, o = pc / k_groups;
+    const __half *src = a.k + o * a.k_os + gi * G * a.k_ts;
+    constexpr int PIECES = G * 16;  // 16-byte pieces of the tile
+    uint4 raw[(PIECES + 127) / 128];
+#pragma unroll
+    for (int i = 0; i < (PIECES + 127) / 128; i++) {
+        int pc8 = i * 128 + t;
+        pc8 = pc8 < PIECES ? pc8 : PIECES - 1;
+        raw[i] = *reinterpret_cast<const uint4 *>(src + (int64_t)(pc8 / 16) * a.k_ts + (pc8 % 16) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < (PIECES + 127) / 128; i++) {
+        const int pc8 = i * 128 + t;
+        if (pc8 < PIECES) *reinterpret_cast<uint4 *>(&tile[half][pc8 / 16][(pc8 % 16) * 8]) = raw[i];
+    }
+    __syncthreads();
+    float v[G];
+#pragma unroll
+    for (int r = 0; r < G; r++) v[r] = h16_to_f32(tile[half][r][t]);
+    if (valid) key_group_store<G, MODE>(a, v, gi, o, t);
 }
 
 template <int G, int MODE>
@@ -438,10 +498,22 @@ __global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
 // launch costs about what either part costs alone.
 // ---------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, int64_t k_groups,
-                                                      int64_t k_threads, unsigned k_blocks, QuantArgs va,
-                                                      int64_t v_groups_per_row, int64_t v_total_groups)
+                                                      int64_t k_threads, unsigned k_blocks, int k_tiled,
+                                                      QuantArgs va, int64_t v_groups_per_row,
+                                                      int64_t v_total_groups)
 {
-    if (blockIdx.x < k_blocks) {
+    __shared__ __attribute__((aligned(16))) uint16_t tile[2][32][128];
+    if (blockIdx.x < k_blocks && k_tiled) {
+        // (k_threads = pairs * 128: one block = two (group, outer) pairs)
+        const int64_t pairs = k_threads / 128, first = (int64_t)blockIdx.x * 2;
+        switch (kmode) {
+        case 1: key_tokens_tile_body<32, 1>(ka, k_groups, pairs, first, tile); break;
+        case 2: key_tokens_tile_body<32, 2>(ka, k_groups, pairs, first, tile); break;
+        case 3: key_tokens_tile_body<11, 3>(ka, k_groups, pairs, first, tile); break;
+        case 4: key_tokens_tile_body<32, 4>(ka, k_groups, pairs, first, tile); break;
+        default: key_tokens_tile_body<32, 30>(ka, k_groups, pairs, first, tile); break;
+        }
+    } else if (blockIdx.x < k_blocks) {
         const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
         if (id >= k_threads) return;
         const int64_t d = id % ka.D, pair = id / ka.D;
@@ -454,12 +526,12 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
         default: key_tokens_body<32, 30>(ka, gi, o, d); break;
         }
     } else {
-        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * 256 + threadIdx.x;
+        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * (256 * KVMIX_FLUSH_V_PIECES) + threadIdx.x;
         switch (va.bits) {
-        case 1: rows_g32_f16_body<1, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        default: rows_g32_f16_body<4, 1, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 1: rows_g32_f16_body<1, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        default: rows_g32_f16_body<4, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
         }
     }
 }
@@ -749,9 +821,12 @@ extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmi
     const int64_t k_threads = kgroups * kf->outer * kf->D;
     const int64_t k_blocks = (k_threads + 255) / 256;
     const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
-    const int64_t v_blocks = (v_total * 4 + 255) / 256;
+    const int64_t v_blocks = (v_total * 4 + 256 * KVMIX_FLUSH_V_PIECES - 1) / (256 * KVMIX_FLUSH_V_PIECES);
     if (k_blocks + v_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    // key tile path: D = 128, token rows 16-byte aligned
+    const int k_tiled = KVMIX_FLUSH_K_TILED && kf->D == 128 && (uintptr_t)kf->k % 16 == 0 && kf->k_token_stride % 8 == 0 &&
+                        kf->k_outer_stride % 8 == 0;
     hipLaunchKernelGGL(quant_kv_flush, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, ka, kmode, kgroups,
-                       k_threads, (unsigned)k_blocks, va, v_groups, v_total);
+                       k_threads, (unsigned)k_blocks, k_tiled, va, v_groups, v_total);
     return launch_status();
 }

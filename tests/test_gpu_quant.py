@@ -250,3 +250,39 @@ def test_prompt_size_inputs_take_the_streaming_kernels(oracle, dev, bits):
         code, scale, mn = KVmix.quantize_pack_last_dim_cuda(torch.from_numpy(x11).to(dev), 11, 3)
         oc, osc, omn = oracle.quantize_pack_last_dim(x11, 11, 3)
         assert same_bits(code.cpu().numpy(), oc) and same_bits(scale.cpu().numpy(), osc) and same_bits(mn.cpu().numpy(), omn)
+
+
+@pytest.mark.parametrize("bits", [4, 2, 3])
+def test_values_at_and_next_to_rounding_ties(oracle, dev, bits):
+    """The kernels decide most codes from (x - min) * (1 / scale) and fall back to the division only
+    near a tie: values exactly on k + 0.5, and a few ulps to either side, must still give the
+    division's code.  fp32 input (every ulp reachable) and fp16 input (exact ties)."""
+    import KVmix
+
+    rng = np.random.default_rng(40 + bits)
+    g = 11 if bits == 3 else 32
+    qmax = 7 if bits == 3 else (1 << bits) - 1
+    rows = 4096
+    x = np.empty((1, 1, rows, g), np.float32)
+    for r in range(rows):
+        mn = np.float32(rng.uniform(-8, 8))
+        scale = np.float32(2.0 ** rng.integers(-12, 6)) * np.float32(rng.uniform(1, 2))
+        mx = np.float32(mn + np.float32(qmax) * scale)
+        k = rng.integers(0, qmax, g).astype(np.float32)
+        v = (mn + (k + np.float32(0.5)) * scale).astype(np.float32)
+        ulps = rng.integers(-3, 4, g)
+        v = (v.view(np.int32) + (ulps * np.sign(v)).astype(np.int32)).astype(np.int32).view(np.float32)
+        v[0], v[1] = mn, mx  # pin the group's min and max
+        x[0, 0, r] = np.clip(v, mn, mx)
+    got = KVmix.quantize_pack_last_dim_cuda(torch.from_numpy(x).to(dev), g, bits)
+    check_triplet(got, oracle.quantize_pack_last_dim(x, g, bits), "fp32 ties")
+    # fp16: min 0, max qmax * 2^e -> every k + 0.5 step is an exact tie
+    xh = np.empty((1, 1, 64, g), np.float16)
+    for r in range(64):
+        s = 2.0 ** (r % 8 - 3)
+        k = rng.integers(0, qmax, g)
+        v = (k + 0.5) * s
+        v[0], v[1] = 0.0, qmax * s
+        xh[0, 0, r] = v
+    got = KVmix.quantize_pack_last_dim_cuda(torch.from_numpy(xh).to(dev), g, bits)
+    check_triplet(got, oracle.quantize_pack_last_dim(xh, g, bits), "fp16 ties")
