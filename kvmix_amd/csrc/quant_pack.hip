@@ -460,8 +460,8 @@ __device__ __forceinline__ void key_tokens_tile_body(const KeyTokArgs &a, int64_
     const int half = threadIdx.x / 128, t = threadIdx.x % 128;
     const int64_t pair = first_pair + half;
     const bool valid = pair < pairs;
-    const int64_t pc = valid ? pair : pairs - 1;
-    const int64_t gi = pc % k_groups, o = pc / k_groups;
+    const uint32_t pc = (uint32_t)(valid ? pair : pairs - 1);  // (the host keeps pairs below 2^31)
+    const int64_t o = pc / (uint32_t)k_groups, gi = pc - (uint32_t)o * (uint32_t)k_groups;
     const __half *src = a.k + o * a.k_os + gi * G * a.k_ts;
     constexpr int PIECES = G * 16;  // 16-byte pieces of the tile
     uint4 raw[(PIECES + 127) / 128];
@@ -516,8 +516,10 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
     } else if (blockIdx.x < k_blocks) {
         const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
         if (id >= k_threads) return;
-        const int64_t d = id % ka.D, pair = id / ka.D;
-        const int64_t gi = pair % k_groups, o = pair / k_groups;
+        // (32-bit divisions: the host keeps the thread count below 2^31)
+        const uint32_t id32 = (uint32_t)id, D32 = (uint32_t)ka.D, pair = id32 / D32;
+        const int64_t d = id32 - pair * D32;
+        const int64_t o = pair / (uint32_t)k_groups, gi = pair - (uint32_t)o * (uint32_t)k_groups;
         switch (kmode) {
         case 1: key_tokens_body<32, 1>(ka, gi, o, d); break;
         case 2: key_tokens_body<32, 2>(ka, gi, o, d); break;
@@ -822,7 +824,7 @@ extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmi
     const int64_t k_blocks = (k_threads + 255) / 256;
     const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
     const int64_t v_blocks = (v_total * 4 + 256 * KVMIX_FLUSH_V_PIECES - 1) / (256 * KVMIX_FLUSH_V_PIECES);
-    if (k_blocks + v_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    if (k_blocks + v_blocks > 0x7fffffff || k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
     // key tile path: D = 128, token rows 16-byte aligned
     const int k_tiled = KVMIX_FLUSH_K_TILED && kf->D == 128 && (uintptr_t)kf->k % 16 == 0 && kf->k_token_stride % 8 == 0 &&
                         kf->k_outer_stride % 8 == 0;
