@@ -33,8 +33,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 # device kernel behind each tag at this workload (the names the rocprofv3 summaries list)
 DEVICE_KERNEL = {
-    "gemv_cols[ref3]": "kvmix::gemv_cols3<2, 2, 8>", "gemv_cols[b4]": "kvmix::gemv_cols_mfma<4, 1>",
-    "gemv_cols[b2]": "kvmix::gemv_cols_mfma<2, 1>", "gemv_rows[b4]": "kvmix::gemv_rows_mfma<4, 1, 1>",
+    "gemv_cols[ref3]": "kvmix::gemv_cols3<2, 2, 8>", "gemv_cols[b4]": "kvmix::gemv_cols_mfma2<4>",
+    "gemv_cols[b2]": "kvmix::gemv_cols_mfma2<2>", "gemv_rows[b4]": "kvmix::gemv_rows_mfma<4, 1, 1>",
     "gemv_rows[b2]": "kvmix::gemv_rows_mfma<2, 1, 1>", "gemv_rows[dense3]": "kvmix::gemv_rows_mfma<30, 1, 1>",
 }
 

@@ -36,6 +36,12 @@
 #ifndef KVMIX_COLS3_HEADS_OCC
 #define KVMIX_COLS3_HEADS_OCC 2
 #endif
+#ifndef KVMIX_MFMA2_OCC4
+#define KVMIX_MFMA2_OCC4 2
+#endif
+#ifndef KVMIX_COLS_MFMA2
+#define KVMIX_COLS_MFMA2 1  // 2/4-bit MHA q.K^T: two elements per lane
+#endif
 #ifndef KVMIX_COLS_MFMA
 #define KVMIX_COLS_MFMA 1  // 1/2/4-bit q.K^T on the matrix cores
 #endif
@@ -1432,6 +1438,228 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// gemv_cols_mfma2<BITS>   q.K^T, 4- or 2-bit codes, one query head per kv head: gemv_cols_mfma with
+// TWO 8-code elements per lane, so that a wave reads twice as many contiguous bytes of a row per
+// load instruction (512 for 4 bits: measured, the length of the contiguous pieces is what bounds
+// the streaming rate of this shape).  Tile = 128 elements = 1024 codes = 32 groups.
+//   A lane loads elements 2l and 2l+1 of every row (one dwordx2 / dword).  A quad of lanes then
+//   holds two quantization groups: lanes 0,1 the four elements of the first, lanes 2,3 those of
+//   the second.  Two MFMA sets per quad: set 0 works on the first group (lanes 2,3 fetch the
+//   second elements of lanes 0,1 with a DPP quad permute), set 1 on the second.  Per set the
+//   scheme is gemv_cols_mfma's: k = 4 channel rows, three exact bf16 parts of x*scale*2^90 as A.
+//   Rows are walked in chunks of 16 (4 k-steps); the chunk's [16][32] scales and zeros are one
+//   128-bit load per lane each (64-byte pieces per row).  LDS tile: per (k-step, set) a row of
+//   64 eight-byte cells in four sub-rows at a pitch of 17 cells, rows at a pitch of 74: staging
+//   stores and operand reads are bank-conflict free.
+//   block = (64, 2..4) waves on neighbouring tiles, a wave walks `splits` tiles;
+//   grid = (tiles/(waves*splits), samples, M), XCD-swizzled.
+// ---------------------------------------------------------------------------------------
+constexpr int kColsMfma2Row = 74 * 4;                   // bf16 elements per (k-step, set) row
+constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets
+
+template <int BITS>
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(KVMIX_MFMA2_OCC4)))
+gemv_cols_mfma2(GemvArgs a)
+{
+    static_assert(BITS == 4 || BITS == 2, "two elements per lane: a dwordx2 or a dword");
+    constexpr int CH = 16;             // rows per chunk
+    constexpr int KB = CH / 4;         // MFMA k-steps per chunk
+    constexpr int AT = kColsMfma2Tile;
+    constexpr int NPOS = 8;
+    constexpr int FPB = 8 / BITS;
+    constexpr int TG = 32;             // groups per tile
+    constexpr int WL = BITS / 2;       // dwords per lane and row (2 or 1)
+
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x;
+    const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int nw = (int)blockDim.y;
+    uint16_t *atile = reinterpret_cast<uint16_t *>(lds) + wy * (AT + TG * 2);
+    float *zl = reinterpret_cast<float *>(atile + AT);  // [32] zero terms of a tile
+    int64_t bx, sample;
+    xcd_swizzled_block(bx, sample, true);
+    const int64_t m = blockIdx.z;
+    const int64_t kv = sample / a.heads_per_kv;
+    const int K = (int)a.K;
+    const int ngroups = (int)(a.N / 32);
+    const int tpw = a.splits;
+    const int tile0 = (int)bx * tpw * nw + wy;
+    if (tile0 * TG >= ngroups) return;  // (no block barrier below)
+    const int nch = (K + CH - 1) / CH;
+    const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
+
+    const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
+    const uint32_t *cbase = a.code + kv * a.c_bs + lane * WL;
+    const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
+    const int sub = lane % 4;   // staging: row lane/4 of the chunk, groups 8*sub .. 8*sub+7
+    const int srow = lane / 4;
+    const uint16_t *sbase = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs + 8 * sub;
+    const uint16_t *zbase = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs + 8 * sub;
+    const int j4 = lane % 4;    // position in the quad
+
+    f32x4_t acc[2][NPOS];
+    float zacc[8];
+    auto clear = [&]() {
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) acc[q][p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) zacc[j] = 0.f;
+    };
+    clear();
+    for (int i = lane; i < AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+
+    // cell (four bf16 k-slots) of (k-step t, set s, operand lane l)
+    auto cell = [](int t, int s, int l) { return (2 * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
+    // staged row srow is k-slot srow%4 of k-step srow/4; its group g = 8*sub + jj is set g%2 of quad g/2,
+    // i.e. operand lanes 4*(g/2) + i = 16*sub + 4*(jj/2) + i
+    const int aoff = cell(srow / 4, 0, 16 * sub) + srow % 4;
+
+    Half8 s8, z8;
+    uint16_t xh;
+    uint32_t w[KB][4][WL];
+
+    auto tile_g0 = [&](int it) {
+        const int g = (tile0 + (it / nch) * nw) * TG;
+        return g + TG <= ngroups ? g : ngroups - TG;
+    };
+    auto chunk_k0 = [&](int it) { return (it % nch) * CH; };
+    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
+    auto load_small = [&](int it) {
+        const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
+        const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
+        s8 = *reinterpret_cast<const Half8 *>(sbase + off);
+        z8 = *reinterpret_cast<const Half8 *>(zbase + off);
+        xh = xp[d];
+    };
+    auto load_codes = [&](int it, int t) {
+        // (a group of 32 codes is BITS words)
+        const uint32_t *base = cbase + ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const Words<WL> v = *reinterpret_cast<const Words<WL> *>(base + (uint32_t)k * c_rs);
+#pragma unroll
+            for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
+        }
+    };
+    auto stage = [&](int it) {
+        const int k0 = chunk_k0(it);
+        const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
+        const float xv = srow >= skip ? h16_to_f32(xh) : 0.f;
+        const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            zacc[jj] = fmaf(xv, h16_to_f32(z8.v[jj]), zacc[jj]);
+            const float v0 = x2 * h16_to_f32(s8.v[jj]);  // split into three bf16 by truncation (exact)
+            const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+            const float v1 = v0 - __uint_as_float(b0);
+            const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+            const float v2 = v1 - __uint_as_float(b1);
+            const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+            for (int pt = 0; pt < 3; pt++)
+                atile[aoff + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+        }
+    };
+    // first element (8 codes) of the group set s works on, as this lane sees it: for 4 bits the
+    // word itself, for 2 bits the half of the word given by the byte offset in the selector
+    auto compute = [&](int t) {
+        const bf16x4_t av0 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 0, lane));
+        const bf16x4_t av1 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 1, lane));
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            // set 0: lanes 0,1 of a quad hold the group's elements 0,2 (their first) and lanes 2,3
+            // take elements 1,3 (the second of lanes 0,1); set 1 mirrors it for lanes 2,3
+            uint32_t src[4];
+            uint32_t hi = 0;  // 2 bits: byte offset (0 or 2) of the element inside the word
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if constexpr (BITS == 4) {
+                    const uint32_t other = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][1], 0x44, 0xf, 0xf, false)
+                                                  : __builtin_amdgcn_mov_dpp(w[t][k][1], 0xEE, 0xf, 0xf, false);
+                    const bool own = s == 0 ? j4 < 2 : j4 >= 2;
+                    src[k] = own ? w[t][k][0] : other;
+                } else {
+                    src[k] = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][0], 0x44, 0xf, 0xf, false)
+                                    : __builtin_amdgcn_mov_dpp(w[t][k][0], 0xEE, 0xf, 0xf, false);
+                }
+            }
+            if constexpr (BITS == 2) hi = (s == 0 ? j4 >= 2 : j4 < 2) ? 2u : 0u;
+#pragma unroll
+            for (int b = 0; b < BITS; b++) {
+                const uint32_t sel = (0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16)) + hi * 0x00010001u;
+                const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
+#pragma unroll
+                for (int f = 0; f < FPB; f++) {
+                    const uint32_t mask = (((1u << BITS) - 1u) * 0x00010001u) << (BITS * f);
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+                    acc[s][b * FPB + f] =
+                        __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(s == 0 ? av0 : av1, bv, acc[s][b * FPB + f], 0, 0, 0);
+                }
+            }
+        }
+    };
+    struct __attribute__((packed, aligned(2))) Out8 {
+        uint16_t v[8];
+    };
+    auto finish_tile = [&](int it) {
+        // zero terms: zacc[jj] summed over the 16 lanes with the same `sub`; group 8*sub+jj -> LDS
+        float z[8];
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) z[jj] = zacc[jj];
+        const int first = scatter_reduce<8, 4, 1>(z, lane);  // lane bits 2..4
+        z[0] += __shfl_xor(z[0], 32);
+        zl[8 * sub + first] = z[0];
+        wave_lds_fence();
+        const int q = lane / 4;
+        uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)tile_g0(it) * 32;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const float zt = zl[2 * q + s];
+            // element of the quad's 8 that this lane's accumulators of set s belong to
+            const int elem = s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1)));
+            Out8 o;
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) {
+                const float sum = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
+                o.v[p] = f32_to_h16(fmaf(sum, __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
+            }
+            *reinterpret_cast<Out8 *>(orow + (8 * q + elem) * 8) = o;
+        }
+        wave_lds_fence();
+        clear();
+    };
+
+    wave_lds_fence();
+    load_small(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < KB; t++) {
+        load_codes(0, t);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll 1
+    for (int it = 0; it < items; it++) {
+        const int nx = it + 1 < items ? it + 1 : it;  // (past the end: the same item again)
+        stage(it);
+        wave_lds_fence();
+        load_small(nx);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < KB; t++) {
+            compute(t);
+            load_codes(nx, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wave_lds_fence();  // the next chunk overwrites the tile
+        if (it % nch == nch - 1) finish_tile(it);
+    }
+}
+
 __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
 {
     const int64_t sample = blockIdx.y;
@@ -1690,9 +1918,34 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     hipLaunchKernelGGL((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a);
 }
 
+template <int BITS>
+static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    const int64_t tiles = (a.N / 32 + 31) / 32;
+    const int64_t batch = samples * a.M;
+    int64_t tpw = batch * tiles / kTargetWaves;  // tiles per wave: about one resident round of waves
+    tpw = tpw < 1 ? 1 : (tpw > 8 ? 8 : tpw);
+    const int64_t slots = (tiles + tpw - 1) / tpw;
+    const int wpb = pick_waves_per_block(slots);
+    a.splits = (int)tpw;
+    const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
+    const size_t lds = (size_t)wpb * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
+    hipLaunchKernelGGL((gemv_cols_mfma2<BITS>), grid, dim3(kWave, wpb), lds, st, a);
+}
+
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
+    if constexpr (MODE == 2 || MODE == 4) {
+        // two-element matrix-core kernel: measured faster than gemv_cols and gemv_cols_mfma up to
+        // one resident round of waves (B = 16 at T = 8k); beyond that gemv_cols streams better
+        const int64_t tiles2 = (a.N / 32 + 31) / 32;
+        if (KVMIX_COLS_MFMA2 && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
+            samples * a.M * tiles2 <= kTargetWaves) {
+            launch_cols_mfma2<MODE>(a, samples, st);
+            return;
+        }
+    }
     if constexpr (MODE == 1 || MODE == 2 || MODE == 4) {
         // Matrix-core kernel: always for GQA (the query heads of a kv head share one pass over
         // the codes); for one head per kv head only when the problem is small enough that
