@@ -25,9 +25,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
-
-# Residual ratio the reference's profiler assigns to each bit width (myprofileKV.py:75-80).
-RESIDUAL_RATIO_BY_BITS = {4: 0.3, 3: 0.2, 2: 0.2, 1: 0.1}
+from .cache import RESIDUAL_RATIO_BY_BITS, PackedKVCache, flush_length  # noqa: F401 (re-exported)
 
 
 def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
@@ -37,24 +35,6 @@ def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
         return hidden_states
     hidden_states = hidden_states[:, :, None, :, :].expand(batch, num_key_value_heads, n_rep, slen, head_dim)
     return hidden_states.reshape(batch, num_key_value_heads * n_rep, slen, head_dim)
-
-
-def flush_length(tail_len: int, ratio: float, group: int, residual_length: Optional[int] = None,
-                 prompt: bool = False) -> int:
-    """Number of oldest tail tokens to quantize now.
-
-    Ratio rule (models/modeling_llama_KVmix.py:119-127,152-155 and, for the prompt, :219-224):
-    keep int(ratio * L) tokens in fp16, quantize the rest rounded down to a multiple of the group.
-    Fixed window (residual_length = R): once the tail holds R tokens, flush floor(R/g)*g; for a
-    prompt, everything but the newest R tokens, rounded down to a multiple of the group."""
-    if residual_length is not None:
-        if prompt:
-            return (max(tail_len - residual_length, 0) // group) * group
-        return (residual_length // group) * group if tail_len >= residual_length else 0
-    keep = int(ratio * tail_len)
-    if tail_len > keep and keep >= 0:
-        return ((tail_len - keep) // group) * group
-    return 0
 
 
 def _cat(old: Optional[torch.Tensor], new: torch.Tensor, dim: int) -> torch.Tensor:
@@ -119,25 +99,42 @@ class KVmixAttention:
             vq = (_cat(vq[0], vc, 2), _cat(vq[1], vs, 2), _cat(vq[2], vm, 2))
         return k_tail, kq, v_tail, vq
 
+    def new_cache(self, capacity: int = 4096, k_fmt: int = ops.FMT_REF, v_fmt: int = ops.FMT_REF) -> PackedKVCache:
+        """An empty in-place cache with this layer's bit widths and flush policy; pass it as
+        past_key_value from the prompt on (the same object comes back, updated)."""
+        return PackedKVCache(self.k_bits, self.v_bits, self.Vgroup_size, self.k_residual_ratio,
+                             self.v_residual_ratio, self.residual_length, capacity, k_fmt, v_fmt)
+
     # -- the step --------------------------------------------------------------------------
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
-                past_key_value: Optional[Tuple] = None, attention_mask: Optional[torch.Tensor] = None,
-                use_cache: bool = True):
+                past_key_value=None, attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True):
         """query_states [B,nh,Q,D], key/value_states [B,Hkv,Q,D] (fp16, after RoPE).
+        past_key_value: None (prompt), the reference's 9-tuple (a new tuple is returned, grown by
+        concatenation as the reference does), or a PackedKVCache (updated in place and returned;
+        an empty one means prompt).
         Returns (attn_output [B,nh,Q,D] fp16, attn_weights fp16, past_key_value or None)."""
         B, nh, q_len, D = query_states.shape
         n_rep = nh // key_states.shape[1]
-        kv_seq_len = key_states.shape[-2] + (past_key_value[-1] if past_key_value is not None else 0)
+        inplace = past_key_value if isinstance(past_key_value, PackedKVCache) else None
+        prompt = past_key_value is None or (inplace is not None and inplace.kv_seq_len == 0)
+        k_fmt = inplace.k_fmt if inplace is not None else ops.FMT_REF
+        v_fmt = inplace.v_fmt if inplace is not None else ops.FMT_REF
+        k_group = inplace.Kgroup_size if inplace is not None else self.Kgroup_size
 
-        if past_key_value is not None:
-            kc, k_tail, ks, km, vc, v_tail, vs, vm, _ = past_key_value
-            k_tail = key_states if k_tail is None else torch.cat([k_tail, key_states], dim=2)
-            v_tail = value_states if v_tail is None else torch.cat([v_tail, value_states], dim=2)
-            k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(k_tail, (kc, ks, km), v_tail, (vc, vs, vm))
+        if not prompt:
+            if inplace is not None:
+                inplace.append(key_states, value_states)
+                kc, k_tail, ks, km, vc, v_tail, vs, vm, kv_seq_len = inplace.as_tuple()
+            else:
+                kv_seq_len = key_states.shape[-2] + past_key_value[-1]
+                kc, k_tail, ks, km, vc, v_tail, vs, vm, _ = past_key_value
+                k_tail = key_states if k_tail is None else torch.cat([k_tail, key_states], dim=2)
+                v_tail = value_states if v_tail is None else torch.cat([v_tail, value_states], dim=2)
+                k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(k_tail, (kc, ks, km), v_tail, (vc, vs, vm))
 
             att_full = _grouped_matmul_qk(query_states, k_tail, n_rep)
             if kc is not None:
-                att_quant = ops.quantized_gemm(self.Kgroup_size, query_states, kc, ks, km, self.k_bits)
+                att_quant = ops.quantized_gemm(k_group, query_states, kc, ks, km, self.k_bits, k_fmt)
                 attn_weights = torch.cat([att_quant.to(torch.float32), att_full.to(torch.float32)], dim=-1)
             else:
                 attn_weights = att_full.to(torch.float32)
@@ -155,15 +152,20 @@ class KVmixAttention:
             else:
                 lv = v_tail.shape[-2]
                 tq = attn_weights.shape[-1] - lv
-                out_quant = ops.quantized_gemm(self.Vgroup_size, attn_weights[..., :tq], vc, vs, vm, self.v_bits)
+                out_quant = ops.quantized_gemm(self.Vgroup_size, attn_weights[..., :tq], vc, vs, vm, self.v_bits, v_fmt)
                 out_full = _grouped_matmul_pv(attn_weights[..., tq:], v_tail, n_rep)
                 attn_output = out_quant + out_full
         else:
             # prompt: dense fp16 attention; the cache keeps the oldest tokens quantized
             # (models/modeling_llama_KVmix.py:213-266)
-            k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(key_states, (None,) * 3, value_states,
-                                                                     (None,) * 3, prompt=True)
-            k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
+            kv_seq_len = key_states.shape[-2]
+            if inplace is not None:
+                if use_cache:
+                    inplace.append(key_states, value_states, prompt=True)
+            else:
+                k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(key_states, (None,) * 3, value_states,
+                                                                         (None,) * 3, prompt=True)
+                k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
             attn_weights = _grouped_matmul_qk(query_states, key_states, n_rep) / math.sqrt(D)
             if attention_mask is not None:
                 if attention_mask.shape[-2:] != attn_weights.shape[-2:]:
@@ -174,7 +176,12 @@ class KVmixAttention:
             attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
             attn_output = _grouped_matmul_pv(attn_weights, value_states, n_rep)
 
-        cache = (kc, k_tail, ks, km, vc, v_tail, vs, vm, kv_seq_len) if use_cache else None
+        if not use_cache:
+            cache = None
+        elif inplace is not None:
+            cache = inplace
+        else:
+            cache = (kc, k_tail, ks, km, vc, v_tail, vs, vm, kv_seq_len)
         return attn_output, attn_weights, cache
 
     __call__ = forward

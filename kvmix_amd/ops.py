@@ -150,25 +150,68 @@ def quantize_kv_flush(k_chunk: torch.Tensor, k_group: int, k_bits: int, v_chunk:
     def words(steps, bits, fmt):
         return steps * 3 // 32 if (bits == 3 and fmt == _lib.FMT_DENSE3) else steps // _values_per_word(bits)
 
-    if k_chunk.stride(3) != 1 or (B > 1 and k_chunk.stride(0) != H * k_chunk.stride(1)):
-        k_chunk = k_chunk.contiguous()
-    v_chunk, vo, vi = _rows3(v_chunk)
     kc = torch.empty((B, H, D, words(n, k_bits, k_fmt)), dtype=torch.int32, device=dev)
     ks = torch.empty((B, H, D, n // k_group if k_group > 0 else 0), dtype=torch.float16, device=dev)
     km = torch.empty_like(ks)
     vc = torch.empty((Bv, Hv, nv, words(Dv, v_bits, v_fmt)), dtype=torch.int32, device=dev)
     vs = torch.empty((Bv, Hv, nv, Dv // v_group if v_group > 0 else 0), dtype=torch.float16, device=dev)
     vm = torch.empty_like(vs)
-    kf = _lib.KeyFlush(k_chunk.data_ptr(), B * H, n, D, k_chunk.stride(1), k_chunk.stride(2), k_group, k_bits, k_fmt,
-                       _lib.SCALE_RECIPROCAL, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(), km.data_ptr(),
-                       ks.stride(1), ks.stride(2))
-    vf = _lib.ValueFlush(v_chunk.data_ptr(), Bv * Hv, nv, Dv, vo, vi, v_group, v_bits, v_fmt, _lib.SCALE_RECIPROCAL,
-                         vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(), vm.data_ptr(), vs.stride(1),
-                         vs.stride(2))
-    import ctypes
-    with torch.cuda.device(dev):
-        _lib.check(L.kvmix_quant_pack_kv_flush(ctypes.byref(kf), ctypes.byref(vf), _stream(k_chunk)))
+    quantize_kv_flush_into(k_chunk, k_group, k_bits, (kc, ks, km), v_chunk, v_group, v_bits, (vc, vs, vm), k_fmt, v_fmt)
     return kc, ks, km, vc, vs, vm
+
+
+def quantize_kv_flush_into(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v_group: int, v_bits: int, v_out,
+                           k_fmt: int = _lib.FMT_REF, v_fmt: int = _lib.FMT_REF) -> None:
+    """quantize_kv_flush writing into tensors the caller owns: k_out = (code [B,H,D,n/vpw],
+    scale, min [B,H,D,n/g]) and v_out = (code [B,H,nv,D/vpw], scale, min [B,H,nv,D/g]) may be
+    slices of larger pre-allocated cache buffers (unit stride along the last dimension, (B, H)
+    collapsible).  Either half may be None (k_chunk and k_out, or v_chunk and v_out)."""
+    import ctypes
+
+    L = _lib.load()
+    kf, vf = _lib.KeyFlush(), _lib.ValueFlush()
+    kf.group, kf.bits, kf.fmt, kf.scale_mode = max(k_group, 1), k_bits, k_fmt, _lib.SCALE_RECIPROCAL
+    vf.group, vf.bits, vf.fmt, vf.scale_mode = max(v_group, 1), v_bits, v_fmt, _lib.SCALE_RECIPROCAL
+    ref = k_chunk if k_chunk is not None else v_chunk
+    if ref is None:
+        return
+    _need_gpu(ref)
+
+    def out_strides(code, scale, mn, B, H):
+        for t in (code, scale, mn):
+            if t.dim() != 4 or (t.shape[3] > 1 and t.stride(3) != 1) or (B > 1 and t.stride(0) != H * t.stride(1)):
+                raise RuntimeError("output views must be 4-D, unit-stride along the last dimension, (B, H) collapsible")
+        if (scale.stride(1), scale.stride(2)) != (mn.stride(1), mn.stride(2)):
+            raise RuntimeError("scale and min outputs must share their strides")
+
+    if k_chunk is not None and k_chunk.shape[2] > 0:
+        B, H, n, D = k_chunk.shape
+        ref3 = k_bits == 3 and k_fmt == _lib.FMT_REF
+        if not ref3 and k_group != 32:
+            # the token-major key kernel is built for group 32 (and the reference's 3-bit group 11)
+            _quantize_into(k_chunk.transpose(2, 3).contiguous(), k_group, k_bits, k_fmt, _lib.SCALE_RECIPROCAL, *k_out)
+        else:
+            if k_chunk.stride(3) != 1 or (B > 1 and k_chunk.stride(0) != H * k_chunk.stride(1)):
+                k_chunk = k_chunk.contiguous()
+            kc, ks, km = k_out
+            out_strides(kc, ks, km, B, H)
+            kf.k, kf.outer, kf.n, kf.D = k_chunk.data_ptr(), B * H, n, D
+            kf.k_outer_stride, kf.k_token_stride = k_chunk.stride(1), k_chunk.stride(2)
+            kf.code, kf.code_outer_stride, kf.code_inner_stride = kc.data_ptr(), kc.stride(1), kc.stride(2)
+            kf.scale, kf.zero = ks.data_ptr(), km.data_ptr()
+            kf.sz_outer_stride, kf.sz_inner_stride = ks.stride(1), ks.stride(2)
+    if v_chunk is not None and v_chunk.shape[2] > 0:
+        Bv, Hv, nv, Dv = v_chunk.shape
+        v_chunk, vo, vi = _rows3(v_chunk)
+        vc, vs, vm = v_out
+        out_strides(vc, vs, vm, Bv, Hv)
+        vf.x, vf.outer, vf.inner, vf.steps = v_chunk.data_ptr(), Bv * Hv, nv, Dv
+        vf.x_outer_stride, vf.x_inner_stride = vo, vi
+        vf.code, vf.code_outer_stride, vf.code_inner_stride = vc.data_ptr(), vc.stride(1), vc.stride(2)
+        vf.scale, vf.zero = vs.data_ptr(), vm.data_ptr()
+        vf.sz_outer_stride, vf.sz_inner_stride = vs.stride(1), vs.stride(2)
+    with torch.cuda.device(ref.device):
+        _lib.check(L.kvmix_quant_pack_kv_flush(ctypes.byref(kf), ctypes.byref(vf), _stream(ref)))
 
 
 def _batched3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:
