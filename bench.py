@@ -335,6 +335,119 @@ def gqa_shape_extra(torch, _lib, lib, dev, stream):
     return res
 
 
+def sweep_extra(torch, _lib, lib, dev, stream):
+    """BASELINE configs[3]: MHA 32 x 128, T=4096 with a 32-token fp16 window (4064 quantized tokens),
+    1- and 2-bit keys and values, batch 1 / 16 / 64 / 128.  Each entry is one q.K^T or p.V launch;
+    enough buffer sets are rotated that no set is still in the 256 MB Infinity Cache when reused."""
+    H, D, Tq = 32, 128, 4064
+    res = {}
+    for bits in (1, 2):
+        for B in (1, 16, 64, 128):
+            nbytes = B * H * Tq * bytes_per_token(bits, "")
+            nsets = int(min(64, max(2, -(-(600 << 20) // int(nbytes)))))
+            sets = []
+            for _ in range(nsets):
+                kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+                ks = torch.rand(B, H, D, Tq // 32, device=dev).half()
+                kz = torch.randn(B, H, D, Tq // 32, device=dev).half()
+                vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+                vs = torch.rand(B, H, Tq, D // 32, device=dev).half()
+                vz = torch.randn(B, H, Tq, D // 32, device=dev).half()
+                sets.append((kc, ks, kz, vc, vs, vz))
+            q = torch.randn(B, H, 1, D, device=dev).half()
+            p = torch.softmax(torch.randn(B, H, 1, Tq, device=dev), -1).half()
+            lo = torch.empty(B, H, 1, Tq, device=dev, dtype=torch.float16)
+            o = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+            wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, Tq, D)
+            ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+
+            def qk(i):
+                kc, ks, kz = sets[i % nsets][:3]
+                return lib.kvmix_quantized_gemv(32, q.data_ptr(), D, D, kc.data_ptr(), kc.stride(1), kc.stride(2),
+                                                ks.data_ptr(), kz.data_ptr(), ks.stride(1), ks.stride(2), bits, 0, B * H, 1,
+                                                1, D, Tq, lo.data_ptr(), Tq, Tq, None, 0, stream)
+
+            def pv(i):
+                vc, vs, vz = sets[i % nsets][3:]
+                return lib.kvmix_quantized_gemv(32, p.data_ptr(), Tq, Tq, vc.data_ptr(), vc.stride(1), vc.stride(2),
+                                                vs.data_ptr(), vz.data_ptr(), vs.stride(1), vs.stride(2), bits, 0, B * H, 1,
+                                                1, Tq, D, o.data_ptr(), D, D, ws.data_ptr(), wsb, stream)
+
+            iters = max(30, 2 * nsets)
+            for name, fn in (("qk", qk), ("pv", pv)):
+                for i in range(nsets):
+                    assert fn(i) == 0
+                torch.cuda.synchronize()
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                for i in range(iters):
+                    fn(i)
+                e.record()
+                torch.cuda.synchronize()
+                us = s.elapsed_time(e) * 1e3 / iters
+                res[f"{name}_{bits}bit_B{B}"] = {"us": round(us, 2), "packed_MB": round(nbytes / 1e6, 1),
+                                                 "GBps": round(nbytes / us / 1e3, 1),
+                                                 "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            del sets
+            torch.cuda.empty_cache()
+    return res
+
+
+def e2e_extra(torch, dev, batch=4, prompt_len=2048, new_tokens=512):
+    """BASELINE configs[4]: greedy decoding on a random-init Llama-2-7B (fp16 weights ~N(0, 0.02), seed 4),
+    prompt of random token ids, mixed per-layer bits as in configs[1], 128-token fp16 window, in-place
+    caches.  The host loop is eager PyTorch (projections, RoPE, norms, MLP through torch / hipBLASLt);
+    the KV path is the library's.  Tokens/s as the reference's driver counts them
+    (Inference-comparision.py:147-151): new tokens and all tokens over the whole wall time; the
+    decode-only rate is given beside them."""
+    from kvmix_amd.decoder import Decoder, DecoderConfig, GraphDecoder, init_weights, kvmix_layers
+
+    cfg = DecoderConfig()
+    kbits, vbits = layer_bits(cfg.num_layers)
+    weights = init_weights(cfg, dev)
+    gen = torch.Generator(device="cpu").manual_seed(4)
+
+    def run(B, T, new, graph=True):
+        atts, caches = kvmix_layers(cfg, kbits, vbits, residual_length=128, capacity=T + new)
+        dec = (GraphDecoder if graph else Decoder)(cfg, weights, atts, caches)
+        prompt = torch.randint(0, cfg.vocab_size, (B, T), generator=gen).to(dev)
+        marks = {}
+
+        def on_step(step, logits):
+            if step == 0:
+                torch.cuda.synchronize()
+                marks["prefill_end"] = time.perf_counter()
+
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        tokens = dec.generate(prompt, new, on_step)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        steps = (dec.graph_steps, dec.eager_steps, dec.captures) if graph else (0, new, 0)
+        return tokens, marks["prefill_end"] - t0, t1 - marks["prefill_end"], [c.k_tokens for c in caches], steps
+
+    run(batch, 256, 8)  # warm-up: library heuristics, kernel loading
+    _, _, eager_decode_s, _, _ = run(batch, prompt_len, new_tokens, graph=False)
+    tokens, prefill_s, decode_s, k_tokens, steps = run(batch, prompt_len, new_tokens)
+    total = prefill_s + decode_s
+    return {
+        "model": "Llama-2-7B shape (32 layers, hidden 4096, 32 heads, ffn 11008, vocab 32000), random init, fp16",
+        "batch": batch, "prompt_tokens": prompt_len, "new_tokens": new_tokens, "residual": 128,
+        "k_bits": kbits, "v_bits": vbits,
+        "prefill_s": round(prefill_s, 3), "decode_s": round(decode_s, 3),
+        "decode_ms_per_step": round(decode_s * 1e3 / (new_tokens - 1), 3),
+        "new_tokens_per_s": round(batch * new_tokens / total, 1),
+        "all_tokens_per_s": round(batch * (prompt_len + new_tokens) / total, 1),
+        "decode_only_tokens_per_s": round(batch * (new_tokens - 1) / decode_s, 1),
+        "quantized_key_tokens_at_end": [int(min(k_tokens)), int(max(k_tokens))],
+        "host_loop": "decode steps replayed from a HIP graph, re-captured after every step that flushes "
+                     "(those steps run eagerly); prompt eager",
+        "graph_steps": steps[0], "eager_steps": steps[1], "graph_captures": steps[2],
+        "eager_host_loop": {"decode_ms_per_step": round(eager_decode_s * 1e3 / (new_tokens - 1), 3),
+                            "decode_only_tokens_per_s": round(batch * (new_tokens - 1) / eager_decode_s, 1)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -346,6 +459,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-target-shape", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end Llama-2-7B-shape decode loop")
+    ap.add_argument("--e2e-only", action="store_true", help="run only the end-to-end decode loop")
     ap.add_argument("--shapes-only", action="store_true",
                     help="skip the step: only the B=16/T=8192 target shape and the GQA configuration (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -364,6 +479,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, D, T, R = args.batch, 32, 128, args.context, 128
+    if args.e2e_only:
+        print(json.dumps({"e2e_config4_llama2_7b": e2e_extra(torch, dev)}))
+        return
     if args.shapes_only:
         if args.copy_calibration:
             src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -374,7 +492,8 @@ def main():
             del src, dst
         st = torch.cuda.current_stream().cuda_stream
         print(json.dumps({"target_shape_B16_T8192": target_shape_extra(torch, _lib, lib, dev, st),
-                          "gqa_config2_B16_T32768": gqa_shape_extra(torch, _lib, lib, dev, st)}))
+                          "gqa_config2_B16_T32768": gqa_shape_extra(torch, _lib, lib, dev, st),
+                          "sweep_config3_T4096": sweep_extra(torch, _lib, lib, dev, st)}))
         return
     kbits, vbits = layer_bits(args.layers)
     layers = build_layers(torch, ops, lib, B, H, D, T, R, kbits, vbits, dev)
@@ -497,6 +616,14 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
         torch.cuda.empty_cache()
         result["gqa_config2_B16_T32768"] = gqa_shape_extra(torch, _lib, lib, dev,
                                                            torch.cuda.current_stream().cuda_stream)
+        torch.cuda.empty_cache()
+        result["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, torch.cuda.current_stream().cuda_stream)
+    if not args.no_e2e:
+        torch.cuda.empty_cache()
+        try:
+            result["e2e_config4_llama2_7b"] = e2e_extra(torch, dev)
+        except Exception as ex:  # the headline line must still be printed
+            result["e2e_config4_llama2_7b"] = {"error": f"{type(ex).__name__}: {ex}"}
     print(json.dumps(result))
 
 

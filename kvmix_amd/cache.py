@@ -59,12 +59,12 @@ class _Tail:
     def append(self, new: torch.Tensor, reserve: int) -> None:
         B, H, n, D = new.shape
         if self.buf is None:
-            self.buf = torch.empty((B, H, max(reserve, 2 * n), D), dtype=new.dtype, device=new.device)
+            self.buf = torch.zeros((B, H, max(reserve, 2 * n), D), dtype=new.dtype, device=new.device)
         cap = self.buf.shape[2]
         if self.start + self.len + n > cap:
             live = self.view()
             if 2 * (self.len + n) > cap:  # the tail itself has grown: a longer buffer
-                buf = torch.empty((B, H, max(2 * cap, 2 * (self.len + n)), D), dtype=new.dtype, device=new.device)
+                buf = torch.zeros((B, H, max(2 * cap, 2 * (self.len + n)), D), dtype=new.dtype, device=new.device)
                 buf[:, :, :self.len].copy_(live)
                 self.buf = buf
             else:  # room at the front: move the live tokens there (regions may overlap)
@@ -76,6 +76,17 @@ class _Tail:
     def drop_front(self, n: int) -> None:
         self.start += n
         self.len -= n
+
+    def window(self, slots: int) -> torch.Tensor:
+        """A fixed-size view [B,H,slots,D] that starts at the live region (which is moved to the front
+        of the buffer first if the view would not fit): slots beyond the live tokens hold finite
+        leftovers (the buffer starts out zeroed), never uninitialised memory."""
+        if self.start + slots > self.buf.shape[2]:
+            if slots > self.buf.shape[2]:
+                raise RuntimeError("tail buffer shorter than the requested window")
+            self.buf[:, :, :self.len].copy_(self.view().clone())
+            self.start = 0
+        return self.buf[:, :, self.start:self.start + slots]
 
 
 class PackedKVCache:
@@ -200,6 +211,25 @@ class PackedKVCache:
         if self.v_tokens > 0:
             vc, vs, vm = (t[:, :, :self.v_tokens] for t in self._v)
         self._packed_views = (kc, ks, km, vc, vs, vm)
+
+    # -- hooks for a decode step replayed from a captured graph --------------------------------
+    def flushes_on_next_append(self) -> bool:
+        """Would appending one token make either tail flush?"""
+        nk = flush_length(self._k_tail.len + 1, self.k_residual_ratio, self.Kgroup_size, self.residual_length)
+        nv = flush_length(self._v_tail.len + 1, self.v_residual_ratio, self.Vgroup_size, self.residual_length)
+        return nk > 0 or nv > 0
+
+    def tail_windows(self, slots: int):
+        """(key window, value window, live key tokens, live value tokens): fixed-size views of the
+        fp16 tails for a step whose append is done by the caller on the device (the token goes to
+        slot `live tokens` of each window); follow every such step with note_device_append()."""
+        return self._k_tail.window(slots), self._v_tail.window(slots), self._k_tail.len, self._v_tail.len
+
+    def note_device_append(self) -> None:
+        """Book-keeping for one token that a device-side step wrote into the tail windows."""
+        self._k_tail.len += 1
+        self._v_tail.len += 1
+        self.kv_seq_len += 1
 
     # -- views -----------------------------------------------------------------------------
     def as_tuple(self) -> Tuple:

@@ -56,6 +56,12 @@
 #define KVMIX_MFMA_HEADS_OCC 2
 #endif
 
+#ifndef KVMIX_MFMA2_MAX_WAVES
+#define KVMIX_MFMA2_MAX_WAVES KVMIX_TARGET_WAVES  // two-element matrix-core q.K^T kernel up to this many tiles
+#endif
+#ifndef KVMIX_MFMA1_MAX_WAVES
+#define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
+#endif
 #ifndef KVMIX_TARGET_WAVES
 #define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
 #endif
@@ -1941,7 +1947,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // one resident round of waves (B = 16 at T = 8k); beyond that gemv_cols streams better
         const int64_t tiles2 = (a.N / 32 + 31) / 32;
         if (KVMIX_COLS_MFMA2 && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
-            samples * a.M * tiles2 <= kTargetWaves) {
+            samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES) {
             launch_cols_mfma2<MODE>(a, samples, st);
             return;
         }
@@ -1957,7 +1963,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
                 launch_cols_mfma<MODE, 4>(a, samples, st);
                 return;
             }
-            if (batch * ((units + 31) / 32) < kTargetWaves) {
+            if (batch * ((units + 31) / 32) < (int64_t)KVMIX_MFMA1_MAX_WAVES) {
                 launch_cols_mfma<MODE, 1>(a, samples, st);
                 return;
             }
