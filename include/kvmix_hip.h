@@ -175,6 +175,69 @@ int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride, int64
                          int64_t out_row_stride, void *workspace, size_t workspace_bytes,
                          kvmix_stream_t stream);
 
+/*
+ * One decode step of attention over the packed cache and its fp16 residual tails: what
+ * LlamaAttention_KVmix.forward does between RoPE and the output projection once the cache is up to
+ * date (models/modeling_llama_KVmix.py:68-75,180-211; Mistral twin: models/modeling_mistral_KVmix.py
+ * :114-121,217-262), on the caller's stream:
+ *
+ *   logits = cat(fp16 q.K^T over the quantized keys, fp16 q.K_tail^T) / sqrt(D)  (+ mask, clamped to
+ *            the lowest finite fp32), softmax in fp32, probabilities rounded to fp16;
+ *   out    = fp16(p.V over the quantized values) + fp16(p_tail . V_tail)
+ *
+ * The two quantized products are kvmix_quantized_gemv launches; the tail products and the softmax
+ * are two small kernels, so a step is four or five launches instead of the reference's dozen.
+ *
+ *   q        [samples, D] fp16 (samples = B * query heads, one row per head), row stride q_stride
+ *   k_..., v_...  the packed operands exactly as kvmix_quantized_gemv takes them (keys [.., D, Tk/vpw],
+ *            values [.., Tv, D/vpw]); k_tokens / v_tokens = Tk / Tv may be 0
+ *   k_tail, v_tail  [samples / heads_per_kv, slots, D] fp16 windows of the residual tails, of which
+ *            the first *_tail_len slots hold tokens.  If *_tail_len_dev is not NULL the length is
+ *            read from that device location when the kernel runs (a step replayed from a captured
+ *            graph) and *_tail_len is ignored.
+ *   mask     optional fp32 [samples / heads, width] added to the scaled logits (row = batch element)
+ *   probs    [samples, width] fp16, width = max(k_tokens + k_tail_slots, v_tokens + v_tail_slots):
+ *            out: the probabilities (position i of a row is token i; slots past a tail's length are 0)
+ *   out      [samples, D] fp16
+ * With host-side lengths, k_tokens + k_tail_len must equal v_tokens + v_tail_len.
+ * workspace: at least kvmix_decode_attention_workspace_bytes() bytes of device scratch.
+ */
+typedef struct kvmix_decode_attn {
+    const void *q;
+    int64_t q_stride;
+    const uint32_t *k_code;
+    int64_t k_code_batch_stride, k_code_row_stride;
+    const void *k_scale, *k_zero;
+    int64_t k_sz_batch_stride, k_sz_row_stride;
+    int k_bits, k_fmt, k_group;
+    int64_t k_tokens;
+    const uint32_t *v_code;
+    int64_t v_code_batch_stride, v_code_row_stride;
+    const void *v_scale, *v_zero;
+    int64_t v_sz_batch_stride, v_sz_row_stride;
+    int v_bits, v_fmt, v_group;
+    int64_t v_tokens;
+    const void *k_tail;
+    int64_t k_tail_batch_stride, k_tail_token_stride, k_tail_slots, k_tail_len;
+    const int64_t *k_tail_len_dev;
+    const void *v_tail;
+    int64_t v_tail_batch_stride, v_tail_token_stride, v_tail_slots, v_tail_len;
+    const int64_t *v_tail_len_dev;
+    const float *mask;
+    int64_t mask_stride;
+    int64_t samples;
+    int heads, heads_per_kv;
+    int64_t D;
+    void *probs;
+    int64_t probs_stride;
+    void *out;
+    int64_t out_stride;
+} kvmix_decode_attn_t;
+
+size_t kvmix_decode_attention_workspace_bytes(const kvmix_decode_attn_t *step);
+int kvmix_decode_attention(const kvmix_decode_attn_t *step, void *workspace, size_t workspace_bytes,
+                           kvmix_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,8 @@ EXPORTS = (
     "kvmix_quant_pack_kv_flush",
     "kvmix_gemv_workspace_bytes",
     "kvmix_quantized_gemv",
+    "kvmix_decode_attention_workspace_bytes",
+    "kvmix_decode_attention",
 )
 
 _lib = None
@@ -46,6 +48,25 @@ class ValueFlush(ctypes.Structure):
                 ("code", ctypes.c_void_p), ("code_outer_stride", ctypes.c_int64), ("code_inner_stride", ctypes.c_int64),
                 ("scale", ctypes.c_void_p), ("zero", ctypes.c_void_p),
                 ("sz_outer_stride", ctypes.c_int64), ("sz_inner_stride", ctypes.c_int64)]
+
+
+class DecodeAttn(ctypes.Structure):
+    """kvmix_decode_attn_t"""
+    _i64, _i32, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    _fields_ = [("q", _vp), ("q_stride", _i64),
+                ("k_code", _vp), ("k_code_batch_stride", _i64), ("k_code_row_stride", _i64),
+                ("k_scale", _vp), ("k_zero", _vp), ("k_sz_batch_stride", _i64), ("k_sz_row_stride", _i64),
+                ("k_bits", _i32), ("k_fmt", _i32), ("k_group", _i32), ("k_tokens", _i64),
+                ("v_code", _vp), ("v_code_batch_stride", _i64), ("v_code_row_stride", _i64),
+                ("v_scale", _vp), ("v_zero", _vp), ("v_sz_batch_stride", _i64), ("v_sz_row_stride", _i64),
+                ("v_bits", _i32), ("v_fmt", _i32), ("v_group", _i32), ("v_tokens", _i64),
+                ("k_tail", _vp), ("k_tail_batch_stride", _i64), ("k_tail_token_stride", _i64),
+                ("k_tail_slots", _i64), ("k_tail_len", _i64), ("k_tail_len_dev", _vp),
+                ("v_tail", _vp), ("v_tail_batch_stride", _i64), ("v_tail_token_stride", _i64),
+                ("v_tail_slots", _i64), ("v_tail_len", _i64), ("v_tail_len_dev", _vp),
+                ("mask", _vp), ("mask_stride", _i64),
+                ("samples", _i64), ("heads", _i32), ("heads_per_kv", _i32), ("D", _i64),
+                ("probs", _vp), ("probs_stride", _i64), ("out", _vp), ("out_stride", _i64)]
 
 
 class KVmixLibraryMissing(ImportError):
@@ -79,6 +100,10 @@ def load() -> ctypes.CDLL:
     L.kvmix_quantized_gemv.restype = i32
     L.kvmix_quantized_gemv.argtypes = [i32, vp, i64, i64, vp, i64, i64, vp, vp, i64, i64, i32, i32,
                                        i64, i32, i64, i64, i64, vp, i64, i64, vp, sz, vp]
+    L.kvmix_decode_attention_workspace_bytes.restype = sz
+    L.kvmix_decode_attention_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
+    L.kvmix_decode_attention.restype = i32
+    L.kvmix_decode_attention.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
     _lib = L
     return L
 

@@ -105,6 +105,37 @@ class KVmixAttention:
         return PackedKVCache(self.k_bits, self.v_bits, self.Vgroup_size, self.k_residual_ratio,
                              self.v_residual_ratio, self.residual_length, capacity, k_fmt, v_fmt)
 
+    def _decode_with_torch_glue(self, query_states, kc, ks, km, k_tail, vc, vs, vm, v_tail, k_group, k_fmt, v_fmt, n_rep,
+                                attention_mask):
+        """The decode branch composed as the reference composes it (models/modeling_llama_KVmix.py:180-211):
+        two quantized_gemm calls around torch's matmul / cat / softmax.  Used for several query
+        positions at once and for masks or dtypes the library's fused step does not take."""
+        D = query_states.shape[-1]
+        att_full = _grouped_matmul_qk(query_states, k_tail, n_rep)
+        if kc is not None:
+            att_quant = ops.quantized_gemm(k_group, query_states, kc, ks, km, self.k_bits, k_fmt)
+            attn_weights = torch.cat([att_quant.to(torch.float32), att_full.to(torch.float32)], dim=-1)
+        else:
+            attn_weights = att_full.to(torch.float32)
+        attn_weights = attn_weights / math.sqrt(D)
+        if attention_mask is not None:
+            if attention_mask.shape[-2:] != attn_weights.shape[-2:]:
+                raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
+                                 f"{attn_weights.shape}")
+            attn_weights = attn_weights + attention_mask
+            attn_weights = torch.clamp(attn_weights, min=torch.finfo(attn_weights.dtype).min)
+        attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
+
+        if vc is None:
+            attn_output = _grouped_matmul_pv(attn_weights, v_tail, n_rep)
+        else:
+            lv = v_tail.shape[-2]
+            tq = attn_weights.shape[-1] - lv
+            out_quant = ops.quantized_gemm(self.Vgroup_size, attn_weights[..., :tq], vc, vs, vm, self.v_bits, v_fmt)
+            out_full = _grouped_matmul_pv(attn_weights[..., tq:], v_tail, n_rep)
+            attn_output = out_quant + out_full
+        return attn_output, attn_weights
+
     # -- the step --------------------------------------------------------------------------
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
                 past_key_value=None, attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True):
@@ -132,29 +163,20 @@ class KVmixAttention:
                 v_tail = value_states if v_tail is None else torch.cat([v_tail, value_states], dim=2)
                 k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(k_tail, (kc, ks, km), v_tail, (vc, vs, vm))
 
-            att_full = _grouped_matmul_qk(query_states, k_tail, n_rep)
-            if kc is not None:
-                att_quant = ops.quantized_gemm(k_group, query_states, kc, ks, km, self.k_bits, k_fmt)
-                attn_weights = torch.cat([att_quant.to(torch.float32), att_full.to(torch.float32)], dim=-1)
-            else:
-                attn_weights = att_full.to(torch.float32)
-            attn_weights = attn_weights / math.sqrt(D)
-            if attention_mask is not None:
-                if attention_mask.shape[-2:] != attn_weights.shape[-2:]:
+            mask_ok = attention_mask is None or (attention_mask.dtype == torch.float32 and attention_mask.dim() == 4
+                                                 and attention_mask.shape[1] == 1)
+            if q_len == 1 and query_states.dtype == torch.float16 and D % 8 == 0 and mask_ok:
+                # the whole step in the library: logits over packed keys and fp16 tail, softmax,
+                # output over packed values and fp16 tail
+                if attention_mask is not None and attention_mask.shape[-2:] != (1, kv_seq_len):
                     raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
-                                     f"{attn_weights.shape}")
-                attn_weights = attn_weights + attention_mask
-                attn_weights = torch.clamp(attn_weights, min=torch.finfo(attn_weights.dtype).min)
-            attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
-
-            if vc is None:
-                attn_output = _grouped_matmul_pv(attn_weights, v_tail, n_rep)
+                                     f"{(B, nh, 1, kv_seq_len)}")
+                attn_output, attn_weights = ops.decode_attention(
+                    query_states, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, k_group, self.k_bits, self.Vgroup_size,
+                    self.v_bits, k_fmt, v_fmt, attention_mask)
             else:
-                lv = v_tail.shape[-2]
-                tq = attn_weights.shape[-1] - lv
-                out_quant = ops.quantized_gemm(self.Vgroup_size, attn_weights[..., :tq], vc, vs, vm, self.v_bits, v_fmt)
-                out_full = _grouped_matmul_pv(attn_weights[..., tq:], v_tail, n_rep)
-                attn_output = out_quant + out_full
+                attn_output, attn_weights = self._decode_with_torch_glue(
+                    query_states, kc, ks, km, k_tail, vc, vs, vm, v_tail, k_group, k_fmt, v_fmt, n_rep, attention_mask)
         else:
             # prompt: dense fp16 attention; the cache keeps the oldest tokens quantized
             # (models/modeling_llama_KVmix.py:213-266)

@@ -154,8 +154,8 @@ class GraphDecoder(Decoder):
     launch overhead, not by the GPU.  Between two flushes everything about a step is static except
     three numbers (the position and the lengths of the two fp16 tails); those live in device
     counters that the graph itself increments, the new token goes to slot `tail length` of a
-    fixed-size tail window through an indexed copy, and the window's unused slots are masked out of
-    the softmax.  A step in which some layer flushes runs eagerly (the flush changes the packed
+    fixed-size tail window through an indexed copy, and the attention step reads the tail lengths
+    from the counters, so that the window's unused slots get probability zero.  A step in which some layer flushes runs eagerly (the flush changes the packed
     lengths, which are launch arguments), after which the graph is captured again.
     Needs in-place caches (PackedKVCache) with a fixed residual window."""
 
@@ -175,7 +175,6 @@ class GraphDecoder(Decoder):
     # one decode step with static shapes; mutates the device counters
     def _static_step(self, ids: torch.Tensor) -> torch.Tensor:
         from . import ops
-        from .attention import _grouped_matmul_pv, _grouped_matmul_qk
 
         cfg, R = self.cfg, self.window
         B = ids.shape[0]
@@ -186,36 +185,20 @@ class GraphDecoder(Decoder):
         ang = self._pos.to(torch.float32)[:, None] * inv_freq[None, :]
         emb = torch.cat([ang, ang], dim=-1)
         cos, sin = emb.cos()[None, None].to(x.dtype), emb.sin()[None, None].to(x.dtype)
-        slots = torch.arange(R, device=dev)
-        neg = float("-inf")
         for li, lw in enumerate(self.w["layers"]):
             cache = self.caches[li]
             h = rms_norm(x, lw["input_norm"], cfg.rms_norm_eps)
             q, k, v = project_qkv(cfg, h, lw["wqkv"], cos, sin)
-            n_rep = cfg.num_heads // cfg.num_kv_heads
-
             kwin, vwin, _, _ = cache.tail_windows(R)
             klen, vlen = self._len[li]
             kwin.index_copy_(2, klen, k)
             vwin.index_copy_(2, vlen, v)
-            kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
-            tqk, tqv = cache.k_tokens, cache.v_tokens
-            width = max(tqk, tqv) + R  # room for either tail window behind either quantized part
-            parts = []
-            if tqk > 0:
-                parts.append(ops.quantized_gemm(cache.Kgroup_size, q, kc, ks, km, cache.k_bits, cache.k_fmt).to(torch.float32))
-            tail = _grouped_matmul_qk(q, kwin, n_rep).to(torch.float32)
-            parts.append(tail.masked_fill(slots > klen, neg))  # slots 0..klen hold tokens
-            if width - tqk - R > 0:
-                parts.append(torch.full((B, cfg.num_heads, 1, width - tqk - R), neg, device=dev, dtype=torch.float32))
-            wts = torch.cat(parts, dim=-1) / (D ** 0.5)
-            wts = F.softmax(wts, dim=-1, dtype=torch.float32).to(q.dtype)
-            out = _grouped_matmul_pv(wts[..., tqv:tqv + R], vwin, n_rep)  # unused slots have weight 0
-            if tqv > 0:
-                out = out + ops.quantized_gemm(cache.Vgroup_size, wts[..., :tqv], vc, vs, vm, cache.v_bits, cache.v_fmt)
-            klen.add_(1)
+            klen.add_(1)  # now the number of live slots, which is what the attention step reads
             vlen.add_(1)
-
+            kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
+            out, _ = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, cache.Kgroup_size, cache.k_bits,
+                                          cache.Vgroup_size, cache.v_bits, cache.k_fmt, cache.v_fmt,
+                                          k_tail_len=klen, v_tail_len=vlen)
             out = out.transpose(1, 2).reshape(B, 1, cfg.hidden_size)
             x = x + F.linear(out, lw["wo"])
             h = rms_norm(x, lw["post_norm"], cfg.rms_norm_eps)

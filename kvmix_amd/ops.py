@@ -275,6 +275,102 @@ def quantized_gemm(group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: 
     return out
 
 
+def decode_attention(q: torch.Tensor, k_packed, v_packed, k_tail: torch.Tensor, v_tail: torch.Tensor,
+                     k_group: int, k_bits: int, v_group: int, v_bits: int, k_fmt: int = _lib.FMT_REF,
+                     v_fmt: int = _lib.FMT_REF, attention_mask=None, k_tail_len=None, v_tail_len=None):
+    """One decode step of attention over the packed cache plus its fp16 tails, in four or five
+    launches (no reference operator: it is what models/modeling_llama_KVmix.py:180-211 composes
+    from quantized_gemm, matmul, cat and softmax).
+
+    q [B,nh,1,D] fp16; k_packed = (code [B,Hkv,D,Tk/vpw], scale, min) or None; v_packed =
+    (code [B,Hkv,Tv,D/vpw], scale, min) or None; k_tail, v_tail [B,Hkv,slots,D] fp16.
+    *_tail_len: None (every slot holds a token), an int, or a device int64 tensor of one element
+    read when the kernels run (for steps replayed from a captured graph).
+    attention_mask: None or fp32 [B,1,1,width].
+    Returns (out [B,nh,1,D] fp16, probs [B,nh,1,width] fp16), width = max(Tk + key slots, Tv + value slots)."""
+    import ctypes
+
+    if q.dim() != 4 or q.shape[2] != 1:
+        raise RuntimeError("decode_attention takes one query position: q must be [B, nh, 1, D]")
+    for t in (q, k_tail, v_tail):
+        if t.dtype != torch.float16:
+            raise RuntimeError(f"expected scalar type Half but found {t.dtype}")
+    _need_gpu(q, k_tail, v_tail)
+    _check_bits(k_bits)
+    _check_bits(v_bits)
+    L = _lib.load()
+    B, nh, _, D = q.shape
+    nkv = k_tail.shape[1]
+    if nkv == 0 or nh % nkv != 0:
+        raise RuntimeError("Total heads must be divisible by KV heads")
+    st = _lib.DecodeAttn()
+    q, q_bs, _ = _batched3(q)
+    st.q, st.q_stride = q.data_ptr(), q_bs
+    keep = [q]
+
+    def packed(prefix, triple, tokens_of):
+        if triple is None or triple[0] is None:
+            setattr(st, prefix + "_tokens", 0)
+            return
+        code, scale, zero = triple
+        code, c_bs, c_rs = _batched3(code)
+        scale, s_bs, s_rs = _batched3(scale)
+        zero, z_bs, z_rs = _batched3(zero)
+        if (z_bs, z_rs) != (s_bs, s_rs):
+            scale, zero = scale.contiguous(), zero.contiguous()
+            scale, s_bs, s_rs = _batched3(scale)
+            zero, z_bs, z_rs = _batched3(zero)
+        keep.extend((code, scale, zero))
+        setattr(st, prefix + "_code", code.data_ptr())
+        setattr(st, prefix + "_code_batch_stride", c_bs)
+        setattr(st, prefix + "_code_row_stride", c_rs)
+        setattr(st, prefix + "_scale", scale.data_ptr())
+        setattr(st, prefix + "_zero", zero.data_ptr())
+        setattr(st, prefix + "_sz_batch_stride", s_bs)
+        setattr(st, prefix + "_sz_row_stride", s_rs)
+        setattr(st, prefix + "_tokens", tokens_of(code, zero))
+
+    packed("k", k_packed, lambda code, zero: zero.shape[-1] * k_group)
+    packed("v", v_packed, lambda code, zero: code.shape[2])
+    st.k_bits, st.k_fmt, st.k_group = k_bits, k_fmt, k_group
+    st.v_bits, st.v_fmt, st.v_group = v_bits, v_fmt, v_group
+
+    def tail(prefix, t, length):
+        t, t_bs, t_ts = _batched3(t)
+        keep.append(t)
+        setattr(st, prefix + "_tail", t.data_ptr())
+        setattr(st, prefix + "_tail_batch_stride", t_bs)
+        setattr(st, prefix + "_tail_token_stride", t_ts)
+        setattr(st, prefix + "_tail_slots", t.shape[2])
+        if torch.is_tensor(length):
+            if length.dtype != torch.int64 or length.numel() != 1 or not length.is_cuda:
+                raise RuntimeError("a device-side tail length must be one int64 element on the GPU")
+            setattr(st, prefix + "_tail_len_dev", length.data_ptr())
+        else:
+            setattr(st, prefix + "_tail_len", t.shape[2] if length is None else int(length))
+
+    tail("k", k_tail, k_tail_len)
+    tail("v", v_tail, v_tail_len)
+    width = max(st.k_tokens + st.k_tail_slots, st.v_tokens + st.v_tail_slots)
+    if attention_mask is not None:
+        if attention_mask.dtype != torch.float32 or tuple(attention_mask.shape) != (B, 1, 1, width):
+            raise RuntimeError(f"attention_mask must be fp32 of shape {(B, 1, 1, width)}")
+        if attention_mask.stride(3) != 1:
+            attention_mask = attention_mask.contiguous()
+        keep.append(attention_mask)
+        st.mask, st.mask_stride = attention_mask.data_ptr(), attention_mask.stride(0) if B > 1 else width
+    st.samples, st.heads, st.heads_per_kv, st.D = B * nh, nh, nh // nkv, D
+    probs = torch.empty((B, nh, 1, width), dtype=torch.float16, device=q.device)
+    out = torch.empty((B, nh, 1, D), dtype=torch.float16, device=q.device)
+    st.probs, st.probs_stride, st.out, st.out_stride = probs.data_ptr(), width, out.data_ptr(), D
+    ws_bytes = L.kvmix_decode_attention_workspace_bytes(ctypes.byref(st))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    with torch.cuda.device(q.device):
+        _lib.check(L.kvmix_decode_attention(ctypes.byref(st), ws.data_ptr() if ws is not None else None, ws_bytes,
+                                            _stream(q)))
+    return out, probs
+
+
 def _append_checks(input, prev_scale, prev_min):
     if input.dim() != 4:
         raise RuntimeError("input_tensor must be a 4D tensor")

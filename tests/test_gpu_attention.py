@@ -95,3 +95,95 @@ def test_mask_shape_error(dev):
     q = torch.zeros(1, 2, 1, 128, dtype=torch.float16, device=dev)
     with pytest.raises(ValueError, match="does not match"):
         att(q, q, q, (None,) * 8 + (0,), attention_mask=torch.zeros(1, 1, 1, 7, device=dev))
+
+
+def _cache_after_steps(att, dev, rng, B, nh, nkv, D, steps):
+    cache = att.new_cache(capacity=512)
+    for step in range(steps):
+        k = to_t(kv_like(rng, (B, nkv, 1, D)), dev)
+        v = to_t(kv_like(rng, (B, nkv, 1, D)), dev)
+        cache.append(k, v)
+    return cache
+
+
+@pytest.mark.parametrize("k_bits,v_bits,nkv", [(4, 2, 4), (3, 4, 2), (1, 2, 1)])
+def test_library_step_equals_the_torch_composition(dev, k_bits, v_bits, nkv):
+    """ops.decode_attention against the same step composed from quantized_gemm and torch's matmul /
+    cat / softmax (the way the reference composes it), with and without a padding mask."""
+    from kvmix_amd import ops
+    from kvmix_amd.attention import KVmixAttention
+
+    rng = np.random.default_rng(70 + k_bits)
+    B, nh, D = 2, 4, 128
+    att = KVmixAttention(k_bits, v_bits, residual_length=48)
+    cache = _cache_after_steps(att, dev, rng, B, nh, nkv, D, 150)
+    kc, k_tail, ks, km, vc, v_tail, vs, vm, n = cache.as_tuple()
+    assert kc is not None and vc is not None and k_tail.shape[2] > 0
+    q = to_t(rng.standard_normal((B, nh, 1, D)).astype(np.float16), dev)
+    mask = torch.zeros(B, 1, 1, n, device=dev)
+    mask[1, :, :, :40] = torch.finfo(torch.float32).min  # left padding of the second sequence
+    for m in (None, mask):
+        out_l, p_l = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, cache.Kgroup_size, k_bits,
+                                          cache.Vgroup_size, v_bits, attention_mask=m)
+        out_t, p_t = att._decode_with_torch_glue(q, kc, ks, km, k_tail, vc, vs, vm, v_tail, cache.Kgroup_size, 0, 0,
+                                                 nh // nkv, m)
+        torch.testing.assert_close(p_l, p_t, rtol=5e-3, atol=2e-5)
+        torch.testing.assert_close(out_l, out_t, rtol=5e-3, atol=5e-3)
+        if m is not None:
+            assert float(p_l[1, :, :, :40].abs().max()) == 0.0
+        assert abs(float(p_l.float().sum(-1).mean()) - 1.0) < 2e-3
+
+
+def test_tail_windows_with_device_side_lengths(dev):
+    """Fixed-size tail windows whose live lengths are read from device memory give, position by
+    position, the bits of the exact-size call; slots past the lengths hold probability zero."""
+    from kvmix_amd import ops
+    from kvmix_amd.attention import KVmixAttention
+
+    rng = np.random.default_rng(81)
+    B, nh, nkv, D, R = 2, 8, 2, 128, 64
+    att = KVmixAttention(3, 2, residual_length=R)   # reference 3-bit keys: the two tails differ in length
+    cache = _cache_after_steps(att, dev, rng, B, nh, nkv, D, 200)
+    kc, k_tail, ks, km, vc, v_tail, vs, vm, n = cache.as_tuple()
+    lk, lv = k_tail.shape[2], v_tail.shape[2]
+    assert lk != lv and cache.k_tokens != cache.v_tokens
+    q = to_t(rng.standard_normal((B, nh, 1, D)).astype(np.float16), dev)
+    args = (cache.Kgroup_size, 3, cache.Vgroup_size, 2)
+    out_e, p_e = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, *args)
+    kwin, vwin, nk, nv = cache.tail_windows(R)
+    assert (nk, nv) == (lk, lv)
+    kwin[:, :, lk:] = 1000.0   # whatever lies in the unused slots must not matter
+    vwin[:, :, lv:] = -1000.0
+    klen = torch.tensor([lk], dtype=torch.int64, device=dev)
+    vlen = torch.tensor([lv], dtype=torch.int64, device=dev)
+    out_w, p_w = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, *args, k_tail_len=klen, v_tail_len=vlen)
+    assert p_w.shape[-1] == max(cache.k_tokens, cache.v_tokens) + R
+    assert torch.equal(p_w[..., :n], p_e) and float(p_w[..., n:].abs().max()) == 0.0
+    assert torch.equal(out_w, out_e)
+    # host-side lengths for the same windows
+    out_h, p_h = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, *args, k_tail_len=lk, v_tail_len=lv)
+    assert torch.equal(out_h, out_e) and torch.equal(p_h[..., :n], p_e)
+
+
+def test_library_step_without_a_quantized_part_and_argument_errors(dev):
+    from kvmix_amd import ops
+
+    rng = np.random.default_rng(5)
+    B, nh, nkv, D, L = 1, 4, 2, 128, 9
+    q = to_t(rng.standard_normal((B, nh, 1, D)).astype(np.float16), dev)
+    k = to_t(rng.standard_normal((B, nkv, L, D)).astype(np.float16), dev)
+    v = to_t(rng.standard_normal((B, nkv, L, D)).astype(np.float16), dev)
+    out, p = ops.decode_attention(q, None, None, k, v, 32, 4, 32, 4)
+    kk = k.float().repeat_interleave(nh // nkv, 1)
+    vv = v.float().repeat_interleave(nh // nkv, 1)
+    w = torch.softmax((q.float() @ kk.transpose(2, 3)).half().float() / np.float32(np.sqrt(D)), -1)
+    torch.testing.assert_close(p.float(), w, rtol=2e-3, atol=2e-5)
+    torch.testing.assert_close(out.float(), w.half().float() @ vv, rtol=2e-3, atol=2e-3)
+    with pytest.raises(RuntimeError, match="one query position"):
+        ops.decode_attention(q.expand(B, nh, 2, D), None, None, k, v, 32, 4, 32, 4)
+    with pytest.raises(RuntimeError, match="KV heads"):
+        ops.decode_attention(q[:, :3], None, None, k, v, 32, 4, 32, 4)
+    with pytest.raises(RuntimeError, match="attention_mask"):
+        ops.decode_attention(q, None, None, k, v, 32, 4, 32, 4, attention_mask=torch.zeros(B, 1, 1, L + 1, device=dev))
+    with pytest.raises(RuntimeError):  # keys and values must cover the same positions
+        ops.decode_attention(q, None, None, k, v[:, :, :5], 32, 4, 32, 4)
