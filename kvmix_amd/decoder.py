@@ -170,6 +170,7 @@ class GraphDecoder(Decoder):
         self._warm = False
         self._ids = self._logits = None
         self._pos = self._len = None
+        self._counters = {}
         self.graph_steps = self.eager_steps = self.captures = 0
 
     # one decode step with static shapes; mutates the device counters
@@ -190,37 +191,48 @@ class GraphDecoder(Decoder):
             h = rms_norm(x, lw["input_norm"], cfg.rms_norm_eps)
             q, k, v = project_qkv(cfg, h, lw["wqkv"], cos, sin)
             kwin, vwin, _, _ = cache.tail_windows(R)
-            klen, vlen = self._len[li]
-            kwin.index_copy_(2, klen, k)
-            vwin.index_copy_(2, vlen, v)
-            klen.add_(1)  # now the number of live slots, which is what the attention step reads
-            vlen.add_(1)
+            (kslot, klive), (vslot, vlive) = self._len[li]
+            kwin.index_copy_(2, kslot, k)
+            vwin.index_copy_(2, vslot, v)
             kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
             out, _ = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, cache.Kgroup_size, cache.k_bits,
                                           cache.Vgroup_size, cache.v_bits, cache.k_fmt, cache.v_fmt,
-                                          k_tail_len=klen, v_tail_len=vlen)
+                                          k_tail_len=klive, v_tail_len=vlive)
             out = out.transpose(1, 2).reshape(B, 1, cfg.hidden_size)
             x = x + F.linear(out, lw["wo"])
             h = rms_norm(x, lw["post_norm"], cfg.rms_norm_eps)
             x = x + mlp(h, lw["w_gate_up"], lw["w_down"])
         self._pos.add_(1)
+        for slot, live in self._counters.values():
+            slot.add_(1)
+            live.add_(1)
         x = rms_norm(x[:, -1], self.w["norm"], cfg.rms_norm_eps)
         return F.linear(x, self.w["lm_head"]).to(torch.float32)
 
     def _sync_counters(self) -> None:
+        """Device counters for the coming steps.  Tails of equal length stay equal until the next
+        flush, so they share one pair of counters (slot of the next token, live slots once it is
+        written): a step then increments a handful of counters instead of two per layer."""
+        dev = self._pos.device
         self._pos.fill_(self.position)
-        for li, cache in enumerate(self.caches):
+        lengths = []
+        for cache in self.caches:
             _, _, nk, nv = cache.tail_windows(self.window)
-            self._len[li][0].fill_(nk)
-            self._len[li][1].fill_(nv)
+            lengths.append((nk, nv))
+        for n in {n for pair in lengths for n in pair}:
+            if n not in self._counters:
+                self._counters[n] = (torch.empty(1, dtype=torch.int64, device=dev), torch.empty(1, dtype=torch.int64, device=dev))
+        self._counters = {n: c for n, c in self._counters.items() if any(n in pair for pair in lengths)}
+        for n, (slot, live) in self._counters.items():
+            slot.fill_(n)
+            live.fill_(n + 1)
+        self._len = [(self._counters[nk], self._counters[nv]) for nk, nv in lengths]
 
     def _capture(self, ids: torch.Tensor) -> None:
         dev = ids.device
         if self._ids is None:
             self._ids = torch.zeros_like(ids)
             self._pos = torch.zeros(1, dtype=torch.int64, device=dev)
-            self._len = [(torch.zeros(1, dtype=torch.int64, device=dev), torch.zeros(1, dtype=torch.int64, device=dev))
-                         for _ in self.caches]
         self._ids.copy_(ids)
         self._sync_counters()  # (also settles where the tail windows lie before anything is recorded)
         side = torch.cuda.Stream(device=dev)
