@@ -1684,14 +1684,29 @@ __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
 // (dequantization_gemv_cuda.cu:23-24).
 // ---------------------------------------------------------------------------------------
 template <int MODE>
-__global__ void __launch_bounds__(256) gemv_generic(GemvArgs a)
+struct GenericCfg {
+    static constexpr int VALS = MODE == 30 ? 32 : (MODE == 3 ? 11 : 32 / MODE);
+    static constexpr int THREADS = VALS == 32 ? 256 : 512;  // (THREADS * (VALS + 1) floats of LDS stay under 64 KB)
+};
+
+// A block covers UB = 2^ub_log2 units; when that is fewer than the block has threads, the
+// remaining factor KS = THREADS / UB slices K: thread (unit, slice) walks rows slice, slice + KS, ...
+// and the slices are summed through LDS.  Short rows (few quantized tokens) would otherwise leave
+// a handful of threads per output row walking all of K one after the other.
+template <int MODE>
+__global__ void __launch_bounds__(GenericCfg<MODE>::THREADS) gemv_generic(GemvArgs a, int ub_log2)
 {
     constexpr int BITS = MODE == 30 ? 3 : MODE;
-    constexpr int VALS = MODE == 30 ? 32 : (MODE == 3 ? 11 : 32 / BITS);
+    constexpr int VALS = GenericCfg<MODE>::VALS;
+    constexpr int THREADS = GenericCfg<MODE>::THREADS;
     constexpr int WORDS = MODE == 30 ? 3 : 1;
-    const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    extern __shared__ float red[];  // [THREADS][VALS + 1] when K is sliced
+    const int tid = threadIdx.x;
+    const int UB = 1 << ub_log2, KS = THREADS >> ub_log2;
+    const int ul = tid & (UB - 1), slice = tid >> ub_log2;
+    const int64_t u = (int64_t)blockIdx.x * UB + ul;
     const int64_t units = a.N / VALS;
-    if (u >= units) return;
+    const bool live = u < units;
     const int64_t sample = blockIdx.y;
     const int64_t m = blockIdx.z;
     const int64_t kv = sample / a.heads_per_kv;
@@ -1704,26 +1719,51 @@ __global__ void __launch_bounds__(256) gemv_generic(GemvArgs a)
 #pragma unroll
     for (int i = 0; i < VALS; i++) acc[i] = 0.f;
     float zsum = 0.f;
-    for (int64_t k = 0; k < a.K; k++) {
-        uint32_t w[WORDS];
+    if (live) {
+#pragma unroll 4
+        for (int64_t k = slice; k < a.K; k += KS) {
+            uint32_t w[WORDS];
 #pragma unroll
-        for (int t = 0; t < WORDS; t++) w[t] = cp[k * a.c_rs + t];
-        const float xv = __half2float(xp[k]);
-        const float qs = xv * __half2float(sp[k * a.s_rs]);
-        zsum = fmaf(xv, __half2float(zp[k * a.s_rs]), zsum);
-        if constexpr (MODE == 30) {
-            accumulate_unit<30>(w, qs, acc);
-        } else if constexpr (MODE == 3) {
-            accumulate_unit<3>(w, qs, acc);
-        } else {
+            for (int t = 0; t < WORDS; t++) w[t] = cp[k * a.c_rs + t];
+            const float xv = __half2float(xp[k]);
+            const float qs = xv * __half2float(sp[k * a.s_rs]);
+            zsum = fmaf(xv, __half2float(zp[k * a.s_rs]), zsum);
+            if constexpr (MODE == 30) {
+                accumulate_unit<30>(w, qs, acc);
+            } else if constexpr (MODE == 3) {
+                accumulate_unit<3>(w, qs, acc);
+            } else {
 #pragma unroll
-            for (int i = 0; i < VALS; i++)
-                acc[i] = fmaf(qs, (float)((w[0] >> (i * BITS)) & ((1u << BITS) - 1u)), acc[i]);
+                for (int i = 0; i < VALS; i++)
+                    acc[i] = fmaf(qs, (float)((w[0] >> (i * BITS)) & ((1u << BITS) - 1u)), acc[i]);
+            }
         }
     }
-    __half *op = a.out + sample * a.o_bs + m * a.o_rs + u * VALS;
+    __half *orow = a.out + sample * a.o_bs + m * a.o_rs;
+    if (KS == 1) {  // (the same for every thread of the grid)
+        if (live) {
 #pragma unroll
-    for (int i = 0; i < VALS; i++) op[i] = __float2half_rn(fmaf(acc[i], Fmt<MODE>::OUT_SCALE, zsum));
+            for (int i = 0; i < VALS; i++) orow[u * VALS + i] = __float2half_rn(fmaf(acc[i], Fmt<MODE>::OUT_SCALE, zsum));
+        }
+        return;
+    }
+    float *mine = red + tid * (VALS + 1);
+#pragma unroll
+    for (int i = 0; i < VALS; i++) mine[i] = acc[i];
+    mine[VALS] = zsum;
+    __syncthreads();
+    for (int o = tid; o < UB * VALS; o += THREADS) {
+        const int ul2 = o / VALS, i = o % VALS;
+        const int64_t u2 = (int64_t)blockIdx.x * UB + ul2;
+        if (u2 >= units) continue;
+        float sum = 0.f, z = 0.f;
+        for (int sl = 0; sl < KS; sl++) {
+            const float *r = red + (sl * UB + ul2) * (VALS + 1);
+            sum += r[i];
+            z += r[VALS];
+        }
+        orow[u2 * VALS + i] = __float2half_rn(fmaf(sum, Fmt<MODE>::OUT_SCALE, z));
+    }
 }
 
 // --------------------------- host side ---------------------------
@@ -2011,10 +2051,15 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 template <int MODE>
 static void launch_generic(GemvArgs &a, int64_t samples, hipStream_t st)
 {
-    constexpr int VALS = MODE == 30 ? 32 : (MODE == 3 ? 11 : 32 / MODE);
+    constexpr int VALS = GenericCfg<MODE>::VALS;
+    constexpr int THREADS = GenericCfg<MODE>::THREADS;
     const int64_t units = a.N / VALS;
-    const dim3 grid((unsigned)((units + 255) / 256), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL(gemv_generic<MODE>, grid, dim3(256), 0, st, a);
+    int ub_log2 = 0;
+    while ((1 << ub_log2) < THREADS && (1 << ub_log2) < units) ub_log2++;
+    const int ub = 1 << ub_log2;
+    const size_t lds = ub < THREADS ? (size_t)THREADS * (VALS + 1) * sizeof(float) : 0;
+    const dim3 grid((unsigned)((units + ub - 1) / ub), (unsigned)samples, (unsigned)a.M);
+    hipLaunchKernelGGL(gemv_generic<MODE>, grid, dim3(THREADS), lds, st, a, ub_log2);
 }
 
 }  // namespace kvmix
