@@ -28,6 +28,10 @@ from . import ops
 from .cache import RESIDUAL_RATIO_BY_BITS, PackedKVCache, flush_length  # noqa: F401 (re-exported)
 
 
+# longest fp16 tail for which a decode step goes through the library's fused step
+LIBRARY_STEP_MAX_TAIL = 512
+
+
 def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
     """models/modeling_llama_KVmix.py:19-28 (kept for callers that still want the copy)."""
     batch, num_key_value_heads, slen, head_dim = hidden_states.shape
@@ -165,7 +169,10 @@ class KVmixAttention:
 
             mask_ok = attention_mask is None or (attention_mask.dtype == torch.float32 and attention_mask.dim() == 4
                                                  and attention_mask.shape[1] == 1)
-            if q_len == 1 and query_states.dtype == torch.float16 and D % 8 == 0 and mask_ok:
+            # (a long fp16 tail -- the ratio rule right after a long prompt -- is a plain fp16 GEMV over
+            # hundreds of KB per head; torch's batched matmul streams that better than one block per head)
+            short_tails = max(k_tail.shape[2], v_tail.shape[2]) <= LIBRARY_STEP_MAX_TAIL
+            if q_len == 1 and query_states.dtype == torch.float16 and D % 8 == 0 and mask_ok and short_tails:
                 # the whole step in the library: logits over packed keys and fp16 tail, softmax,
                 # output over packed values and fp16 tail
                 if attention_mask is not None and attention_mask.shape[-2:] != (1, kv_seq_len):

@@ -58,8 +58,11 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scrat
     return r;
 }
 
-// grid = samples, block = 256.  Sixteen lanes share a tail token (eight head dimensions each), so a
-// wave has four tokens in flight per load and a block sixteen.
+// grid = samples, block = 256.  Sixteen lanes share a tail token (eight head dimensions each) and every
+// lane group has four tokens in flight, so a block covers 64 tail tokens per step.  The softmax keeps
+// a row of up to 16384 entries in registers (eight 8-entry vectors per thread): one read, one write.
+constexpr int kRowVecs = 8;
+
 __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
 {
     __shared__ float scratch[4];
@@ -74,20 +77,29 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
     const int sub = tid % 16;
     const uint16_t *qp = a.q + sample * a.q_bs;
     const uint16_t *kt = a.k_tail + kv * a.kt_bs;
-    for (int64_t j0 = 0; j0 < a.k_slots; j0 += 16) {
-        const int64_t j = j0 + tid / 16;
-        float dot = 0.f;
-        if (j < k_len) {
-            for (int d = sub * 8; d < D; d += 128) {
-                const H8 kk = *reinterpret_cast<const H8 *>(kt + j * a.kt_ts + d);
-                const H8 qq = *reinterpret_cast<const H8 *>(qp + d);
+    for (int64_t j0 = 0; j0 < a.k_slots; j0 += 64) {
+        float dot[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int d = sub * 8; d < D; d += 128) {
+            const H8 qq = *reinterpret_cast<const H8 *>(qp + d);
+            H8 kk[4];
 #pragma unroll
-                for (int i = 0; i < 8; i++) dot = fmaf(h16_to_f32(qq.v[i]), h16_to_f32(kk.v[i]), dot);
+            for (int t = 0; t < 4; t++) {
+                const int64_t j = j0 + 16 * t + tid / 16;
+                kk[t] = *reinterpret_cast<const H8 *>(kt + (j < k_len ? j : 0) * a.kt_ts + d);  // (slot 0 stands in past the end)
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) dot[t] = fmaf(h16_to_f32(qq.v[i]), h16_to_f32(kk[t].v[i]), dot[t]);
             }
         }
 #pragma unroll
-        for (int o = 8; o >= 1; o >>= 1) dot += __shfl_xor(dot, o);
-        if (sub == 0 && j < a.k_slots) row[a.k_tokens + j] = j < k_len ? f32_to_h16(dot) : (uint16_t)0xfc00u;  // -inf
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int o = 8; o >= 1; o >>= 1) dot[t] += __shfl_xor(dot[t], o);
+            const int64_t j = j0 + 16 * t + tid / 16;
+            if (sub == 0 && j < a.k_slots) row[a.k_tokens + j] = j < k_len ? f32_to_h16(dot[t]) : (uint16_t)0xfc00u;  // -inf
+        }
     }
     // entries between the key window and the row's width (a value window that reaches further)
     for (int64_t i = a.k_tokens + a.k_slots + tid; i < a.width; i += 256) row[i] = (uint16_t)0xfc00u;
@@ -95,18 +107,68 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
 
     // 2. softmax of the row in fp32: x = fp32(logit) / sqrt(D) (+ mask, clamped to the lowest finite value)
     const float *mrow = a.mask ? a.mask + (sample / a.heads) * a.mask_bs : nullptr;
-    auto value = [&](int64_t i) {
-        float x = h16_to_f32(row[i]) * a.inv_sqrt_d;
+    auto value = [&](int64_t i, uint16_t h) {
+        float x = h16_to_f32(h) * a.inv_sqrt_d;
         if (mrow) x = fmaxf(x + mrow[i], -3.4028234663852886e38f);
         return x;
     };
+    if (a.width <= (int64_t)256 * 8 * kRowVecs) {
+        // thread t holds entries 8*(256*v + t) .. +7 of vector round v; a ragged end is read entry by entry
+        float x[kRowVecs][8];
+#pragma unroll
+        for (int v = 0; v < kRowVecs; v++) {
+            const int64_t i0 = ((int64_t)v * 256 + tid) * 8;
+            if (i0 + 8 <= a.width) {
+                const H8 h = *reinterpret_cast<const H8 *>(row + i0);
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[v][i] = value(i0 + i, h.v[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[v][i] = i0 + i < a.width ? value(i0 + i, row[i0 + i]) : -INFINITY;
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < kRowVecs; v++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) mx = fmaxf(mx, x[v][i]);
+        }
+        mx = block_reduce(mx, true, scratch);
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < kRowVecs; v++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                x[v][i] = expf(x[v][i] - mx);
+                sum += x[v][i];
+            }
+        }
+        sum = block_reduce(sum, false, scratch);
+#pragma unroll
+        for (int v = 0; v < kRowVecs; v++) {
+            const int64_t i0 = ((int64_t)v * 256 + tid) * 8;
+            if (i0 + 8 <= a.width) {
+                H8 h;
+#pragma unroll
+                for (int i = 0; i < 8; i++) h.v[i] = f32_to_h16(x[v][i] / sum);
+                *reinterpret_cast<H8 *>(row + i0) = h;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    if (i0 + i < a.width) row[i0 + i] = f32_to_h16(x[v][i] / sum);
+                }
+            }
+        }
+        return;
+    }
+    // longer rows: three passes over the row (it stays in L2)
     float mx = -INFINITY;
-    for (int64_t i = tid; i < a.width; i += 256) mx = fmaxf(mx, value(i));
+    for (int64_t i = tid; i < a.width; i += 256) mx = fmaxf(mx, value(i, row[i]));
     mx = block_reduce(mx, true, scratch);
     float sum = 0.f;
-    for (int64_t i = tid; i < a.width; i += 256) sum += expf(value(i) - mx);
+    for (int64_t i = tid; i < a.width; i += 256) sum += expf(value(i, row[i]) - mx);
     sum = block_reduce(sum, false, scratch);
-    for (int64_t i = tid; i < a.width; i += 256) row[i] = f32_to_h16(expf(value(i) - mx) / sum);
+    for (int64_t i = tid; i < a.width; i += 256) row[i] = f32_to_h16(expf(value(i, row[i]) - mx) / sum);
 }
 
 // grid = samples, block = 256: thread t owns head dimensions 8*(t%16).. of the tokens t/16, t/16+16, ...
@@ -126,11 +188,21 @@ __global__ void __launch_bounds__(256) attn_tail_output(AttnArgs a)
         const int d = d0 + sub * 8;
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (d < a.D) {
-            for (int64_t j = grp; j < v_len; j += 16) {
-                const float p = h16_to_f32(prow[j]);
-                const H8 vv = *reinterpret_cast<const H8 *>(vt + j * a.vt_ts + d);
+            for (int64_t j0 = grp; j0 < v_len; j0 += 64) {
+                float p[4];
+                H8 vv[4];
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[i] = fmaf(p, h16_to_f32(vv.v[i]), acc[i]);
+                for (int t = 0; t < 4; t++) {
+                    const int64_t j = j0 + 16 * t;
+                    const bool in = j < v_len;
+                    p[t] = in ? h16_to_f32(prow[j]) : 0.f;
+                    vv[t] = *reinterpret_cast<const H8 *>(vt + (in ? j : j0) * a.vt_ts + d);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[i] = fmaf(p[t], h16_to_f32(vv[t].v[i]), acc[i]);
+                }
             }
         }
         __syncthreads();

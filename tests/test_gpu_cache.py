@@ -73,7 +73,9 @@ def test_inplace_prompt_then_decode(oracle, dev):
         out_o, p_o, cache_o = oracle.attention_decode_step(q, k, v, cache_o, 3, 2, 0.2, 0.2, group_size=g)
         out_i, p_i, _ = att(to_t(q, dev), to_t(k, dev), to_t(v, dev), cache_i)
         same_cache(cache_i.as_tuple(), cache_o)
-        np.testing.assert_allclose(out_i.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
+        # the quantized and the fp16-tail halves of the output are rounded to fp16 before they are added
+        # and may cancel; with |V| up to ~40 in the outlier channels one fp16 ulp of a half is 0.0078
+        np.testing.assert_allclose(out_i.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=1.6e-2)
 
 
 def test_inplace_dense3_formats(oracle, dev):
