@@ -28,8 +28,9 @@ from . import ops
 from .cache import RESIDUAL_RATIO_BY_BITS, PackedKVCache, flush_length  # noqa: F401 (re-exported)
 
 
-# longest fp16 tail for which a decode step goes through the library's fused step
-LIBRARY_STEP_MAX_TAIL = 512
+# longest fp16 tail for which a decode step goes through the library's fused step (one block per
+# (batch, head) walks the tail; measured faster than torch's composition up to a few thousand tokens)
+LIBRARY_STEP_MAX_TAIL = 16384
 
 
 def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
@@ -169,8 +170,6 @@ class KVmixAttention:
 
             mask_ok = attention_mask is None or (attention_mask.dtype == torch.float32 and attention_mask.dim() == 4
                                                  and attention_mask.shape[1] == 1)
-            # (a long fp16 tail -- the ratio rule right after a long prompt -- is a plain fp16 GEMV over
-            # hundreds of KB per head; torch's batched matmul streams that better than one block per head)
             short_tails = max(k_tail.shape[2], v_tail.shape[2]) <= LIBRARY_STEP_MAX_TAIL
             if q_len == 1 and query_states.dtype == torch.float16 and D % 8 == 0 and mask_ok and short_tails:
                 # the whole step in the library: logits over packed keys and fp16 tail, softmax,

@@ -40,9 +40,14 @@ struct __attribute__((packed, aligned(2))) H8 {
     uint16_t v[8];
 };
 
+// One block per (batch, head) and nothing else resident on its CU: the kernels are chains of short
+// latency-bound phases, so the block is as wide as it can be (16 waves) to shorten each phase.
+constexpr int kAttnThreads = 1024;
+constexpr int kAttnGroups = kAttnThreads / 16;  // 16-lane groups, one tail token each
+
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scratch)
 {
-    // 256 threads = 4 waves; xor-shuffles inside the wave, then four values through LDS
+    // kAttnThreads / 64 waves; xor-shuffles inside the wave, then one value per wave through LDS
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) {
         const float other = __shfl_xor(v, o);
@@ -54,18 +59,19 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scrat
     __syncthreads();
     float r = scratch[0];
 #pragma unroll
-    for (int w = 1; w < 4; w++) r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+    for (int w = 1; w < kAttnThreads / kWave; w++) r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
     return r;
 }
 
-// grid = samples, block = 256.  Sixteen lanes share a tail token (eight head dimensions each) and every
-// lane group has four tokens in flight, so a block covers 64 tail tokens per step.  The softmax keeps
-// a row of up to 16384 entries in registers (eight 8-entry vectors per thread): one read, one write.
-constexpr int kRowVecs = 8;
+// grid = samples.  Sixteen lanes share a tail token (eight head dimensions each) and every lane group
+// has two tokens in flight, so a block covers 128 tail tokens per step.  The softmax keeps a row of up
+// to 16384 entries in registers (two 8-entry vectors per thread): one read, one write.
+constexpr int kRowVecs = 2;
+constexpr int kTailUnroll = 2;
 
-__global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
+__global__ void __launch_bounds__(kAttnThreads) attn_tail_softmax(AttnArgs a)
 {
-    __shared__ float scratch[4];
+    __shared__ float scratch[kAttnThreads / kWave];
     const int64_t sample = blockIdx.x;
     const int64_t kv = sample / a.heads_per_kv;
     const int tid = threadIdx.x;
@@ -77,32 +83,32 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
     const int sub = tid % 16;
     const uint16_t *qp = a.q + sample * a.q_bs;
     const uint16_t *kt = a.k_tail + kv * a.kt_bs;
-    for (int64_t j0 = 0; j0 < a.k_slots; j0 += 64) {
-        float dot[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t j0 = 0; j0 < a.k_slots; j0 += kAttnGroups * kTailUnroll) {
+        float dot[kTailUnroll] = {};
         for (int d = sub * 8; d < D; d += 128) {
             const H8 qq = *reinterpret_cast<const H8 *>(qp + d);
-            H8 kk[4];
+            H8 kk[kTailUnroll];
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const int64_t j = j0 + 16 * t + tid / 16;
+            for (int t = 0; t < kTailUnroll; t++) {
+                const int64_t j = j0 + kAttnGroups * t + tid / 16;
                 kk[t] = *reinterpret_cast<const H8 *>(kt + (j < k_len ? j : 0) * a.kt_ts + d);  // (slot 0 stands in past the end)
             }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < kTailUnroll; t++) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) dot[t] = fmaf(h16_to_f32(qq.v[i]), h16_to_f32(kk[t].v[i]), dot[t]);
             }
         }
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < kTailUnroll; t++) {
 #pragma unroll
             for (int o = 8; o >= 1; o >>= 1) dot[t] += __shfl_xor(dot[t], o);
-            const int64_t j = j0 + 16 * t + tid / 16;
+            const int64_t j = j0 + kAttnGroups * t + tid / 16;
             if (sub == 0 && j < a.k_slots) row[a.k_tokens + j] = j < k_len ? f32_to_h16(dot[t]) : (uint16_t)0xfc00u;  // -inf
         }
     }
     // entries between the key window and the row's width (a value window that reaches further)
-    for (int64_t i = a.k_tokens + a.k_slots + tid; i < a.width; i += 256) row[i] = (uint16_t)0xfc00u;
+    for (int64_t i = a.k_tokens + a.k_slots + tid; i < a.width; i += kAttnThreads) row[i] = (uint16_t)0xfc00u;
     __syncthreads();
 
     // 2. softmax of the row in fp32: x = fp32(logit) / sqrt(D) (+ mask, clamped to the lowest finite value)
@@ -112,12 +118,12 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
         if (mrow) x = fmaxf(x + mrow[i], -3.4028234663852886e38f);
         return x;
     };
-    if (a.width <= (int64_t)256 * 8 * kRowVecs) {
-        // thread t holds entries 8*(256*v + t) .. +7 of vector round v; a ragged end is read entry by entry
+    if (a.width <= (int64_t)kAttnThreads * 8 * kRowVecs) {
+        // thread t holds entries 8*(kAttnThreads*v + t) .. +7 of vector round v; a ragged end is read entry by entry
         float x[kRowVecs][8];
 #pragma unroll
         for (int v = 0; v < kRowVecs; v++) {
-            const int64_t i0 = ((int64_t)v * 256 + tid) * 8;
+            const int64_t i0 = ((int64_t)v * kAttnThreads + tid) * 8;
             if (i0 + 8 <= a.width) {
                 const H8 h = *reinterpret_cast<const H8 *>(row + i0);
 #pragma unroll
@@ -146,7 +152,7 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
         sum = block_reduce(sum, false, scratch);
 #pragma unroll
         for (int v = 0; v < kRowVecs; v++) {
-            const int64_t i0 = ((int64_t)v * 256 + tid) * 8;
+            const int64_t i0 = ((int64_t)v * kAttnThreads + tid) * 8;
             if (i0 + 8 <= a.width) {
                 H8 h;
 #pragma unroll
@@ -163,19 +169,19 @@ __global__ void __launch_bounds__(256) attn_tail_softmax(AttnArgs a)
     }
     // longer rows: three passes over the row (it stays in L2)
     float mx = -INFINITY;
-    for (int64_t i = tid; i < a.width; i += 256) mx = fmaxf(mx, value(i, row[i]));
+    for (int64_t i = tid; i < a.width; i += kAttnThreads) mx = fmaxf(mx, value(i, row[i]));
     mx = block_reduce(mx, true, scratch);
     float sum = 0.f;
-    for (int64_t i = tid; i < a.width; i += 256) sum += expf(value(i, row[i]) - mx);
+    for (int64_t i = tid; i < a.width; i += kAttnThreads) sum += expf(value(i, row[i]) - mx);
     sum = block_reduce(sum, false, scratch);
-    for (int64_t i = tid; i < a.width; i += 256) row[i] = f32_to_h16(expf(value(i, row[i]) - mx) / sum);
+    for (int64_t i = tid; i < a.width; i += kAttnThreads) row[i] = f32_to_h16(expf(value(i, row[i]) - mx) / sum);
 }
 
-// grid = samples, block = 256: thread t owns head dimensions 8*(t%16).. of the tokens t/16, t/16+16, ...
+// grid = samples: thread t owns head dimensions 8*(t%16).. of the tokens t/16, t/16 + 64, ...
 // out = fp16( fp16(out from the quantized values) + fp16(sum_j p[v_tokens + j] * v_tail[j]) )
-__global__ void __launch_bounds__(256) attn_tail_output(AttnArgs a)
+__global__ void __launch_bounds__(kAttnThreads) attn_tail_output(AttnArgs a)
 {
-    __shared__ float part[16][129];
+    __shared__ float part[kAttnGroups][129];
     const int64_t sample = blockIdx.x;
     const int64_t kv = sample / a.heads_per_kv;
     const int tid = threadIdx.x;
@@ -188,18 +194,18 @@ __global__ void __launch_bounds__(256) attn_tail_output(AttnArgs a)
         const int d = d0 + sub * 8;
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (d < a.D) {
-            for (int64_t j0 = grp; j0 < v_len; j0 += 64) {
-                float p[4];
-                H8 vv[4];
+            for (int64_t j0 = grp; j0 < v_len; j0 += kAttnGroups * kTailUnroll) {
+                float p[kTailUnroll];
+                H8 vv[kTailUnroll];
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const int64_t j = j0 + 16 * t;
+                for (int t = 0; t < kTailUnroll; t++) {
+                    const int64_t j = j0 + kAttnGroups * t;
                     const bool in = j < v_len;
                     p[t] = in ? h16_to_f32(prow[j]) : 0.f;
                     vv[t] = *reinterpret_cast<const H8 *>(vt + (in ? j : j0) * a.vt_ts + d);
                 }
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
+                for (int t = 0; t < kTailUnroll; t++) {
 #pragma unroll
                     for (int i = 0; i < 8; i++) acc[i] = fmaf(p[t], h16_to_f32(vv[t].v[i]), acc[i]);
                 }
@@ -212,7 +218,7 @@ __global__ void __launch_bounds__(256) attn_tail_output(AttnArgs a)
         if (tid < 128 && d0 + tid < a.D) {
             float s = 0.f;
 #pragma unroll
-            for (int g = 0; g < 16; g++) s += part[g][tid];
+            for (int g = 0; g < kAttnGroups; g++) s += part[g][tid];
             const float tail = h16_to_f32(f32_to_h16(s));
             const float quant = a.v_tokens > 0 ? h16_to_f32(op[d0 + tid]) : 0.f;
             op[d0 + tid] = f32_to_h16(quant + tail);
@@ -295,7 +301,7 @@ extern "C" int kvmix_decode_attention(const kvmix_decode_attn_t *p, void *worksp
     a.inv_sqrt_d = 1.0f / sqrtf((float)p->D);
     hipStream_t st = (hipStream_t)stream;
     if (p->samples > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_tail_softmax, dim3((unsigned)p->samples), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_tail_softmax, dim3((unsigned)p->samples), dim3(kAttnThreads), 0, st, a);
     int rc = launch_status();
     if (rc != KVMIX_OK) return rc;
     if (p->v_tokens > 0) {
@@ -305,6 +311,6 @@ extern "C" int kvmix_decode_attention(const kvmix_decode_attn_t *p, void *worksp
                                   p->out_stride, p->out_stride, workspace, workspace_bytes, stream);
         if (rc != KVMIX_OK) return rc;
     }
-    hipLaunchKernelGGL(attn_tail_output, dim3((unsigned)p->samples), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_tail_output, dim3((unsigned)p->samples), dim3(kAttnThreads), 0, st, a);
     return launch_status();
 }
