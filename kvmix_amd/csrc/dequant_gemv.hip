@@ -62,6 +62,9 @@
 #ifndef KVMIX_MFMA1_MAX_WAVES
 #define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
 #endif
+#ifndef KVMIX_ROWS_SINGLE_BLOCK_CHUNKS
+#define KVMIX_ROWS_SINGLE_BLOCK_CHUNKS 2  // p.V: keep one block per output row up to this many chunks per wave
+#endif
 #ifndef KVMIX_TARGET_WAVES
 #define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
 #endif
@@ -1794,6 +1797,9 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
     int64_t waves = want < max_waves ? want : max_waves;
     if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
     int64_t splits = (want + waves - 1) / waves;
+    // a second block per output row brings the reduce_splits launch with it: not worth it while
+    // one block's waves get at most KVMIX_ROWS_SINGLE_BLOCK_CHUNKS chunks each
+    if (splits > 1 && chunks <= waves * KVMIX_ROWS_SINGLE_BLOCK_CHUNKS) splits = 1;
     if (splits > 64) splits = 64;
     int64_t rps = (K + splits - 1) / splits;
     rps = (rps + chunk - 1) / chunk * chunk;
