@@ -62,6 +62,9 @@
 #ifndef KVMIX_MFMA1_MAX_WAVES
 #define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
 #endif
+#ifndef KVMIX_MFMA2_KSPLIT_WAVES
+#define KVMIX_MFMA2_KSPLIT_WAVES 1536  // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
+#endif
 #ifndef KVMIX_ROWS_SINGLE_BLOCK_CHUNKS
 #define KVMIX_ROWS_SINGLE_BLOCK_CHUNKS 2  // p.V: keep one block per output row up to this many chunks per wave
 #endif
@@ -88,6 +91,7 @@ struct GemvArgs {
     int heads_per_kv;
     int group;
     int splits;
+    int ksplit;  // gemv_cols_mfma2: waves that share a tile and slice K
 };
 
 // MODE: 1, 2, 4 = reference layout with that many bits (group 32 in the fast kernels),
@@ -1493,9 +1497,20 @@ gemv_cols_mfma2(GemvArgs a)
     const int K = (int)a.K;
     const int ngroups = (int)(a.N / 32);
     const int tpw = a.splits;
-    const int tile0 = (int)bx * tpw * nw + wy;
-    if (tile0 * TG >= ngroups) return;  // (no block barrier below)
-    const int nch = (K + CH - 1) / CH;
+    // ks > 1 (small problems, tpw == 1): ks neighbouring waves share a tile and slice its K rows
+    // chunk-wise, which shortens each wave's chain of dependent loads; their sums meet in LDS
+    const int ks = a.ksplit;
+    const int slice = wy % ks;
+    const int ntw = nw / ks;            // tiles a block works on at a time
+    const int tile0 = (int)bx * tpw * ntw + wy / ks;
+    if (tile0 * TG >= ngroups) {
+        if (ks > 1) __syncthreads();    // (the one block barrier of finish_tile)
+        return;
+    }
+    const int nch_all = (K + CH - 1) / CH;
+    const int nch_slice = (nch_all + ks - 1) / ks;
+    const int ch0 = slice * nch_slice;  // this wave's chunks: [ch0, ch0 + nch)
+    const int nch = ch0 >= nch_all ? 0 : (ch0 + nch_slice <= nch_all ? nch_slice : nch_all - ch0);
     const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
@@ -1532,10 +1547,10 @@ gemv_cols_mfma2(GemvArgs a)
     uint32_t w[KB][4][WL];
 
     auto tile_g0 = [&](int it) {
-        const int g = (tile0 + (it / nch) * nw) * TG;
+        const int g = (tile0 + (nch > 0 ? it / nch : 0) * ntw) * TG;
         return g + TG <= ngroups ? g : ngroups - TG;
     };
-    auto chunk_k0 = [&](int it) { return (it % nch) * CH; };
+    auto chunk_k0 = [&](int it) { return (ch0 + (nch > 0 ? it % nch : 0)) * CH; };
     auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
     auto load_small = [&](int it) {
         const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
@@ -1623,27 +1638,63 @@ gemv_cols_mfma2(GemvArgs a)
         const int first = scatter_reduce<8, 4, 1>(z, lane);  // lane bits 2..4
         z[0] += __shfl_xor(z[0], 32);
         zl[8 * sub + first] = z[0];
-        wave_lds_fence();
-        const int q = lane / 4;
-        uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)tile_g0(it) * 32;
+        float sum[2][NPOS];
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-            const float zt = zl[2 * q + s];
-            // element of the quad's 8 that this lane's accumulators of set s belong to
-            const int elem = s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1)));
-            Out8 o;
 #pragma unroll
-            for (int p = 0; p < NPOS; p++) {
-                const float sum = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
-                o.v[p] = f32_to_h16(fmaf(sum, __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
+            for (int p = 0; p < NPOS; p++) sum[s][p] = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
+        }
+        wave_lds_fence();
+        if (ks > 1) {
+            // slices 1.. park their sums in their own (now idle) A tile; slice 0 adds them up
+            float *mine = reinterpret_cast<float *>(atile);
+            if (slice > 0) {
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+#pragma unroll
+                    for (int p = 0; p < NPOS; p++) mine[(s * NPOS + p) * kWave + lane] = sum[s][p];
+                }
             }
-            *reinterpret_cast<Out8 *>(orow + (8 * q + elem) * 8) = o;
+            __syncthreads();
+            if (slice == 0) {
+                for (int o = 1; o < ks; o++) {
+                    const uint16_t *other_tile = atile + o * (AT + TG * 2);
+                    const float *other = reinterpret_cast<const float *>(other_tile);
+                    const float *ozl = reinterpret_cast<const float *>(other_tile + AT);
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+#pragma unroll
+                        for (int p = 0; p < NPOS; p++) sum[s][p] += other[(s * NPOS + p) * kWave + lane];
+                    }
+                    if (lane < TG) zl[lane] += ozl[lane];
+                }
+                wave_lds_fence();
+            }
+        }
+        if (slice == 0) {
+            const int q = lane / 4;
+            uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)tile_g0(it) * 32;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                const float zt = zl[2 * q + s];
+                // element of the quad's 8 that this lane's accumulators of set s belong to
+                const int elem = s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1)));
+                Out8 o;
+#pragma unroll
+                for (int p = 0; p < NPOS; p++)
+                    o.v[p] = f32_to_h16(fmaf(sum[s][p], __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
+                *reinterpret_cast<Out8 *>(orow + (8 * q + elem) * 8) = o;
+            }
         }
         wave_lds_fence();
         clear();
     };
 
     wave_lds_fence();
+    if (nch == 0) {  // (a slice beyond the last chunk: only its zeros take part)
+        finish_tile(0);
+        return;
+    }
     load_small(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1977,6 +2028,18 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     const int64_t batch = samples * a.M;
     int64_t tpw = batch * tiles / kTargetWaves;  // tiles per wave: about one resident round of waves
     tpw = tpw < 1 ? 1 : (tpw > 8 ? 8 : tpw);
+    // few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
+    const int64_t chunks = (a.K + 15) / 16;
+    int ks = 1;
+    while (ks < kColsWaves && batch * tiles * ks * 2 <= KVMIX_MFMA2_KSPLIT_WAVES && chunks >= ks * 4) ks *= 2;
+    a.ksplit = ks;
+    if (ks > 1) {
+        a.splits = 1;
+        const dim3 grid((unsigned)tiles, (unsigned)samples, (unsigned)a.M);  // one tile per block of ks waves
+        const size_t lds = (size_t)ks * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
+        hipLaunchKernelGGL((gemv_cols_mfma2<BITS>), grid, dim3(kWave, ks), lds, st, a);
+        return;
+    }
     const int64_t slots = (tiles + tpw - 1) / tpw;
     const int wpb = pick_waves_per_block(slots);
     a.splits = (int)tpw;
@@ -2138,6 +2201,7 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
     a.heads_per_kv = heads_per_kv;
     a.group = group;
     a.splits = 1;
+    a.ksplit = 1;
     a.rows_per_split = K > 0 ? K : 1;
     hipStream_t st = (hipStream_t)stream;
 

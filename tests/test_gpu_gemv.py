@@ -70,6 +70,9 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
     run_case(oracle, dev, bits, g, B=1, nh=8, nkv=2, K=128, N=32 * 41, seed=41)      # GQA, 4 heads per block
     run_case(oracle, dev, bits, g, B=1, nh=6, nkv=2, K=128, N=32 * 20, seed=42)      # GQA, 3 heads per kv head
     run_case(oracle, dev, bits, g, B=4, nh=16, nkv=16, K=64, N=512 * 9, seed=43)     # many tiles
+    # few tiles: several waves share a tile and slice K (9 chunks of 16 rows over 4 waves leave one idle)
+    run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=144, N=2048 + 64, seed=46)
+    run_case(oracle, dev, bits, g, B=2, nh=4, nkv=4, K=128, N=32 * 75, seed=47)
     # p.V: chunks of 128 rows, K ragged; GQA with split-K; M = 2
     for K in (128, 129, 255, 1000):
         run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=K, N=128, seed=K)
