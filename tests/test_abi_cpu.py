@@ -77,6 +77,41 @@ def test_host_validation_needs_no_gpu(lib):
     assert lib.kvmix_gemv_workspace_bytes(0, 1, 4096, 128) == 0
 
 
+def test_decode_attention_host_validation_needs_no_gpu(lib):
+    """kvmix_decode_attention checks its descriptor on the host before the first launch."""
+    from kvmix_amd import _lib
+
+    def desc(**kw):
+        st = _lib.DecodeAttn()
+        st.q, st.q_stride, st.probs, st.out = 16, 128, 16, 16
+        st.k_tail, st.v_tail = 16, 16
+        st.k_tail_batch_stride = st.v_tail_batch_stride = 8 * 128
+        st.k_tail_token_stride = st.v_tail_token_stride = 128
+        st.k_tail_slots = st.v_tail_slots = st.k_tail_len = st.v_tail_len = 8
+        st.samples, st.heads, st.heads_per_kv, st.D = 4, 4, 1, 128
+        st.probs_stride, st.out_stride = 8, 128
+        st.k_bits = st.v_bits = 4
+        st.k_group = st.v_group = 32
+        for k, v in kw.items():
+            setattr(st, k, v)
+        return st
+
+    call = lambda st: lib.kvmix_decode_attention(ctypes.byref(st), None, 0, None)
+    assert lib.kvmix_decode_attention(None, None, 0, None) == -7
+    assert call(desc(heads_per_kv=3)) == -5          # 4 rows are not a multiple of 3 heads per kv head
+    assert call(desc(heads=3)) == -5
+    assert call(desc(D=100)) == -9                   # head dimension must be a multiple of 8
+    assert call(desc(k_tail_len=9)) == -8            # more live tokens than slots
+    assert call(desc(v_tail_len=5)) == -8            # keys and values must cover the same positions
+    assert call(desc(probs_stride=7)) == -8          # a probability row is 8 wide here
+    assert call(desc(q=None)) == -7
+    assert call(desc(k_tail=None)) == -7
+    assert call(desc(samples=0)) == 0                # nothing to do
+    assert lib.kvmix_decode_attention_workspace_bytes(ctypes.byref(desc())) == 0  # no quantized values: no scratch
+    big = desc(v_tokens=4096)
+    assert lib.kvmix_decode_attention_workspace_bytes(ctypes.byref(big)) == lib.kvmix_gemv_workspace_bytes(4, 1, 4096, 128)
+
+
 def test_python_ops_reject_bad_arguments_like_the_reference():
     import KVmix
 

@@ -187,3 +187,38 @@ def test_library_step_without_a_quantized_part_and_argument_errors(dev):
         ops.decode_attention(q, None, None, k, v, 32, 4, 32, 4, attention_mask=torch.zeros(B, 1, 1, L + 1, device=dev))
     with pytest.raises(RuntimeError):  # keys and values must cover the same positions
         ops.decode_attention(q, None, None, k, v[:, :, :5], 32, 4, 32, 4)
+
+
+def test_full_size_step_properties_b16_t8192(dev):
+    """The library step at the size the target is quoted on (B=16, 32 heads, 8064 quantized + 128 fp16
+    tokens, 4-bit keys, 2-bit values), through properties that need no CPU pass over 1.3 GB:
+    probabilities are non-negative and sum to one, the step equals its composition from the two
+    GEMVs and torch's matmul / softmax, and it is linear in V's zero points (adding a constant c
+    to every zero point of the quantized values adds c * sum of their probabilities)."""
+    from kvmix_amd import ops
+    from kvmix_amd.attention import KVmixAttention
+
+    torch.manual_seed(11)
+    B, H, D, Tq, L = 16, 32, 128, 8064, 128
+    kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq // 8), dtype=torch.int64, device=dev).to(torch.int32)
+    ks = (torch.rand(B, H, D, Tq // 32, device=dev) * 0.02).half()
+    km = (torch.randn(B, H, D, Tq // 32, device=dev) * 0.1).half()
+    vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D // 16), dtype=torch.int64, device=dev).to(torch.int32)
+    vs = (torch.rand(B, H, Tq, D // 32, device=dev) * 0.5).half()
+    vm = (torch.randn(B, H, Tq, D // 32, device=dev)).half()
+    k_tail = torch.randn(B, H, L, D, device=dev).half()
+    v_tail = torch.randn(B, H, L, D, device=dev).half()
+    q = torch.randn(B, H, 1, D, device=dev).half()
+    out, p = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, 32, 4, 32, 2)
+    assert p.shape == (B, H, 1, Tq + L) and float(p.min()) >= 0.0
+    assert float((p.float().sum(-1) - 1.0).abs().max()) < 3e-3   # 8192 fp16 roundings of up to 2^-11 relative each
+    att = KVmixAttention(4, 2, residual_length=L)
+    out_t, p_t = att._decode_with_torch_glue(q, kc, ks, km, k_tail, vc, vs, vm, v_tail, 32, 0, 0, 1, None)
+    torch.testing.assert_close(p, p_t, rtol=5e-3, atol=2e-6)
+    torch.testing.assert_close(out, out_t, rtol=5e-3, atol=5e-3)
+    c = 0.25
+    out_c, p_c = ops.decode_attention(q, (kc, ks, km), (vc, vs, (vm.float() + c).half()), k_tail, v_tail, 32, 4, 32, 2)
+    assert torch.equal(p_c, p)
+    shift = c * p[..., :Tq].float().sum(-1)   # [B,H,1]
+    # zero points were rounded to fp16 after the shift: allow their ulp (2^-10 of |zero| <= 4) on top of the output's
+    torch.testing.assert_close(out_c.float() - out.float(), shift.unsqueeze(-1).expand(B, H, 1, D), rtol=0, atol=1.2e-2)
