@@ -479,8 +479,9 @@ def main():
                     help="also run plain 1 GiB device copies (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (every (batch, kv-head) slice is independent; "
-              "see DESIGN.md for how the path would shard). Re-run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only. Every (batch, kv-head) slice is independent, so the path "
+              "shards over batch or kv heads without any exchange; no multi-GPU figure is produced. "
+              "Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
