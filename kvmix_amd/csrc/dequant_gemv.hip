@@ -567,8 +567,16 @@ gemv_cols3(GemvArgs a)
     }
     __syncthreads();
 
-    int t0 = (int)(bx * blockDim.y + wy) * TU;
-    if (t0 >= nunits) return;  // (after the only block barrier)
+    // ks > 1: ks neighbouring waves share a tile and each takes a share of the K rows (wide tiles --
+    // long contiguous pieces per row -- for launches that would otherwise have too few waves);
+    // their sums meet in LDS behind the x vector
+    const int ks = a.ksplit;
+    const int slice = wy % ks;
+    int t0 = (int)(bx * (blockDim.y / ks) + wy / ks) * TU;
+    if (t0 >= nunits) {
+        if (ks > 1) __syncthreads();  // (the barrier of the combine step)
+        return;
+    }
     t0 = t0 + TU <= nunits ? t0 : nunits - TU;
     const int unit0 = t0 + gl * UPL;
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
@@ -589,8 +597,8 @@ gemv_cols3(GemvArgs a)
     }
 
     // this lane's rows: [kbeg, kend), walked in steps of U
-    const int kq = (K + RQ - 1) / RQ;
-    const int kbeg = rq * kq;
+    const int kq = (K + RQ * ks - 1) / (RQ * ks);
+    const int kbeg = (slice * RQ + rq) * kq;
     const int kend = kbeg + kq < K ? kbeg + kq : K;
     const int steps = (kq + U - 1) / U;  // the same for every section: uniform control flow
 
@@ -657,6 +665,22 @@ gemv_cols3(GemvArgs a)
 
     // ---- combine the RQ row sections, store fp16 (2^59 undoes the fp32-subnormal scaling) ----
     constexpr int TOT = UPL * VALS;  // consecutive outputs of this lane
+    float *part = xs + NREP * (K + 1);  // [waves][NREP][TOT][64] when ks > 1
+    if (ks > 1) {
+        if (slice > 0) {
+#pragma unroll
+            for (int h = 0; h < NREP; h++) {
+#pragma unroll
+                for (int j = 0; j < UPL; j++) {
+#pragma unroll
+                    for (int i = 0; i < VALS; i++)
+                        part[((wy * NREP + h) * TOT + j * VALS + i) * kWave + lane] = fmaf(acc[j][h][i], kHeadsOutScale, zsum[h][j]);
+                }
+            }
+        }
+        __syncthreads();
+        if (slice > 0) return;
+    }
 #pragma unroll
     for (int h = 0; h < NREP; h++) {
         float flat[TOT];
@@ -664,6 +688,10 @@ gemv_cols3(GemvArgs a)
         for (int j = 0; j < UPL; j++) {
 #pragma unroll
             for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], kHeadsOutScale, zsum[h][j]);
+        }
+        for (int o = 1; o < ks; o++) {
+#pragma unroll
+            for (int e = 0; e < TOT; e++) flat[e] += part[(((wy + o) * NREP + h) * TOT + e) * kWave + lane];
         }
         uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + (sample0 + h) * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
         if constexpr (RQ == 1) {
@@ -1974,6 +2002,9 @@ static int64_t cols_min_units()
     return MODE == 3 ? 64 : 16 * ColsUpl<MODE>::value;
 }
 
+#ifndef KVMIX_COLS3_KSPLIT
+#define KVMIX_COLS3_KSPLIT 1  // gemv_cols3: wide tiles shared by two K-slicing waves when there are half as many tiles as waves wanted
+#endif
 #ifndef KVMIX_COLS3_WIDE_WAVES
 #define KVMIX_COLS3_WIDE_WAVES 4096
 #endif
@@ -1985,14 +2016,22 @@ static int64_t cols_min_units()
 #endif
 
 template <int RQ, int UPL, int NREP>
-static void launch_cols3_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
+static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int ks = 1)
 {
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / 11;
     const int64_t tiles = (units + TU - 1) / TU;
+    constexpr int U = NREP > 1 ? KVMIX_COLS3_HEADS_U : KVMIX_COLS3_U;  // rows in flight per lane
+    a.ksplit = ks;
+    if (ks > 1) {
+        // one tile per block: its ks waves slice K and leave their sums behind the x vector in LDS
+        const dim3 grid((unsigned)tiles, (unsigned)(samples / NREP), (unsigned)a.M);
+        const size_t lds = sizeof(float) * ((size_t)NREP * (size_t)(a.K + 1) + (size_t)ks * NREP * UPL * 11 * kWave);
+        hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, ks), lds, st, a);
+        return;
+    }
     const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
-    constexpr int U = NREP > 1 ? KVMIX_COLS3_HEADS_U : KVMIX_COLS3_U;  // rows in flight per lane
     hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, wpb),
                        sizeof(float) * (size_t)NREP * (size_t)(a.K + 1), st, a);
 }
@@ -2087,6 +2126,11 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
         else if (units >= 256 && waves(256) >= KVMIX_COLS3_WIDE_WAVES)
             launch_cols3_cfg<1, 4, 1>(a, samples, st);
+        else if (KVMIX_COLS3_KSPLIT && units >= 256 && a.K >= 64 && a.K <= 4096 && waves(256) * 2 >= KVMIX_COLS3_WIDE_WAVES)
+            // half as many wide tiles as that: the widest tile all the same (1 KiB of codes per row and
+            // wave), two waves per tile slicing K (measured: +6 % at B = 32, T = 8k; no gain from four
+            // waves per tile at smaller batches, which keep the narrower tiles below)
+            launch_cols3_cfg<1, 4, 1>(a, samples, st, 2);
         else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
             launch_cols3_cfg<2, 4, 1>(a, samples, st);
         else

@@ -89,6 +89,7 @@ def test_reference_3bit_kernel_edges(oracle, dev):
     run_case(oracle, dev, 3, 11, B=1, nh=8, nkv=2, K=50, N=11 * 64, seed=54)     # smallest fast tile, GQA
     run_case(oracle, dev, 3, 11, B=1, nh=2, nkv=2, K=128, N=11 * 131, seed=55, M=2)
     run_case(oracle, dev, 3, 11, B=8, nh=8, nkv=8, K=128, N=11 * 733, seed=56)   # wide tiles (4 words per lane)
+    run_case(oracle, dev, 3, 11, B=32, nh=32, nkv=32, K=64, N=11 * 300, seed=57)  # wide tiles, two waves per tile slicing K
 
 
 @pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
