@@ -222,3 +222,31 @@ def test_full_size_step_properties_b16_t8192(dev):
     shift = c * p[..., :Tq].float().sum(-1)   # [B,H,1]
     # zero points were rounded to fp16 after the shift: allow their ulp (2^-10 of |zero| <= 4) on top of the output's
     torch.testing.assert_close(out_c.float() - out.float(), shift.unsqueeze(-1).expand(B, H, 1, D), rtol=0, atol=1.2e-2)
+
+
+def test_library_step_with_a_row_longer_than_the_register_path(dev):
+    """More than 16384 positions: the softmax walks the row in three passes instead of holding it in
+    registers.  Against the composition from the GEMVs and torch, GQA, with a padding mask."""
+    from kvmix_amd import ops
+    from kvmix_amd.attention import KVmixAttention
+
+    torch.manual_seed(12)
+    B, H, Hkv, D, Tq, L = 2, 4, 2, 128, 20000 - 32, 37
+    kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, D, Tq // 16), dtype=torch.int64, device=dev).to(torch.int32)
+    ks = (torch.rand(B, Hkv, D, Tq // 32, device=dev) * 0.05).half()
+    km = (torch.randn(B, Hkv, D, Tq // 32, device=dev) * 0.1).half()
+    vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, Hkv, Tq, D // 8), dtype=torch.int64, device=dev).to(torch.int32)
+    vs = (torch.rand(B, Hkv, Tq, D // 32, device=dev) * 0.1).half()
+    vm = torch.randn(B, Hkv, Tq, D // 32, device=dev).half()
+    k_tail = torch.randn(B, Hkv, L, D, device=dev).half()
+    v_tail = torch.randn(B, Hkv, L, D, device=dev).half()
+    q = torch.randn(B, H, 1, D, device=dev).half()
+    mask = torch.zeros(B, 1, 1, Tq + L, device=dev)
+    mask[0, :, :, :5000] = torch.finfo(torch.float32).min
+    att = KVmixAttention(2, 4, residual_length=64)
+    for m in (None, mask):
+        out, p = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, 32, 2, 32, 4, attention_mask=m)
+        out_t, p_t = att._decode_with_torch_glue(q, kc, ks, km, k_tail, vc, vs, vm, v_tail, 32, 0, 0, H // Hkv, m)
+        torch.testing.assert_close(p, p_t, rtol=5e-3, atol=2e-6)
+        torch.testing.assert_close(out, out_t, rtol=5e-3, atol=5e-3)
+    assert float(p[0, :, :, :5000].abs().max()) == 0.0
