@@ -1049,9 +1049,6 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
 #pragma unroll
         for (int g = 0; g < LPR; g++) zacc[h][g] = 0.f;
     }
-    // some A rows are never written: clear the tiles once
-    for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
-
     // staging: this lane owns elements [8*lane, 8*lane+8) of the chunk's [128][4] scale array,
     // i.e. rows 2*lane and 2*lane+1, all four groups.  Row r of a chunk is k-slot (r%16)/4 of
     // A-lanes  (r%4)*16 + 4*g + i  in k-block r/16.
@@ -1173,7 +1170,6 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         }
     };
 
-    wave_lds_fence();
     if (kfirst < ke32) {
         // (the first loads are issued in the loop's own order, each pinned in place: the wait
         // counts at the loop head must hold for the entry path too)
@@ -1187,6 +1183,11 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        // some A rows are never written: clear the tiles once -- behind the first loads, whose
+        // latency covers it (every wave of a launch starts at the same time)
+        for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+        wave_lds_fence();
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
         for (int k0 = kfirst; k0 < ke32; k0 += DEPTH * stride) {
 #pragma unroll
@@ -1344,7 +1345,6 @@ __global__ void __launch_bounds__(64 * kColsWaves)
         }
     };
     clear();
-    for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
 
     // cell of (k-step t, operand lane l): four bf16 k-slots
     auto cell = [](int t, int l) { return ((2 * t + l / 32) * 33 + l % 32) * 4; };
@@ -1453,7 +1453,6 @@ __global__ void __launch_bounds__(64 * kColsWaves)
         clear();
     };
 
-    wave_lds_fence();
     load_small(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1461,6 +1460,11 @@ __global__ void __launch_bounds__(64 * kColsWaves)
         load_codes(0, t);
         __builtin_amdgcn_sched_barrier(0);
     }
+    // some A rows are never written: clear the tile once -- behind the first loads, whose latency
+    // covers it (every wave of a launch starts at the same time)
+    for (int i = lane; i < NM * AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+    wave_lds_fence();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
     for (int it = 0; it < items; it++) {
         const int nx = it + 1 < items ? it + 1 : it;  // (past the end: the same item again)
@@ -1562,7 +1566,6 @@ gemv_cols_mfma2(GemvArgs a)
         for (int j = 0; j < 8; j++) zacc[j] = 0.f;
     };
     clear();
-    for (int i = lane; i < AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
 
     // cell (four bf16 k-slots) of (k-step t, set s, operand lane l)
     auto cell = [](int t, int s, int l) { return (2 * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
@@ -1718,7 +1721,6 @@ gemv_cols_mfma2(GemvArgs a)
         clear();
     };
 
-    wave_lds_fence();
     if (nch == 0) {  // (a slice beyond the last chunk: only its zeros take part)
         finish_tile(0);
         return;
@@ -1730,6 +1732,11 @@ gemv_cols_mfma2(GemvArgs a)
         load_codes(0, t);
         __builtin_amdgcn_sched_barrier(0);
     }
+    // some A rows are never written: clear the tile once -- behind the first loads, whose latency
+    // covers it (every wave of a launch starts at the same time)
+    for (int i = lane; i < AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+    wave_lds_fence();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
     for (int it = 0; it < items; it++) {
         const int nx = it + 1 < items ? it + 1 : it;  // (past the end: the same item again)
