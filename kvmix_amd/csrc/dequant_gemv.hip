@@ -65,6 +65,9 @@
 #ifndef KVMIX_MFMA2_KSPLIT_WAVES
 #define KVMIX_MFMA2_KSPLIT_WAVES 1536  // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
 #endif
+#ifndef KVMIX_ROWS_CHUNKS_PER_WAVE
+#define KVMIX_ROWS_CHUNKS_PER_WAVE 8  // p.V: chunks a wave should get before more waves per row are used
+#endif
 #ifndef KVMIX_ROWS_SINGLE_BLOCK_CHUNKS
 #define KVMIX_ROWS_SINGLE_BLOCK_CHUNKS 2  // p.V: keep one block per output row up to this many chunks per wave
 #endif
@@ -1879,6 +1882,15 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
     const int64_t chunks = (K + chunk - 1) / chunk;  // units of parallelism along K
     int64_t want = (target + batch_rows - 1) / batch_rows;  // waves wanted per output row
     if (want > chunks) want = chunks;
+    // a wave's start-up and the reduction at its end are paid per wave: with fewer than about eight
+    // chunks per wave, fewer and longer-lived waves are faster (measured at B = 8, T = 8k: 16 -> 8
+    // waves per row, 2-bit p.V 22.2 -> 20.3 us), as long as two waves per SIMD remain
+    {
+        const int64_t by_chunks = (chunks + KVMIX_ROWS_CHUNKS_PER_WAVE - 1) / KVMIX_ROWS_CHUNKS_PER_WAVE;
+        const int64_t by_waves = (target / 2 + batch_rows - 1) / batch_rows;
+        const int64_t lean = by_chunks > by_waves ? by_chunks : by_waves;
+        if (lean < want) want = lean;
+    }
     if (want < 1) want = 1;
     int64_t waves = want < max_waves ? want : max_waves;
     if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
