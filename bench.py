@@ -267,16 +267,16 @@ def target_shape_extra(torch, _lib, lib, dev, stream):
 
         nbytes = B * H * Tq * bytes_per_token(bits, "")
         for name, fn in (("qk", qk), ("pv", pv)):
-            for i in range(6):
+            for i in range(30):  # warm-up: 30 launches, then 100 timed ones
                 assert fn(i) == 0
             torch.cuda.synchronize()
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             s.record()
-            for i in range(30):
+            for i in range(100):
                 fn(i)
             e.record()
             torch.cuda.synchronize()
-            us = s.elapsed_time(e) * 1e3 / 30
+            us = s.elapsed_time(e) * 1e3 / 100
             res[f"{name}_{bits}bit"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                                         "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
         del sets
@@ -320,16 +320,16 @@ def gqa_shape_extra(torch, _lib, lib, dev, stream):
     res = {}
     for name, fn, nbytes in (("qk_ref3", qk, B * Hkv * Tk * bytes_per_token(3, "ref3")),
                              ("pv_2bit", pv, B * Hkv * Tv * bytes_per_token(2, ""))):
-        for i in range(4):
+        for i in range(20):  # warm-up: 20 launches, then 100 timed ones
             assert fn(i) == 0
         torch.cuda.synchronize()
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         s.record()
-        for i in range(20):
+        for i in range(100):
             fn(i)
         e.record()
         torch.cuda.synchronize()
-        us = s.elapsed_time(e) * 1e3 / 20
+        us = s.elapsed_time(e) * 1e3 / 100
         res[name] = {"us": round(us, 2), "packed_MB": round(nbytes / 1e6, 1), "GBps": round(nbytes / us / 1e3, 1),
                      "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
     return res
