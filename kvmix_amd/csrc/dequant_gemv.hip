@@ -541,6 +541,14 @@ __device__ __forceinline__ int scatter_reduce(float *v, int lane)
 //   rows).  Tiles as in gemv_cols: TU = (64/RQ)*4 words per wave, last tile shifted left.
 //   block = (64, 2..4); grid = (tiles/waves, samples, M), XCD-swizzled; dynamic LDS = (K+1)*4.
 // ---------------------------------------------------------------------------------------
+// 2^(59 - offset of code i inside its word or inside word >> 24): undoes the fp32-pattern scaling
+__device__ __forceinline__ constexpr float cols3_out_scale(int i)
+{
+    float v = 576460752303423488.0f;  // 2^59
+    for (int k = 0; k < 3 * (i < 8 ? i : i - 8); k++) v *= 0.5f;
+    return v;
+}
+
 template <int RQ, int UPL, int U, int NREP>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_COLS3_HEADS_OCC : 3)))
 gemv_cols3(GemvArgs a)
@@ -616,36 +624,42 @@ gemv_cols3(GemvArgs a)
         sw[u] = *reinterpret_cast<const HalfN *>(sp + kc * s_rs);
         zw[u] = *reinterpret_cast<const HalfN *>(zp + kc * s_rs);
     };
+    // x of the U rows of a step is read from LDS in one go at the head of the step: read row by row,
+    // each read's latency sits in front of that row's arithmetic
+    float xr[U][NREP];
+    auto load_x = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int kx = k0 + u < kend ? k0 + u : K;
+#pragma unroll
+            for (int h = 0; h < NREP; h++) xr[u][h] = xs[h * (K + 1) + kx];
+        }
+    };
     auto compute_row = [&](int u, int k) {
-        const int kx = k < kend ? k : K;
         float xv[NREP];
 #pragma unroll
-        for (int h = 0; h < NREP; h++) xv[h] = xs[h * (K + 1) + kx];
+        for (int h = 0; h < NREP; h++) xv[h] = xr[u][h];
 #pragma unroll
         for (int j = 0; j < UPL; j++) {
             const half2_t sz = __builtin_bit_cast(half2_t, (uint32_t)sw[u].v[j] | ((uint32_t)zw[u].v[j] << 16));
-            if constexpr (NREP == 1) {
-                zsum[0][j] = fmaf(xv[0], (float)sz.y, zsum[0][j]);
-                float mq[4];
-                mq[0] = (xv[0] * 1237940039285380274899124224.0f) * (float)sz.x;  // 2^90, see accumulate_unit
+            // A masked field of the word, read as an fp32 pattern below 2^24, is code * 2^(offset-149)
+            // (subnormals and the first binade share one ulp): codes 0..7 come straight out of the
+            // word (offsets 0..21), codes 8..10 out of word >> 24.  One multiplier x*scale*2^90 per
+            // head serves every position; the factor 2^offset stays in the sum and is taken out once,
+            // at the end (cols3_out_scale) -- a power of two, so nothing is rounded differently.
+            const uint32_t w = cw[u].v[j], hi = w >> 24;
+            float f[VALS];
 #pragma unroll
-                for (int t = 1; t < 4; t++) mq[t] = mq[t - 1] * 0.125f;
-                const uint32_t w = cw[u].v[j];
-                const uint32_t v[3] = {w, w >> 12, w >> 24};
+            for (int i = 0; i < 8; i++) f[i] = __uint_as_float(w & (7u << (3 * i)));
+            f[8] = __uint_as_float(hi & 0x07u);
+            f[9] = __uint_as_float(hi & 0x38u);
+            f[10] = __uint_as_float(hi & 0xC0u);
 #pragma unroll
-                for (int i = 0; i < VALS; i++) {
-                    const uint32_t mask = (i == 10 ? 3u : 7u) << (3 * (i % 4));
-                    acc[j][0][i] = fmaf(mq[i % 4], __uint_as_float(v[i / 4] & mask), acc[j][0][i]);
-                }
-            } else {
-                // the field masks are shared by the heads: one v_and_b32 + NREP v_fmac_f32 per code
-                float qs[NREP];
+            for (int h = 0; h < NREP; h++) {
+                zsum[h][j] = fmaf(xv[h], (float)sz.y, zsum[h][j]);
+                const float mq = (xv[h] * 1237940039285380274899124224.0f) * (float)sz.x;  // 2^90
 #pragma unroll
-                for (int h = 0; h < NREP; h++) {
-                    zsum[h][j] = fmaf(xv[h], (float)sz.y, zsum[h][j]);
-                    qs[h] = xv[h] * (float)sz.x;
-                }
-                accumulate_heads<3, NREP>(&cw[u].v[j], qs, acc[j]);
+                for (int i = 0; i < VALS; i++) acc[j][h][i] = fmaf(mq, f[i], acc[j][h][i]);
             }
         }
     };
@@ -658,6 +672,8 @@ gemv_cols3(GemvArgs a)
 #pragma unroll 1
     for (int st = 0; st < steps; st++) {
         const int k0 = kbeg + st * U;
+        load_x(k0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; u++) {
             compute_row(u, k0 + u);
@@ -677,7 +693,7 @@ gemv_cols3(GemvArgs a)
                 for (int j = 0; j < UPL; j++) {
 #pragma unroll
                     for (int i = 0; i < VALS; i++)
-                        part[((wy * NREP + h) * TOT + j * VALS + i) * kWave + lane] = fmaf(acc[j][h][i], kHeadsOutScale, zsum[h][j]);
+                        part[((wy * NREP + h) * TOT + j * VALS + i) * kWave + lane] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j]);
                 }
             }
         }
@@ -690,7 +706,7 @@ gemv_cols3(GemvArgs a)
 #pragma unroll
         for (int j = 0; j < UPL; j++) {
 #pragma unroll
-            for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], kHeadsOutScale, zsum[h][j]);
+            for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j]);
         }
         for (int o = 1; o < ks; o++) {
 #pragma unroll
