@@ -62,6 +62,9 @@
 #ifndef KVMIX_MFMA1_MAX_WAVES
 #define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
 #endif
+#ifndef KVMIX_MFMA2_MAX_TPW
+#define KVMIX_MFMA2_MAX_TPW 1  // gemv_cols_mfma2: tiles a wave walks at most (measured: one tile per wave and more waves beats several tiles per wave at every size tried)
+#endif
 #ifndef KVMIX_MFMA2_KSPLIT_WAVES
 #define KVMIX_MFMA2_KSPLIT_WAVES 1536  // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
 #endif
@@ -2101,7 +2104,7 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     const int64_t tiles = (a.N / 32 + 31) / 32;
     const int64_t batch = samples * a.M;
     int64_t tpw = batch * tiles / kTargetWaves;  // tiles per wave: about one resident round of waves
-    tpw = tpw < 1 ? 1 : (tpw > 8 ? 8 : tpw);
+    tpw = tpw < 1 ? 1 : (tpw > KVMIX_MFMA2_MAX_TPW ? KVMIX_MFMA2_MAX_TPW : tpw);
     // few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
     const int64_t chunks = (a.K + 15) / 16;
     int ks = 1;
@@ -2129,8 +2132,10 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // two-element matrix-core kernel: measured faster than gemv_cols and gemv_cols_mfma up to
         // one resident round of waves (B = 16 at T = 8k); beyond that gemv_cols streams better
         const int64_t tiles2 = (a.N / 32 + 31) / 32;
+        // ... and at any batch while a row holds no more than two of gemv_cols' 2048-code tiles (T = 4k,
+        // B = 64: 2-bit 111 -> 88 us, 4-bit 133 -> 127 us; at T = 5k gemv_cols is ahead again)
         if (KVMIX_COLS_MFMA2 && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
-            samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES) {
+            (samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES || a.N <= 2 * 2048)) {
             launch_cols_mfma2<MODE>(a, samples, st);
             return;
         }
