@@ -205,7 +205,11 @@ def test_graph_replayed_steps_match_eager_steps(dev):
     atts, caches = kvmix_layers(cfg, kbits, vbits, residual_length=window, capacity=T + new)
     gd = GraphDecoder(cfg, weights, atts, caches)
     seen = []
-    tokens = gd.generate(prompt, new, lambda step, lg: seen.append(lg.clone()))
+    def keep(step, lg):
+        seen.append(lg.clone())
+        torch.cuda.synchronize()  # (a synchronisation and eager work between every two replays)
+
+    tokens = gd.generate(prompt, new, keep)
     assert gd.graph_steps + gd.eager_steps == new and gd.graph_steps > 0.85 * new and gd.captures >= 4
 
     atts2, caches2 = kvmix_layers(cfg, kbits, vbits, residual_length=window, capacity=T + new)
