@@ -62,6 +62,9 @@
 #ifndef KVMIX_MFMA1_MAX_WAVES
 #define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
 #endif
+#ifndef KVMIX_COLS_MFMA2_1BIT
+#define KVMIX_COLS_MFMA2_1BIT 1  // 1-bit q.K^T through the two-element kernel too
+#endif
 #ifndef KVMIX_MFMA2_MAX_TPW
 #define KVMIX_MFMA2_MAX_TPW 1  // gemv_cols_mfma2: tiles a wave walks at most (measured: one tile per wave and more waves beats several tiles per wave at every size tried)
 #endif
@@ -1529,14 +1532,14 @@ template <int BITS>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(KVMIX_MFMA2_OCC4)))
 gemv_cols_mfma2(GemvArgs a)
 {
-    static_assert(BITS == 4 || BITS == 2, "two elements per lane: a dwordx2 or a dword");
+    static_assert(BITS == 4 || BITS == 2 || BITS == 1, "two elements per lane: a dwordx2, a dword or a ushort");
     constexpr int CH = 16;             // rows per chunk
     constexpr int KB = CH / 4;         // MFMA k-steps per chunk
     constexpr int AT = kColsMfma2Tile;
     constexpr int NPOS = 8;
     constexpr int FPB = 8 / BITS;
     constexpr int TG = 32;             // groups per tile
-    constexpr int WL = BITS / 2;       // dwords per lane and row (2 or 1)
+    constexpr int WL = BITS == 4 ? 2 : 1;  // registers per lane and row (1 bit: a ushort in one register)
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
@@ -1568,7 +1571,8 @@ gemv_cols_mfma2(GemvArgs a)
     const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
-    const uint32_t *cbase = a.code + kv * a.c_bs + lane * WL;
+    // (byte pointer: a lane's two elements are 2 * BITS bytes)
+    const uint8_t *cbase = reinterpret_cast<const uint8_t *>(a.code + kv * a.c_bs) + lane * (2 * BITS);
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
     const int sub = lane % 4;   // staging: row lane/4 of the chunk, groups 8*sub .. 8*sub+7
     const int srow = lane / 4;
@@ -1614,12 +1618,16 @@ gemv_cols_mfma2(GemvArgs a)
     };
     auto load_codes = [&](int it, int t) {
         // (a group of 32 codes is BITS words)
-        const uint32_t *base = cbase + ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
+        const uint8_t *base = cbase + 4u * ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const Words<WL> v = *reinterpret_cast<const Words<WL> *>(base + (uint32_t)k * c_rs);
+            if constexpr (BITS == 1) {
+                w[t][k][0] = *reinterpret_cast<const uint16_t *>(base + 4u * (uint32_t)k * c_rs);
+            } else {
+                const Words<WL> v = *reinterpret_cast<const Words<WL> *>(base + 4u * (uint32_t)k * c_rs);
 #pragma unroll
-            for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
+                for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
+            }
         }
     };
     auto stage = [&](int it) {
@@ -1651,7 +1659,7 @@ gemv_cols_mfma2(GemvArgs a)
             // set 0: lanes 0,1 of a quad hold the group's elements 0,2 (their first) and lanes 2,3
             // take elements 1,3 (the second of lanes 0,1); set 1 mirrors it for lanes 2,3
             uint32_t src[4];
-            uint32_t hi = 0;  // 2 bits: byte offset (0 or 2) of the element inside the word
+            uint32_t hi = 0;  // 2 bits / 1 bit: byte offset (0 or 2 / 0 or 1) of the element inside the register
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 if constexpr (BITS == 4) {
@@ -1664,7 +1672,7 @@ gemv_cols_mfma2(GemvArgs a)
                                     : __builtin_amdgcn_mov_dpp(w[t][k][0], 0xEE, 0xf, 0xf, false);
                 }
             }
-            if constexpr (BITS == 2) hi = (s == 0 ? j4 >= 2 : j4 < 2) ? 2u : 0u;
+            if constexpr (BITS != 4) hi = (s == 0 ? j4 >= 2 : j4 < 2) ? (uint32_t)BITS : 0u;  // byte offset of the element
 #pragma unroll
             for (int b = 0; b < BITS; b++) {
                 const uint32_t sel = (0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16)) + hi * 0x00010001u;
@@ -2128,14 +2136,20 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
-    if constexpr (MODE == 2 || MODE == 4) {
+    if constexpr (MODE == 1 || MODE == 2 || MODE == 4) {
         // two-element matrix-core kernel: measured faster than gemv_cols and gemv_cols_mfma up to
         // one resident round of waves (B = 16 at T = 8k); beyond that gemv_cols streams better
         const int64_t tiles2 = (a.N / 32 + 31) / 32;
         // ... and at any batch while a row holds no more than two of gemv_cols' 2048-code tiles (T = 4k,
         // B = 64: 2-bit 111 -> 88 us, 4-bit 133 -> 127 us; at T = 5k gemv_cols is ahead again)
-        if (KVMIX_COLS_MFMA2 && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
-            (samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES || a.N <= 2 * 2048)) {
+        // 1 bit: only beyond the range of the one-element kernel (which, with its several tiles per
+        // wave, is ahead up to one resident round of waves: B = 16, T = 4k: 19.6 against 22.7 us);
+        // there, and for rows of up to two of gemv_cols' tiles, it replaces gemv_cols (B = 64, T = 4k:
+        // 110 -> 87 us; at T = 8k gemv_cols stays ahead)
+        const bool one_bit_ok = MODE != 1 || (KVMIX_COLS_MFMA2_1BIT && a.N <= 2 * 2048 &&
+                                              samples * a.M * ((a.N / 32 + 31) / 32) >= (int64_t)KVMIX_MFMA1_MAX_WAVES);
+        if (KVMIX_COLS_MFMA2 && one_bit_ok && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
+            (MODE == 1 || samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES || a.N <= 2 * 2048)) {
             launch_cols_mfma2<MODE>(a, samples, st);
             return;
         }

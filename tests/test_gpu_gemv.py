@@ -73,6 +73,9 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
     # few tiles: several waves share a tile and slice K (9 chunks of 16 rows over 4 waves leave one idle)
     run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=144, N=2048 + 64, seed=46)
     run_case(oracle, dev, bits, g, B=2, nh=4, nkv=4, K=128, N=32 * 75, seed=47)
+    # a launch beyond one resident round of waves with short rows (the two-element kernel for every width)
+    run_case(oracle, dev, bits, g, B=32, nh=32, nkv=32, K=32, N=32 * 127, seed=48)
+    run_case(oracle, dev, bits, g, B=40, nh=32, nkv=32, K=48, N=32 * 127, seed=49)
     # p.V: chunks of 128 rows, K ragged; GQA with split-K; M = 2
     for K in (128, 129, 255, 1000):
         run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=K, N=128, seed=K)
