@@ -203,34 +203,35 @@ int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride, int64
  * workspace: at least kvmix_decode_attention_workspace_bytes() bytes of device scratch.
  */
 typedef struct kvmix_decode_attn {
-    const void *q;
-    int64_t q_stride;
-    const uint32_t *k_code;
+    const void *q;              /* [samples, D] fp16 */
+    int64_t q_stride;           /* elements between two rows of q */
+    const uint32_t *k_code;     /* [samples / heads_per_kv, D, k_tokens / vpw] */
     int64_t k_code_batch_stride, k_code_row_stride;
-    const void *k_scale, *k_zero;
+    const void *k_scale, *k_zero; /* [samples / heads_per_kv, D, k_tokens / k_group] fp16 */
     int64_t k_sz_batch_stride, k_sz_row_stride;
     int k_bits, k_fmt, k_group;
-    int64_t k_tokens;
-    const uint32_t *v_code;
+    int64_t k_tokens;           /* quantized key tokens (0: none, the k_ pointers are not read) */
+    const uint32_t *v_code;     /* [samples / heads_per_kv, v_tokens, D / vpw] */
     int64_t v_code_batch_stride, v_code_row_stride;
-    const void *v_scale, *v_zero;
+    const void *v_scale, *v_zero; /* [samples / heads_per_kv, v_tokens, D / v_group] fp16 */
     int64_t v_sz_batch_stride, v_sz_row_stride;
     int v_bits, v_fmt, v_group;
-    int64_t v_tokens;
-    const void *k_tail;
+    int64_t v_tokens;           /* quantized value tokens */
+    const void *k_tail;         /* [samples / heads_per_kv, k_tail_slots, D] fp16 */
     int64_t k_tail_batch_stride, k_tail_token_stride, k_tail_slots, k_tail_len;
-    const int64_t *k_tail_len_dev;
-    const void *v_tail;
+    const int64_t *k_tail_len_dev; /* NULL, or where the live length is read when the kernels run */
+    const void *v_tail;         /* [samples / heads_per_kv, v_tail_slots, D] fp16 */
     int64_t v_tail_batch_stride, v_tail_token_stride, v_tail_slots, v_tail_len;
     const int64_t *v_tail_len_dev;
-    const float *mask;
+    const float *mask;          /* NULL, or [samples / heads, width] fp32 */
     int64_t mask_stride;
-    int64_t samples;
-    int heads, heads_per_kv;
-    int64_t D;
-    void *probs;
+    int64_t samples;            /* batch * query heads */
+    int heads;                  /* query heads per batch element (the mask is per batch element) */
+    int heads_per_kv;           /* query heads that share one kv head */
+    int64_t D;                  /* head dimension, a multiple of 8 */
+    void *probs;                /* [samples, width] fp16, out */
     int64_t probs_stride;
-    void *out;
+    void *out;                  /* [samples, D] fp16, out */
     int64_t out_stride;
 } kvmix_decode_attn_t;
 
