@@ -13,13 +13,20 @@
 //
 // Kernels (each documented where it is defined)
 //   gemv_rows_mfma  p.V (K = tokens large, N = 128), 1/2/4-bit and dense 3-bit: matrix cores.
-//   gemv_cols_mfma  q.K^T (K = head_dim small, N = tokens large), 1/2/4-bit: matrix cores; used
-//                   for GQA and for problems too small for gemv_cols' wide tiles.
+//   gemv_cols_mfma2 q.K^T (K = head_dim small, N = tokens large), 1/2/4-bit, one query head per kv
+//                   head: matrix cores, two 8-code elements per lane; small launches let several
+//                   waves share a tile and slice K.
+//   gemv_cols_mfma  q.K^T, 1/2/4-bit: matrix cores, one element per lane; GQA (four query heads per
+//                   pass) and 1-bit.
 //   gemv_cols3      q.K^T, the reference's 3-bit format: register streaming, vector ALU.
-//   gemv_cols       q.K^T, 1/2/4-bit and dense 3-bit: vector ALU, (scale, zero) staged in LDS.
+//   gemv_cols       q.K^T, 1/2/4-bit at large batch with long rows, dense 3-bit: vector ALU,
+//                   (scale, zero) staged in LDS.
 //   gemv_rows       p.V for N = 64 / 256 or strided code rows: vector ALU.
-//   gemv_generic    any shape/group: one thread per packed word, serial over K.
+//   gemv_generic    any shape/group, and rows shorter than one tile of the kernels above: one thread
+//                   per packed word, the block's spare threads slice K.
 //   reduce_splits   sums the split-K partials of the p.V kernels and stores fp16.
+// Which kernel a call gets is decided in launch_cols / launch_rows / kvmix_quantized_gemv at the
+// end of the file; the thresholds there are measured ones.
 //
 // Common rules of the streaming kernels (measured on MI355X): scale/zero never by 2-byte loads
 // per lane (they cost a third of the run time) but by 128-bit loads of whichever lane the
