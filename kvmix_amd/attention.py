@@ -190,7 +190,7 @@ class KVmixAttention:
             if inplace is not None:
                 if use_cache:
                     inplace.append(key_states, value_states, prompt=True)
-            else:
+            elif use_cache:
                 k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(key_states, (None,) * 3, value_states,
                                                                          (None,) * 3, prompt=True)
                 k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()

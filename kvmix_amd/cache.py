@@ -231,6 +231,15 @@ class PackedKVCache:
         self._v_tail.len += 1
         self.kv_seq_len += 1
 
+    def reset(self) -> None:
+        """Forget every token; the buffers stay allocated and are reused by the next prompt."""
+        self.kv_seq_len = self.k_tokens = self.v_tokens = 0
+        for tail in (self._k_tail, self._v_tail):
+            tail.start = tail.len = 0
+            if tail.buf is not None:
+                tail.buf.zero_()  # window() relies on slots past the live length reading as zero
+        self._packed_views = (None,) * 6
+
     # -- views -----------------------------------------------------------------------------
     def as_tuple(self) -> Tuple:
         """The reference's 9-tuple (models/modeling_llama_KVmix.py:270-273) as views of the
