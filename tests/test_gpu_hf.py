@@ -225,3 +225,27 @@ def test_three_bit_values_and_refusals(dev):
         model(ids, past_key_values=DynamicCache(config=model.config), use_cache=True)
     with pytest.raises(RuntimeError):
         stock(ids, past_key_values=model.new_cache(), use_cache=True)
+
+
+def test_recipe_profile_then_generate(dev):
+    """Inference-comparision.py:56-153 in small: profile the stock model, build the KVmix model
+    from the bits it returns, generate from a padded batch."""
+    from kvmix_amd.hf import LlamaForCausalLM_KVmix
+    from kvmix_amd.profiler import profile_model
+
+    stock, _ = build_pair("llama", dev, {i: {} for i in range(10)})
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, 1000, (1, 64), generator=g).to(dev) for _ in range(2)]
+    quant_bits = profile_model(stock, prompts, [torch.ones_like(p) for p in prompts], [p.clone() for p in prompts], 10)
+    assert sorted(e["k_bits"] for e in quant_bits.values()) == [2] * 8 + [3] * 2
+    assert sorted(e["v_bits"] for e in quant_bits.values()) == [2] * 8 + [4] * 2
+    model = LlamaForCausalLM_KVmix(stock.config, quant_bits=quant_bits)
+    model.load_state_dict(stock.state_dict())
+    model = model.half().to(dev).eval()
+    ids = torch.randint(0, 1000, (4, 200), generator=g).to(dev)
+    mask = torch.ones_like(ids)
+    mask[0, :30] = 0
+    out = model.generate(ids, attention_mask=mask, max_new_tokens=48, do_sample=False, pad_token_id=0)
+    assert out.shape == (4, 248)
+    want = stock.eval().generate(ids, attention_mask=mask, max_new_tokens=1, do_sample=False, pad_token_id=0)
+    assert torch.equal(out[:, 200], want[:, 200])
