@@ -239,6 +239,26 @@ size_t kvmix_decode_attention_workspace_bytes(const kvmix_decode_attn_t *step);
 int kvmix_decode_attention(const kvmix_decode_attn_t *step, void *workspace, size_t workspace_bytes,
                            kvmix_stream_t stream);
 
+/*
+ * The same step in one pass over the positions: every block computes the logits of one slab of
+ * positions, keeps exp(logit - slab maximum) on chip and multiplies it into the values of the same
+ * positions; a second small kernel merges the slabs (two launches, no logits or probabilities in
+ * memory).  It takes the same descriptor; `probs` and `probs_stride` are ignored (no probabilities
+ * are returned).  It follows models/modeling_llama_KVmix.py:68-75,180-211 up to the softmax (fp16
+ * logits, 1/sqrt(D), mask, clamp) but not the reference's roundings after it: probabilities are not
+ * rounded to fp16 and the quantized and tail halves of the output are not rounded separately, so the
+ * result differs from kvmix_decode_attention's by up to about 2^-10 of the largest value magnitude.
+ *
+ * Supported (kvmix_decode_attention_fused_supported returns 1, else the call returns
+ * KVMIX_ERR_UNSUPPORTED): D = 128; keys 1/2/4-bit in groups of 32 or the reference's 3-bit words;
+ * values 1/2/4-bit or dense 3-bit in groups of 32; 1, 2, 4 or 8 query heads per kv head.
+ * workspace: at least kvmix_decode_attention_fused_workspace_bytes() bytes of device scratch.
+ */
+int kvmix_decode_attention_fused_supported(const kvmix_decode_attn_t *step);
+size_t kvmix_decode_attention_fused_workspace_bytes(const kvmix_decode_attn_t *step);
+int kvmix_decode_attention_fused(const kvmix_decode_attn_t *step, void *workspace, size_t workspace_bytes,
+                                 kvmix_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,9 @@ EXPORTS = (
     "kvmix_quantized_gemv",
     "kvmix_decode_attention_workspace_bytes",
     "kvmix_decode_attention",
+    "kvmix_decode_attention_fused_supported",
+    "kvmix_decode_attention_fused_workspace_bytes",
+    "kvmix_decode_attention_fused",
 )
 
 _lib = None
@@ -104,6 +107,12 @@ def load() -> ctypes.CDLL:
     L.kvmix_decode_attention_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
     L.kvmix_decode_attention.restype = i32
     L.kvmix_decode_attention.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
+    L.kvmix_decode_attention_fused_supported.restype = i32
+    L.kvmix_decode_attention_fused_supported.argtypes = [ctypes.POINTER(DecodeAttn)]
+    L.kvmix_decode_attention_fused_workspace_bytes.restype = sz
+    L.kvmix_decode_attention_fused_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
+    L.kvmix_decode_attention_fused.restype = i32
+    L.kvmix_decode_attention_fused.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
     _lib = L
     return L
 

@@ -143,12 +143,17 @@ class KVmixAttention:
 
     # -- the step --------------------------------------------------------------------------
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
-                past_key_value=None, attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True):
+                past_key_value=None, attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True,
+                need_weights: bool = True):
         """query_states [B,nh,Q,D], key/value_states [B,Hkv,Q,D] (fp16, after RoPE).
         past_key_value: None (prompt), the reference's 9-tuple (a new tuple is returned, grown by
         concatenation as the reference does), or a PackedKVCache (updated in place and returned;
         an empty one means prompt).
-        Returns (attn_output [B,nh,Q,D] fp16, attn_weights fp16, past_key_value or None)."""
+        need_weights=False lets a single-token step run as one pass over the positions where that
+        is the faster form; no probabilities exist then and attn_weights is None (the output differs
+        from the other form by the reference's roundings after the softmax, about 2^-10 of the
+        largest value).
+        Returns (attn_output [B,nh,Q,D] fp16, attn_weights fp16 or None, past_key_value or None)."""
         B, nh, q_len, D = query_states.shape
         n_rep = nh // key_states.shape[1]
         inplace = past_key_value if isinstance(past_key_value, PackedKVCache) else None
@@ -177,9 +182,12 @@ class KVmixAttention:
                 if attention_mask is not None and attention_mask.shape[-2:] != (1, kv_seq_len):
                     raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
                                      f"{(B, nh, 1, kv_seq_len)}")
+                single = (not need_weights) and ops.prefer_single_pass(
+                    B, nh, key_states.shape[1], D, kv_seq_len, self.k_bits, k_fmt, k_group, self.v_bits, v_fmt,
+                    self.Vgroup_size)
                 attn_output, attn_weights = ops.decode_attention(
                     query_states, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, k_group, self.k_bits, self.Vgroup_size,
-                    self.v_bits, k_fmt, v_fmt, attention_mask)
+                    self.v_bits, k_fmt, v_fmt, attention_mask, single_pass=single)
             else:
                 attn_output, attn_weights = self._decode_with_torch_glue(
                     query_states, kc, ks, km, k_tail, vc, vs, vm, v_tail, k_group, k_fmt, v_fmt, n_rep, attention_mask)

@@ -67,6 +67,29 @@ __device__ __forceinline__ float scale_for_output(float range, float scale_div, 
     return scale_mode == KVMIX_SCALE_RECIPROCAL ? range * inv_qmax : scale_div;
 }
 
+// Halving butterfly over lanes.  v[0..NV) of every lane are summed across the lanes whose
+// indices differ in the bits {FIRST, 2*FIRST, ...} (UP = 1: up to bit 32; UP = 0: FIRST, FIRST/2,
+// ... down to bit 1).  A step halves what a lane holds: the lane with the step's bit clear
+// keeps the lower half, its partner the upper half.  Returns the index (in the original
+// numbering) of the value left in v[0]; the lane's remaining values follow it in order.
+template <int NV, int FIRST, int UP>
+__device__ __forceinline__ int scatter_reduce(float *v, int lane)
+{
+    if constexpr (NV <= 1 || FIRST < 1 || FIRST >= kWave) {
+        return 0;
+    } else {
+        constexpr int H = NV / 2;
+        const bool up = (lane & FIRST) != 0;
+#pragma unroll
+        for (int i = 0; i < H; i++) {
+            const float keep = up ? v[H + i] : v[i];
+            const float send = up ? v[i] : v[H + i];
+            v[i] = keep + __shfl_xor(send, FIRST);
+        }
+        return (up ? H : 0) + scatter_reduce<H, UP ? FIRST * 2 : FIRST / 2, UP>(v, lane);
+    }
+}
+
 inline int launch_status()
 {
     return hipGetLastError() == hipSuccess ? KVMIX_OK : KVMIX_ERR_LAUNCH;

@@ -95,8 +95,8 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
 
 class Decoder:
     """weights: the dict of init_weights; attention: one callable per layer with the signature
-    attention(q [B,nh,Q,D], k [B,nkv,Q,D], v [B,nkv,Q,D], cache, attention_mask=...) ->
-    (out [B,nh,Q,D], attn_weights, cache);  caches: the per-layer cache objects to start from
+    attention(q [B,nh,Q,D], k [B,nkv,Q,D], v [B,nkv,Q,D], cache, attention_mask=..., need_weights=False) ->
+    (out [B,nh,Q,D], attn_weights or None, cache);  caches: the per-layer cache objects to start from
     (None = the reference's "no past" prompt call)."""
 
     def __init__(self, cfg: DecoderConfig, weights: dict, attention: Sequence[Callable],
@@ -120,7 +120,7 @@ class Decoder:
         for li, lw in enumerate(self.w["layers"]):
             h = rms_norm(x, lw["input_norm"], cfg.rms_norm_eps)
             q, k, v = project_qkv(cfg, h, lw["wqkv"], cos, sin)
-            out, _, self.caches[li] = self.attention[li](q, k, v, self.caches[li], attention_mask=mask)
+            out, _, self.caches[li] = self.attention[li](q, k, v, self.caches[li], attention_mask=mask, need_weights=False)
             out = out.transpose(1, 2).reshape(B, Q, cfg.hidden_size)
             x = x + F.linear(out, lw["wo"])
             h = rms_norm(x, lw["post_norm"], cfg.rms_norm_eps)
@@ -195,9 +195,12 @@ class GraphDecoder(Decoder):
             kwin.index_copy_(2, kslot, k)
             vwin.index_copy_(2, vslot, v)
             kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
+            width = max(cache.k_tokens, cache.v_tokens) + R
+            single = ops.prefer_single_pass(B, cfg.num_heads, cfg.num_kv_heads, D, width, cache.k_bits, cache.k_fmt,
+                                            cache.Kgroup_size, cache.v_bits, cache.v_fmt, cache.Vgroup_size)
             out, _ = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, cache.Kgroup_size, cache.k_bits,
                                           cache.Vgroup_size, cache.v_bits, cache.k_fmt, cache.v_fmt,
-                                          k_tail_len=klive, v_tail_len=vlive)
+                                          k_tail_len=klive, v_tail_len=vlive, single_pass=single)
             out = out.transpose(1, 2).reshape(B, 1, cfg.hidden_size)
             x = x + F.linear(out, lw["wo"])
             h = rms_norm(x, lw["post_norm"], cfg.rms_norm_eps)

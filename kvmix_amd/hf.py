@@ -160,7 +160,8 @@ class _KVmixAttentionForward:
             attention_mask = attention_mask.to(torch.float32)
         packed = None if past_key_values is None else past_key_values.packed(self.layer_idx)
         attn_output, attn_weights, _ = self.kvmix(query_states, key_states, value_states, packed,
-                                                  attention_mask=attention_mask, use_cache=packed is not None)
+                                                  attention_mask=attention_mask, use_cache=packed is not None,
+                                                  need_weights=bool(kwargs.get("output_attentions", False)))
         attn_output = attn_output.transpose(1, 2).reshape(*input_shape, -1).contiguous()
         return self.o_proj(attn_output), attn_weights
 

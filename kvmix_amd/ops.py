@@ -13,6 +13,8 @@ from __future__ import annotations
 
 from typing import Tuple
 
+import functools
+
 import torch
 
 from . import _lib
@@ -275,12 +277,51 @@ def quantized_gemm(group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: 
     return out
 
 
+# Up to this many (batch x query head x position) entries the single-pass step is the faster one
+# (measured on MI355X, Llama-2-7B heads: 12-20 us against 20-30 us at 1-4 sequences of 2k-4k tokens;
+# equal at about 2^19 entries, i.e. 1024 blocks, twice slower at 16 x 8k).  Keys in the reference's
+# 3-bit words break even earlier.
+SINGLE_PASS_MAX_ENTRIES = 1 << 19
+SINGLE_PASS_MAX_ENTRIES_REF3 = 360_000
+
+
+def prefer_single_pass(batch: int, heads: int, kv_heads: int, head_dim: int, width: int, k_bits: int, k_fmt: int,
+                       k_group: int, v_bits: int, v_fmt: int, v_group: int) -> bool:
+    """Policy for callers that do not need the probabilities: whether the single-pass step is both
+    available for this layout and the faster of the two at this size."""
+    if kv_heads <= 0 or heads % kv_heads != 0:
+        return False
+    limit = SINGLE_PASS_MAX_ENTRIES_REF3 if (k_bits == 3 and k_fmt == _lib.FMT_REF) else SINGLE_PASS_MAX_ENTRIES
+    if batch * heads * width > limit:
+        return False
+    return single_pass_supported(head_dim, heads // kv_heads, k_bits, k_fmt, k_group, v_bits, v_fmt, v_group)
+
+
+@functools.lru_cache(maxsize=None)
+def single_pass_supported(head_dim: int, heads_per_kv: int, k_bits: int, k_fmt: int, k_group: int, v_bits: int,
+                          v_fmt: int, v_group: int) -> bool:
+    """Whether decode_attention(single_pass=True) takes a cache of this layout (asks the library)."""
+    import ctypes
+
+    st = _lib.DecodeAttn()
+    st.D, st.heads_per_kv, st.heads, st.samples = head_dim, heads_per_kv, heads_per_kv, heads_per_kv
+    st.k_bits, st.k_fmt, st.k_group, st.k_tokens = k_bits, k_fmt, k_group, (11 if k_group == 11 else 32) * 32
+    st.v_bits, st.v_fmt, st.v_group, st.v_tokens = v_bits, v_fmt, v_group, 32
+    return bool(_lib.load().kvmix_decode_attention_fused_supported(ctypes.byref(st)))
+
+
 def decode_attention(q: torch.Tensor, k_packed, v_packed, k_tail: torch.Tensor, v_tail: torch.Tensor,
                      k_group: int, k_bits: int, v_group: int, v_bits: int, k_fmt: int = _lib.FMT_REF,
-                     v_fmt: int = _lib.FMT_REF, attention_mask=None, k_tail_len=None, v_tail_len=None):
+                     v_fmt: int = _lib.FMT_REF, attention_mask=None, k_tail_len=None, v_tail_len=None,
+                     single_pass: bool = False):
     """One decode step of attention over the packed cache plus its fp16 tails, in four or five
     launches (no reference operator: it is what models/modeling_llama_KVmix.py:180-211 composes
     from quantized_gemm, matmul, cat and softmax).
+
+    single_pass=True runs the step as one pass over the positions instead (two launches, logits and
+    probabilities stay on chip); no probabilities are returned (probs is None) and the roundings
+    after the softmax are not the reference's (see the header).  Layouts the single-pass kernels do
+    not take raise RuntimeError; `single_pass_supported` tells beforehand.
 
     q [B,nh,1,D] fp16; k_packed = (code [B,Hkv,D,Tk/vpw], scale, min) or None; v_packed =
     (code [B,Hkv,Tv,D/vpw], scale, min) or None; k_tail, v_tail [B,Hkv,slots,D] fp16.
@@ -360,8 +401,18 @@ def decode_attention(q: torch.Tensor, k_packed, v_packed, k_tail: torch.Tensor, 
         keep.append(attention_mask)
         st.mask, st.mask_stride = attention_mask.data_ptr(), attention_mask.stride(0) if B > 1 else width
     st.samples, st.heads, st.heads_per_kv, st.D = B * nh, nh, nh // nkv, D
-    probs = torch.empty((B, nh, 1, width), dtype=torch.float16, device=q.device)
     out = torch.empty((B, nh, 1, D), dtype=torch.float16, device=q.device)
+    if single_pass:
+        st.out, st.out_stride = out.data_ptr(), D
+        if not L.kvmix_decode_attention_fused_supported(ctypes.byref(st)):
+            raise RuntimeError("the single-pass attention step does not take this layout (head_dim 128, keys 1/2/4-bit "
+                               "group 32 or reference 3-bit, values 1/2/4-bit or dense 3-bit group 32)")
+        ws_bytes = L.kvmix_decode_attention_fused_workspace_bytes(ctypes.byref(st))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        with torch.cuda.device(q.device):
+            _lib.check(L.kvmix_decode_attention_fused(ctypes.byref(st), ws.data_ptr(), ws_bytes, _stream(q)))
+        return out, None
+    probs = torch.empty((B, nh, 1, width), dtype=torch.float16, device=q.device)
     st.probs, st.probs_stride, st.out, st.out_stride = probs.data_ptr(), width, out.data_ptr(), D
     ws_bytes = L.kvmix_decode_attention_workspace_bytes(ctypes.byref(st))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None

@@ -25,8 +25,8 @@ class Recorder:
     def __init__(self, att, keep_prompt_out=True):
         self.att, self.calls, self.keep_prompt_out = att, [], keep_prompt_out
 
-    def __call__(self, q, k, v, cache, attention_mask=None):
-        out, p, cache = self.att(q, k, v, cache, attention_mask=attention_mask)
+    def __call__(self, q, k, v, cache, attention_mask=None, need_weights=True):
+        out, p, cache = self.att(q, k, v, cache, attention_mask=attention_mask, need_weights=need_weights)
         keep_out = self.keep_prompt_out or q.shape[2] == 1
         self.calls.append((q.contiguous().cpu().numpy(), k.contiguous().cpu().numpy(), v.contiguous().cpu().numpy(),
                            out.cpu().numpy() if keep_out else None))
@@ -67,7 +67,7 @@ class OracleAttention:
         return self.o.attention_decode_step(q, k, v, cache, self.k_bits, self.v_bits, 0.0, 0.0, group_size=self.group,
                                             fixed_window=self.window)
 
-    def __call__(self, q, k, v, cache, attention_mask=None):
+    def __call__(self, q, k, v, cache, attention_mask=None, need_weights=True):
         dt = q.dtype
         qn, kn, vn = (np.ascontiguousarray(t.to(torch.float16).numpy()) for t in (q, k, v))
         if cache is None:

@@ -62,8 +62,8 @@ class Tap:
     def __init__(self, att, keep_masks=False):
         self.att, self.calls, self.keep_masks = att, [], keep_masks
 
-    def __call__(self, q, k, v, cache, attention_mask=None, use_cache=True):
-        out, p, cache = self.att(q, k, v, cache, attention_mask=attention_mask, use_cache=use_cache)
+    def __call__(self, q, k, v, cache, attention_mask=None, use_cache=True, need_weights=True):
+        out, p, cache = self.att(q, k, v, cache, attention_mask=attention_mask, use_cache=use_cache, need_weights=need_weights)
         rec = tuple(t.contiguous().cpu().numpy() for t in (q, k, v, out))
         if self.keep_masks:
             rec += (None if attention_mask is None else attention_mask.cpu().numpy(),)
