@@ -404,6 +404,62 @@ def sweep_extra(torch, _lib, lib, dev, stream):
     return res
 
 
+def attention_step_extra(torch, dev):
+    """The whole attention step of one layer (logits over packed keys + fp16 tail, softmax, output
+    over packed values + fp16 tail) in its two forms: four launches with the reference's roundings,
+    and one pass over the positions (two launches).  MHA 32 x 128, 128-token fp16 tails; buffer sets
+    are rotated so that they come from HBM; launches replayed from a HIP graph."""
+    from kvmix_amd import ops
+
+    H, D, R = 32, 128, 128
+    res = {}
+    side = torch.cuda.Stream()
+    for (B, T, kb, vb) in [(1, 4096, 4, 4), (4, 2304, 4, 4), (4, 2304, 3, 2), (4, 2304, 2, 2), (8, 8192, 4, 4), (16, 8192, 4, 4)]:
+        kg = 11 if kb == 3 else 32
+        tk, tv = ((T - R) // kg) * kg, ((T - R) // 32) * 32
+        kbytes = (1024 / 11 if kb == 3 else 16 * kb + 16) * tk
+        nbytes = B * H * (kbytes + (16 * vb + 16) * tv + (2 * T - tk - tv) * 2 * D)
+        nsets = int(min(48, max(2, -(-(600 << 20) // int(nbytes)))))
+        sets = []
+        for _ in range(nsets):
+            kw = tk // 11 if kb == 3 else tk * kb // 32
+            kq = (torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, kw), dtype=torch.int64, device=dev).to(torch.int32),
+                  (torch.rand(B, H, D, tk // kg, device=dev) * 0.05).half(), (torch.randn(B, H, D, tk // kg, device=dev) * 0.3).half())
+            vq = (torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, tv, D * vb // 32), dtype=torch.int64, device=dev).to(torch.int32),
+                  (torch.rand(B, H, tv, D // 32, device=dev) * 0.2).half(), torch.randn(B, H, tv, D // 32, device=dev).half())
+            sets.append((kq, vq, torch.randn(B, H, T - tk, D, device=dev).half(), torch.randn(B, H, T - tv, D, device=dev).half()))
+        q = torch.randn(B, H, 1, D, device=dev).half()
+        entry = {"packed_plus_tail_MB": round(nbytes / 1e6, 1)}
+        for name, single in (("four_launch", False), ("single_pass", True)):
+            def fn(i):
+                kq, vq, kt, vt = sets[i % nsets]
+                return ops.decode_attention(q, kq, vq, kt, vt, kg, kb, 32, vb, single_pass=single)
+            iters = max(30, 2 * nsets)
+            with torch.cuda.stream(side):
+                for i in range(nsets):
+                    fn(i)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(iters):
+                        fn(i)
+                graph.replay()
+                torch.cuda.synchronize()
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                graph.replay()
+                e.record()
+                torch.cuda.synchronize()
+            us = s.elapsed_time(e) * 1e3 / iters
+            del graph
+            entry[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
+        entry["chosen"] = "single_pass" if ops.prefer_single_pass(B, H, H, D, T, kb, 0, kg, vb, 0, 32) else "four_launch"
+        res[f"B{B}_T{T}_k{kb}v{vb}"] = entry
+        del sets
+        torch.cuda.empty_cache()
+    return res
+
+
 def e2e_extra(torch, dev, batch=4, prompt_len=2048, new_tokens=512):
     """BASELINE configs[4]: greedy decoding on a random-init Llama-2-7B (fp16 weights ~N(0, 0.02), seed 4),
     prompt of random token ids, mixed per-layer bits as in configs[1], 128-token fp16 window, in-place
@@ -508,6 +564,8 @@ def main():
                "gqa_config2_B16_T32768": gqa_shape_extra(torch, _lib, lib, dev, st)}
         if not args.no_sweep:
             res["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, st)
+        torch.cuda.empty_cache()
+        res["attention_step"] = attention_step_extra(torch, dev)
         print(json.dumps(res))
         return
     kbits, vbits = layer_bits(args.layers)
@@ -634,6 +692,9 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
         torch.cuda.empty_cache()
     if not args.no_target_shape and not args.no_sweep:
         result["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, torch.cuda.current_stream().cuda_stream)
+    if not args.no_target_shape:
+        torch.cuda.empty_cache()
+        result["attention_step"] = attention_step_extra(torch, dev)
     if not args.no_e2e:
         torch.cuda.empty_cache()
         try:

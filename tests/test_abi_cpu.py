@@ -112,6 +112,54 @@ def test_decode_attention_host_validation_needs_no_gpu(lib):
     assert lib.kvmix_decode_attention_workspace_bytes(ctypes.byref(big)) == lib.kvmix_gemv_workspace_bytes(4, 1, 4096, 128)
 
 
+def test_single_pass_attention_host_validation_needs_no_gpu(lib):
+    """kvmix_decode_attention_fused: what it takes, what it refuses, how much scratch it asks for."""
+    from kvmix_amd import _lib
+
+    def desc(**kw):
+        st = _lib.DecodeAttn()
+        st.q, st.q_stride, st.out, st.out_stride = 16, 128, 16, 128
+        st.k_tail, st.v_tail = 16, 16
+        st.k_tail_batch_stride = st.v_tail_batch_stride = 8 * 128
+        st.k_tail_token_stride = st.v_tail_token_stride = 128
+        st.k_tail_slots = st.v_tail_slots = st.k_tail_len = st.v_tail_len = 8
+        st.samples, st.heads, st.heads_per_kv, st.D = 4, 4, 1, 128
+        st.k_bits = st.v_bits = 4
+        st.k_group = st.v_group = 32
+        for k, v in kw.items():
+            setattr(st, k, v)
+        return st
+
+    sup = lambda st: lib.kvmix_decode_attention_fused_supported(ctypes.byref(st))
+    call = lambda st, ws=None, n=0: lib.kvmix_decode_attention_fused(ctypes.byref(st), ws, n, None)
+    assert sup(desc()) == 1
+    assert sup(desc(D=64)) == 0
+    assert sup(desc(heads_per_kv=3)) == 0
+    assert sup(desc(k_tokens=64, k_group=64)) == 0                       # key groups other than 32
+    assert sup(desc(k_tokens=64, k_bits=3, k_group=32, k_fmt=_lib.FMT_DENSE3)) == 0   # dense 3-bit keys
+    assert sup(desc(k_tokens=66, k_bits=3, k_group=11)) == 1             # the reference's 3-bit words
+    assert sup(desc(v_tokens=32, v_bits=3)) == 0                         # 3-bit values only in the dense format
+    assert sup(desc(v_tokens=32, v_bits=3, v_fmt=_lib.FMT_DENSE3)) == 1
+    assert lib.kvmix_decode_attention_fused(None, None, 0, None) == -7
+    assert call(desc(D=64)) == -9
+    assert call(desc(heads=3)) == -5
+    assert call(desc(k_tail_len=9)) == -8
+    assert call(desc(v_tail_len=5)) == -8
+    assert call(desc(samples=0)) == 0
+    assert call(desc(k_tokens=48, k_code=16, k_scale=16, k_zero=16, k_code_row_stride=6, k_sz_row_stride=2,
+                     k_tail_len=8, v_tail_slots=56, v_tail_len=56)) == -8   # 48 key tokens are not whole groups of 32
+    assert call(desc(k_tokens=64, k_code=16, k_scale=16, k_zero=16, k_code_row_stride=7, k_sz_row_stride=2,
+                     v_tail_slots=72, v_tail_len=72)) == -8               # a key row of 64 4-bit codes is 8 words
+    assert call(desc(k_tokens=64, v_tail_slots=72, v_tail_len=72)) == -7  # quantized keys without their pointers
+    # scratch: (D + 2) floats per row and slab of 512 positions (704 with the reference's 3-bit keys)
+    assert lib.kvmix_decode_attention_fused_workspace_bytes(ctypes.byref(desc())) == 4 * 1 * 130 * 4
+    long = desc(k_tokens=2048, v_tokens=2048)
+    assert lib.kvmix_decode_attention_fused_workspace_bytes(ctypes.byref(long)) == 4 * 5 * 130 * 4
+    ref3 = desc(k_tokens=2046, k_bits=3, k_group=11, v_tokens=2048)
+    assert lib.kvmix_decode_attention_fused_workspace_bytes(ctypes.byref(ref3)) == 4 * 3 * 130 * 4
+    assert call(long, None, 0) in (-7, -11)                               # pointers / scratch missing: refused before any launch
+
+
 def test_python_ops_reject_bad_arguments_like_the_reference():
     import KVmix
 
