@@ -529,6 +529,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the batch sweep of BASELINE configs[3]")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end Llama-2-7B-shape decode loop")
     ap.add_argument("--e2e-only", action="store_true", help="run only the end-to-end decode loop")
+    ap.add_argument("--no-attention-step", action="store_true", help="skip the attention-step comparison")
+    ap.add_argument("--attention-step-only", action="store_true", help="run only the attention-step comparison")
     ap.add_argument("--shapes-only", action="store_true",
                     help="skip the step: only the B=16/T=8192 target shape and the GQA configuration (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -551,6 +553,16 @@ def main():
     if args.e2e_only:
         print(json.dumps({"e2e_config4_llama2_7b": e2e_extra(torch, dev)}))
         return
+    if args.attention_step_only:
+        if args.copy_calibration:
+            src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
+        print(json.dumps({"attention_step": attention_step_extra(torch, dev)}))
+        return
     if args.shapes_only:
         if args.copy_calibration:
             src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -564,8 +576,9 @@ def main():
                "gqa_config2_B16_T32768": gqa_shape_extra(torch, _lib, lib, dev, st)}
         if not args.no_sweep:
             res["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, st)
-        torch.cuda.empty_cache()
-        res["attention_step"] = attention_step_extra(torch, dev)
+        if not args.no_attention_step:
+            torch.cuda.empty_cache()
+            res["attention_step"] = attention_step_extra(torch, dev)
         print(json.dumps(res))
         return
     kbits, vbits = layer_bits(args.layers)
@@ -692,7 +705,7 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
         torch.cuda.empty_cache()
     if not args.no_target_shape and not args.no_sweep:
         result["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, torch.cuda.current_stream().cuda_stream)
-    if not args.no_target_shape:
+    if not args.no_target_shape and not args.no_attention_step:
         torch.cuda.empty_cache()
         result["attention_step"] = attention_step_extra(torch, dev)
     if not args.no_e2e:

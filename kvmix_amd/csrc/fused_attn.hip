@@ -292,9 +292,18 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
     __shared__ float scratch[kFusedWaves];
 
     const int tid = threadIdx.x;
-    const int slab = blockIdx.x;
-    const int64_t kv = blockIdx.y;
-    const int64_t sample0 = kv * a.heads_per_kv + (int64_t)blockIdx.z * NREP;
+    // Workgroups go to the 8 XCDs (each with its own L2) round-robin in launch order.  The launch
+    // index is mapped to a logical one such that consecutive logical indices share an XCD, and the
+    // logical order is slab-fastest, then query head, then kv head: the slabs of one row of scales
+    // (neighbours share 128-byte lines) and the query heads of one kv head meet in one L2.
+    const int64_t n_blocks = (int64_t)gridDim.x * gridDim.y * gridDim.z;
+    const int64_t launch = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    const int64_t per = n_blocks / 8, rem = n_blocks % 8, xcd = launch % 8;
+    const int64_t logical = xcd * per + (xcd < rem ? xcd : rem) + launch / 8;
+    const int slab = (int)(logical % gridDim.x);
+    const int head_group = (int)((logical / gridDim.x) % gridDim.z);
+    const int64_t kv = logical / ((int64_t)gridDim.x * gridDim.z);
+    const int64_t sample0 = kv * a.heads_per_kv + (int64_t)head_group * NREP;
     const int S = a.slab;
     const int64_t t0 = (int64_t)slab * S, t1 = t0 + S;
     int64_t k_len = a.k_len_dev ? *a.k_len_dev : a.k_len;
@@ -454,22 +463,41 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
     }
 }
 
-// grid = samples, one thread per head dimension: out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M)
+// grid = samples, one thread per head dimension: out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M).
+// The slab weights are computed once per block into LDS; the partial outputs are then read with
+// independent loads (a slab without a live position has weight 0, nothing is skipped).
+constexpr int kMergeChunk = 128;  // slabs whose weights are in LDS at a time
 __global__ void __launch_bounds__(kFusedD) attn_fused_merge(const float *ws_o, const float *ws_ml, int slabs, uint16_t *out,
                                                             int64_t o_bs)
 {
+    __shared__ float wgt[kMergeChunk];
+    __shared__ float part[kFusedD / kWave];
     const int64_t sample = blockIdx.x;
     const int c = threadIdx.x;
     const float *ml = ws_ml + sample * slabs * 2;
+    // the row maximum: every thread takes a share of the slabs, then the block combines
     float M = -INFINITY;
-    for (int s = 0; s < slabs; s++) M = fmaxf(M, ml[2 * s]);
+    for (int s = c; s < slabs; s += kFusedD) M = fmaxf(M, ml[2 * s]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+    if (c % kWave == 0) part[c / kWave] = M;
+    __syncthreads();
+    M = fmaxf(part[0], part[1]);
     float L = 0.f, o = 0.f;
-    for (int s = 0; s < slabs; s++) {
-        const float m = ml[2 * s];
-        if (m == -INFINITY) continue;  // a slab without a live position
-        const float w = expf(m - M);
-        L = fmaf(ml[2 * s + 1], w, L);
-        o = fmaf(ws_o[(sample * slabs + s) * kFusedD + c], w, o);
+    for (int s0 = 0; s0 < slabs; s0 += kMergeChunk) {
+        const int n = slabs - s0 < kMergeChunk ? slabs - s0 : kMergeChunk;
+        __syncthreads();  // (wgt may still be read from the previous chunk)
+        if (c < n) {
+            const float m = ml[2 * (s0 + c)];
+            wgt[c] = m == -INFINITY ? 0.f : expf(m - M);
+        }
+        __syncthreads();
+        const float *op = ws_o + (sample * slabs + s0) * kFusedD + c;
+#pragma unroll 8
+        for (int s = 0; s < n; s++) {
+            L = fmaf(ml[2 * (s0 + s) + 1], wgt[s], L);
+            o = fmaf(op[(int64_t)s * kFusedD], wgt[s], o);
+        }
     }
     out[sample * o_bs + c] = f32_to_h16(L > 0.f ? o / L : 0.f);
 }
