@@ -259,6 +259,44 @@ size_t kvmix_decode_attention_fused_workspace_bytes(const kvmix_decode_attn_t *s
 int kvmix_decode_attention_fused(const kvmix_decode_attn_t *step, void *workspace, size_t workspace_bytes,
                                  kvmix_stream_t stream);
 
+/*
+ * The tail append of a decode step fused with the rotary embedding before it: what
+ * LlamaAttention_KVmix.forward does at models/modeling_llama_KVmix.py:102-112 for one new token
+ * (apply_rotary_pos_emb on q and k, then torch.cat of k and v onto the fp16 tails), in one launch
+ * and without re-allocating the tails.
+ *
+ *   qkv     [batch, heads + 2 * kv_heads, D] fp16: the query heads, then the key heads, then the
+ *           value heads of the new token (the output of a fused q/k/v projection)
+ *   cos, sin [D] fp16 for the token's position (rotate-half convention: both halves of D hold the
+ *           same angles)
+ *   q_out   [batch, heads, D] fp16: the rotated queries
+ *   k_tail, v_tail [batch, kv_heads, slots, D] fp16 windows of the cache tails; the rotated key
+ *           heads / the value heads are written to slot k_slot / v_slot, read from *_slot_dev when
+ *           that is not NULL (a step replayed from a captured graph).  A device-side slot outside
+ *           the window writes nothing.
+ * The rotation is evaluated as the fp16 tensor expression x * cos + rotate_half(x) * sin evaluates
+ * it (products and sum each rounded to fp16), so it is bit-identical to that composition.
+ * D must be a multiple of 16.
+ */
+typedef struct kvmix_rope_append {
+    const void *qkv;
+    int64_t qkv_batch_stride;
+    const void *cos, *sin;
+    void *q_out;
+    int64_t q_batch_stride;
+    void *k_tail;
+    int64_t k_tail_batch_stride, k_tail_head_stride, k_tail_token_stride, k_tail_slots, k_slot;
+    const int64_t *k_slot_dev;
+    void *v_tail;
+    int64_t v_tail_batch_stride, v_tail_head_stride, v_tail_token_stride, v_tail_slots, v_slot;
+    const int64_t *v_slot_dev;
+    int64_t batch;
+    int heads, kv_heads;
+    int64_t D;
+} kvmix_rope_append_t;
+
+int kvmix_rope_append(const kvmix_rope_append_t *step, kvmix_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,6 +28,7 @@ EXPORTS = (
     "kvmix_decode_attention_fused_supported",
     "kvmix_decode_attention_fused_workspace_bytes",
     "kvmix_decode_attention_fused",
+    "kvmix_rope_append",
 )
 
 _lib = None
@@ -72,6 +73,18 @@ class DecodeAttn(ctypes.Structure):
                 ("probs", _vp), ("probs_stride", _i64), ("out", _vp), ("out_stride", _i64)]
 
 
+class RopeAppend(ctypes.Structure):
+    """kvmix_rope_append_t"""
+    _i64, _i32, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+    _fields_ = [("qkv", _vp), ("qkv_batch_stride", _i64), ("cos", _vp), ("sin", _vp),
+                ("q_out", _vp), ("q_batch_stride", _i64),
+                ("k_tail", _vp), ("k_tail_batch_stride", _i64), ("k_tail_head_stride", _i64),
+                ("k_tail_token_stride", _i64), ("k_tail_slots", _i64), ("k_slot", _i64), ("k_slot_dev", _vp),
+                ("v_tail", _vp), ("v_tail_batch_stride", _i64), ("v_tail_head_stride", _i64),
+                ("v_tail_token_stride", _i64), ("v_tail_slots", _i64), ("v_slot", _i64), ("v_slot_dev", _vp),
+                ("batch", _i64), ("heads", _i32), ("kv_heads", _i32), ("D", _i64)]
+
+
 class KVmixLibraryMissing(ImportError):
     pass
 
@@ -113,6 +126,8 @@ def load() -> ctypes.CDLL:
     L.kvmix_decode_attention_fused_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
     L.kvmix_decode_attention_fused.restype = i32
     L.kvmix_decode_attention_fused.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
+    L.kvmix_rope_append.restype = i32
+    L.kvmix_rope_append.argtypes = [ctypes.POINTER(RopeAppend), vp]
     _lib = L
     return L
 

@@ -189,11 +189,10 @@ class GraphDecoder(Decoder):
         for li, lw in enumerate(self.w["layers"]):
             cache = self.caches[li]
             h = rms_norm(x, lw["input_norm"], cfg.rms_norm_eps)
-            q, k, v = project_qkv(cfg, h, lw["wqkv"], cos, sin)
             kwin, vwin, _, _ = cache.tail_windows(R)
             (kslot, klive), (vslot, vlive) = self._len[li]
-            kwin.index_copy_(2, kslot, k)
-            vwin.index_copy_(2, vslot, v)
+            # rotary embedding of q and k and the append of k and v to the tail windows: one launch
+            q = ops.rope_append(F.linear(h, lw["wqkv"]), cos, sin, cfg.num_heads, cfg.num_kv_heads, kwin, vwin, kslot, vslot)
             kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
             width = max(cache.k_tokens, cache.v_tokens) + R
             single = ops.prefer_single_pass(B, cfg.num_heads, cfg.num_kv_heads, D, width, cache.k_bits, cache.k_fmt,

@@ -297,6 +297,56 @@ def prefer_single_pass(batch: int, heads: int, kv_heads: int, head_dim: int, wid
     return single_pass_supported(head_dim, heads // kv_heads, k_bits, k_fmt, k_group, v_bits, v_fmt, v_group)
 
 
+def rope_append(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int, kv_heads: int,
+                k_tail: torch.Tensor, v_tail: torch.Tensor, k_slot, v_slot) -> torch.Tensor:
+    """Rotary embedding of the new token's query and key heads and the append of its key and value
+    heads to the cache tails, in one launch (models/modeling_llama_KVmix.py:102-112 for one token).
+
+    qkv [B, 1, (heads + 2 kv_heads) * D] or [B, heads + 2 kv_heads, D] fp16: query, key, value heads
+    of the new token; cos, sin: D fp16 values for its position (any shape with D elements);
+    k_tail, v_tail [B, kv_heads, slots, D] fp16 windows, written in place at slot k_slot / v_slot
+    (ints, or one-element int64 device tensors read when the kernel runs).
+    Returns the rotated queries [B, heads, 1, D].  Bit-identical to x * cos + rotate_half(x) * sin
+    in fp16 tensor arithmetic."""
+    import ctypes
+
+    for t in (qkv, cos, sin, k_tail, v_tail):
+        if t.dtype != torch.float16:
+            raise RuntimeError(f"expected scalar type Half but found {t.dtype}")
+    _need_gpu(qkv, cos, sin, k_tail, v_tail)
+    B, D = qkv.shape[0], k_tail.shape[-1]
+    total = heads + 2 * kv_heads
+    if qkv.numel() != B * total * D or cos.numel() != D or sin.numel() != D:
+        raise RuntimeError("rope_append: qkv must hold heads + 2 * kv_heads rows of D values per batch element, cos and sin D values")
+    if k_tail.dim() != 4 or v_tail.dim() != 4 or k_tail.shape[:2] != (B, kv_heads) or v_tail.shape[:2] != (B, kv_heads) \
+            or v_tail.shape[-1] != D or k_tail.stride(3) != 1 or v_tail.stride(3) != 1:
+        raise RuntimeError("rope_append: tails must be [B, kv_heads, slots, D] with unit stride along D")
+    qkv = qkv.reshape(B, total * D)
+    if qkv.stride(1) != 1:
+        qkv = qkv.contiguous()
+    cos, sin = cos.reshape(D).contiguous(), sin.reshape(D).contiguous()
+    q_out = torch.empty((B, heads, 1, D), dtype=torch.float16, device=qkv.device)
+    st = _lib.RopeAppend()
+    st.qkv, st.qkv_batch_stride, st.cos, st.sin = qkv.data_ptr(), qkv.stride(0) if B > 1 else total * D, cos.data_ptr(), sin.data_ptr()
+    st.q_out, st.q_batch_stride = q_out.data_ptr(), heads * D
+    for prefix, tail, slot in (("k", k_tail, k_slot), ("v", v_tail, v_slot)):
+        setattr(st, prefix + "_tail", tail.data_ptr())
+        setattr(st, prefix + "_tail_batch_stride", tail.stride(0))
+        setattr(st, prefix + "_tail_head_stride", tail.stride(1))
+        setattr(st, prefix + "_tail_token_stride", tail.stride(2))
+        setattr(st, prefix + "_tail_slots", tail.shape[2])
+        if torch.is_tensor(slot):
+            if slot.dtype != torch.int64 or slot.numel() != 1 or not slot.is_cuda:
+                raise RuntimeError("a device-side slot must be one int64 element on the GPU")
+            setattr(st, prefix + "_slot_dev", slot.data_ptr())
+        else:
+            setattr(st, prefix + "_slot", int(slot))
+    st.batch, st.heads, st.kv_heads, st.D = B, heads, kv_heads, D
+    with torch.cuda.device(qkv.device):
+        _lib.check(_lib.load().kvmix_rope_append(ctypes.byref(st), _stream(qkv)))
+    return q_out
+
+
 @functools.lru_cache(maxsize=None)
 def single_pass_supported(head_dim: int, heads_per_kv: int, k_bits: int, k_fmt: int, k_group: int, v_bits: int,
                           v_fmt: int, v_group: int) -> bool:

@@ -160,6 +160,34 @@ def test_single_pass_attention_host_validation_needs_no_gpu(lib):
     assert call(long, None, 0) in (-7, -11)                               # pointers / scratch missing: refused before any launch
 
 
+def test_rope_append_host_validation_needs_no_gpu(lib):
+    from kvmix_amd import _lib
+
+    def desc(**kw):
+        st = _lib.RopeAppend()
+        st.qkv, st.cos, st.sin, st.q_out, st.k_tail, st.v_tail = 16, 16, 16, 16, 16, 16
+        st.batch, st.heads, st.kv_heads, st.D = 2, 8, 2, 128
+        st.qkv_batch_stride, st.q_batch_stride = 12 * 128, 8 * 128
+        st.k_tail_batch_stride = st.v_tail_batch_stride = 2 * 16 * 128
+        st.k_tail_head_stride = st.v_tail_head_stride = 16 * 128
+        st.k_tail_token_stride = st.v_tail_token_stride = 128
+        st.k_tail_slots = st.v_tail_slots = 16
+        for k, v in kw.items():
+            setattr(st, k, v)
+        return st
+
+    call = lambda st: lib.kvmix_rope_append(ctypes.byref(st), None)
+    assert lib.kvmix_rope_append(None, None) == -7
+    assert call(desc(kv_heads=3)) == -5               # 8 query heads over 3 kv heads
+    assert call(desc(D=72)) == -9                     # the head dimension must be a multiple of 16
+    assert call(desc(qkv_batch_stride=11 * 128)) == -8
+    assert call(desc(k_slot=16)) == -8                # host-side slot outside the window
+    assert call(desc(v_slot=-1)) == -8
+    assert call(desc(k_tail_token_stride=64)) == -8
+    assert call(desc(cos=None)) == -7
+    assert call(desc(batch=0)) == 0
+
+
 def test_python_ops_reject_bad_arguments_like_the_reference():
     import KVmix
 
