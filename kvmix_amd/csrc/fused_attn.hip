@@ -3,8 +3,8 @@
 // that slab's logits from the packed keys (and the fp16 key tail where the slab reaches it), turns
 // them into unnormalised probabilities exp(l - m_slab) kept in LDS, multiplies them into the packed
 // values (and the fp16 value tail) of the same positions, and writes (m_slab, sum_slab, partial
-// out[D]) per head; a second small kernel merges the slabs.  Logits and probabilities never go to
-// memory.
+// out[D]) per head; a second small kernel merges the slabs (a row that fits one slab is finished
+// by the first kernel).  Logits and probabilities never go to memory.
 //
 // Arithmetic against the reference's decode branch (models/modeling_llama_KVmix.py:68-75,180-211):
 // logits are rounded to fp16 before the 1/sqrt(D) scaling exactly as there (its GEMV and its tail
@@ -30,6 +30,8 @@ struct FusedArgs {
     const uint16_t *k_tail, *v_tail;  // [kv samples, slots, D]
     const float *mask;        // optional [batch, width]
     const int64_t *k_len_dev, *v_len_dev;
+    uint16_t *out;            // [samples, D]: written by the slab kernel itself when there is one slab
+    int64_t o_bs;
     float *ws_o;              // [samples, slabs, D]
     float *ws_ml;             // [samples, slabs, 2]: slab maximum, slab sum
     int64_t q_bs, kc_bs, kc_rs, ksz_bs, ksz_rs, vc_bs, vc_rs, vsz_bs, vsz_rs;
@@ -452,9 +454,10 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
         float o = 0.f;
 #pragma unroll
         for (int w = 0; w < kFusedWaves; w++) o += red[(w * NREP + h) * kFusedD + c];
-        a.ws_o[((sample0 + h) * a.slabs + slab) * kFusedD + c] = o;
+        if (a.slabs == 1) a.out[(sample0 + h) * a.o_bs + c] = f32_to_h16(l_h[h] > 0.f ? o / l_h[h] : 0.f);
+        else a.ws_o[((sample0 + h) * a.slabs + slab) * kFusedD + c] = o;
     }
-    if (tid == 0) {
+    if (tid == 0 && a.slabs > 1) {
 #pragma unroll
         for (int h = 0; h < NREP; h++) {
             a.ws_ml[((sample0 + h) * a.slabs + slab) * 2 + 0] = m_h[h];
@@ -600,6 +603,8 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     a.mask = p->mask;
     a.k_len_dev = p->k_tail_len_dev;
     a.v_len_dev = p->v_tail_len_dev;
+    a.out = (uint16_t *)p->out;
+    a.o_bs = p->out_stride;
     a.ws_o = (float *)workspace;
     a.ws_ml = a.ws_o + p->samples * slabs * kFusedD;
     a.q_bs = p->q_stride;
@@ -636,7 +641,7 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     const dim3 grid((unsigned)slabs, (unsigned)kv_samples, (unsigned)p->heads_per_kv);
     hipLaunchKernelGGL(attn_fused_slab<1>, grid, dim3(kFusedThreads), 0, st, a);
     int rc = launch_status();
-    if (rc != KVMIX_OK) return rc;
+    if (rc != KVMIX_OK || slabs == 1) return rc;  // a single slab is normalised and stored by the slab kernel
     hipLaunchKernelGGL(attn_fused_merge, dim3((unsigned)p->samples), dim3(kFusedD), 0, st, a.ws_o, a.ws_ml, (int)slabs,
                        (uint16_t *)p->out, p->out_stride);
     return launch_status();
