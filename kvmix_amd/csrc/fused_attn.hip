@@ -57,15 +57,18 @@ struct __attribute__((packed, aligned(2))) H4 {
     uint16_t v[4];
 };
 
-#ifndef KVMIX_FUSED_THREADS
-#define KVMIX_FUSED_THREADS 512
+// Lanes that share a key row.  A lane owns 32 positions (one quantization group) or four of the
+// reference's 3-bit words, so this sets the slab; the block has 32 key rows in flight per step.
+#ifndef KVMIX_FUSED_KEY_LANES
+#define KVMIX_FUSED_KEY_LANES 16
 #endif
-constexpr int kFusedThreads = KVMIX_FUSED_THREADS;
+constexpr int kKeyLanes = KVMIX_FUSED_KEY_LANES;
+constexpr int kFusedThreads = 32 * kKeyLanes;
 constexpr int kFusedWaves = kFusedThreads / kWave;
 constexpr int kFusedD = 128;
-constexpr int kSlabG32 = 512;   // 16 lanes x 32 positions (one quantization group each)
-constexpr int kSlabRef3 = 704;  // 16 lanes x four 11-code words
-constexpr int kRedStride = 16 * 45;  // floats per (wave, head) in `red`: 16 lanes x (44 + 1 pad)
+constexpr int kSlabG32 = kKeyLanes * 32;
+constexpr int kSlabRef3 = kKeyLanes * 44;
+constexpr int kRedStride = kKeyLanes * 45;  // floats per (wave, head) in `red`: lanes x (44 + 1 pad)
 constexpr float kLowest = -3.4028234663852886e38f;
 constexpr float kPatternUp = 1237940039285380274899124224.0f;  // 2^90
 
@@ -113,10 +116,38 @@ __device__ __forceinline__ void fma_fields_ref3(uint32_t w, float m, float *acc)
 
 __device__ __forceinline__ constexpr float ref3_unscale(int i) { return field_unscale(3 * (i < 8 ? i : i - 8)); }
 
-// Logits of the slab's quantized positions.  Sixteen lanes share a key row (one head dimension):
+// Sum v[0..NV) over the lanes whose indices differ in the bits FIRST, 2 FIRST, .. LAST.  While the
+// count is even a step halves what a lane holds (the lane with the bit clear keeps the lower half,
+// its partner the upper half); once it is odd the remaining steps are plain exchanges and the
+// lanes that differ only in those bits end with the same sums.  Returns the index, in the original
+// numbering, of what is left in v[0]; `left` = how many values are left.
+template <int NV, int FIRST, int LAST>
+__device__ __forceinline__ int fold_lanes(float *v, int lane, int &left)
+{
+    if constexpr (FIRST > LAST) {
+        left = NV;
+        return 0;
+    } else if constexpr (NV % 2 == 0) {
+        constexpr int H = NV / 2;
+        const bool up = (lane & FIRST) != 0;
+#pragma unroll
+        for (int i = 0; i < H; i++) {
+            const float keep = up ? v[H + i] : v[i];
+            const float send = up ? v[i] : v[H + i];
+            v[i] = keep + __shfl_xor(send, FIRST);
+        }
+        return (up ? H : 0) + fold_lanes<H, FIRST * 2, LAST>(v, lane, left);
+    } else {
+#pragma unroll
+        for (int i = 0; i < NV; i++) v[i] += __shfl_xor(v[i], FIRST);
+        return fold_lanes<NV, FIRST * 2, LAST>(v, lane, left);
+    }
+}
+
+// Logits of the slab's quantized positions.  kKeyLanes lanes share a key row (one head dimension):
 // a lane owns 32 consecutive positions = one quantization group (16 / 8 / 4 bytes of codes, one
-// scale, one zero), or four of the reference's 3-bit words; a block covers kFusedThreads / 16 head
-// dimensions per step.  The sums of the lanes that share positions meet in `red`
+// scale, one zero), or four of the reference's 3-bit words; a block covers 32 head dimensions per
+// step.  The sums of the lanes that share positions meet in `red`
 // ([wave][head][lane * (LPP + 1) + position]).
 template <int MODE, int NREP>
 __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv, int64_t t0, const float *qs, float *red)
@@ -126,7 +157,7 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
     constexpr int UNIT = MODE == 3 ? 11 : 32;          // positions per (scale, zero)
     constexpr int NSZ = MODE == 3 ? 4 : 1;
     const int tid = threadIdx.x;
-    const int sub = tid % 16, dg = tid / 16;
+    const int sub = tid % kKeyLanes, dg = tid / kKeyLanes;
     const int lane = tid % kWave, wave = tid / kWave;
     const int64_t first = t0 + (int64_t)sub * LPP;       // first position of this lane
     const int64_t left = a.k_tokens - first;               // quantized positions from there on (a multiple of UNIT)
@@ -145,7 +176,7 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
         const uint32_t *codes = a.k_code + kv * a.kc_bs + word0;
         const int64_t sz0 = kv * a.ksz_bs + first / UNIT;
 #pragma unroll
-        for (int d = dg; d < kFusedD; d += kFusedThreads / 16) {
+        for (int d = dg; d < kFusedD; d += kFusedThreads / kKeyLanes) {
             Words<WORDS> w;
             uint16_t sc[NSZ], zr[NSZ];
             const uint32_t *cp = codes + (int64_t)d * a.kc_rs;
@@ -191,8 +222,7 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
             }
         }
     }
-    // undo the pattern scaling, add the zero term, fold the four head-dimension phases of the wave
-    // (halving butterfly: every lane ends with a quarter of the positions)
+    // undo the pattern scaling, add the zero term, fold the head-dimension phases of the wave
 #pragma unroll
     for (int h = 0; h < NREP; h++) {
 #pragma unroll
@@ -200,9 +230,12 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
             if (MODE == 3) acc[h][i] = fmaf(acc[h][i], ref3_unscale(i % 11), zacc[h][i / 11]);
             else acc[h][i] = fmaf(acc[h][i], field_unscale(field_offset(MODE, i % (32 / MODE))), zacc[h][0]);
         }
-        const int at = scatter_reduce<LPP, 16, 1>(acc[h], lane);
+        int left;
+        const int at = fold_lanes<LPP, kKeyLanes, 32>(acc[h], lane, left);
 #pragma unroll
-        for (int i = 0; i < LPP / 4; i++) red[(wave * NREP + h) * kRedStride + sub * (LPP + 1) + at + i] = acc[h][i];
+        for (int i = 0; i < LPP; i++) {
+            if (i < left) red[(wave * NREP + h) * kRedStride + sub * (LPP + 1) + at + i] = acc[h][i];
+        }
     }
 }
 
