@@ -177,6 +177,7 @@ class PackedKVCache:
             raise RuntimeError(f"expected scalar type Half but found {key_states.dtype}")
         if not key_states.is_cuda:
             raise RuntimeError("KVmix operators run on the GPU only: got a tensor on " + str(key_states.device))
+        key_states, value_states = key_states.detach(), value_states.detach()  # the cache is not part of any autograd graph
         n = key_states.shape[2]
         reserve = 4 * max(self.residual_length or 0, 2 * self.Vgroup_size, n)
         self._k_tail.append(key_states, reserve)

@@ -206,12 +206,14 @@ class _KVmixCausalLM:
 
     def forward(self, input_ids=None, attention_mask=None, position_ids=None, past_key_values=None,
                 inputs_embeds=None, labels=None, use_cache=None, **kwargs):
+        # a cache is created when the caller asks for one (or leaves it to the config) and is not
+        # computing a loss; a cache that is passed in is always used
         use = self.config.use_cache if use_cache is None else use_cache
-        if use:
+        if use_cache is None and labels is not None:
+            use = False
+        if use or past_key_values is not None:
             n = input_ids.shape[1] if input_ids is not None else inputs_embeds.shape[1]
             past_key_values = self._with_cache({"past_key_values": past_key_values}, max(4096, 2 * n))["past_key_values"]
-        else:
-            use, past_key_values = False, None
         return super().forward(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids,
                                past_key_values=past_key_values, inputs_embeds=inputs_embeds, labels=labels,
                                use_cache=use, **kwargs)

@@ -249,3 +249,7 @@ def test_recipe_profile_then_generate(dev):
     assert out.shape == (4, 248)
     want = stock.eval().generate(ids, attention_mask=mask, max_new_tokens=1, do_sample=False, pad_token_id=0)
     assert torch.equal(out[:, 200], want[:, 200])
+    # the profiler also runs on the converted model (a loss computation creates no cache) and, the
+    # cache-less forward being the stock one, ranks the layers the same way
+    again = profile_model(model, prompts, [torch.ones_like(p) for p in prompts], [p.clone() for p in prompts], 10)
+    assert again == quant_bits

@@ -75,3 +75,7 @@ def test_cached_forward_needs_the_gpu_and_the_right_cache():
         stock(ids, past_key_values=model.new_cache())
     with pytest.raises(NotImplementedError):
         model.generate(ids, num_beams=4, max_new_tokens=2)
+    # a loss computation creates no cache (and therefore runs anywhere), as the stock model's does
+    fp32 = _pair("llama")[1]
+    out = fp32(ids, labels=ids)
+    assert out.past_key_values is None and out.loss.requires_grad
