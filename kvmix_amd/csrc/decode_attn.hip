@@ -40,14 +40,17 @@ struct __attribute__((packed, aligned(2))) H8 {
     uint16_t v[8];
 };
 
-// One block per (batch, head) and nothing else resident on its CU: the kernels are chains of short
-// latency-bound phases, so the block is as wide as it can be (16 waves) to shorten each phase.
-constexpr int kAttnThreads = 1024;
-constexpr int kAttnGroups = kAttnThreads / 16;  // 16-lane groups, one tail token each
+// One block per (batch, head).  The kernels are chains of short latency-bound phases, so with at
+// most one row per CU the block is as wide as it can be (16 waves) to shorten each phase; with more
+// rows than CUs, 8-wave blocks let two rows share a CU instead of queueing behind each other.
+constexpr int kAttnThreadsWide = 1024;
+constexpr int kAttnThreadsNarrow = 512;
+constexpr int kAttnRowEntries = 16384;  // longest row the softmax keeps in registers
 
+template <int THREADS>
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scratch)
 {
-    // kAttnThreads / 64 waves; xor-shuffles inside the wave, then one value per wave through LDS
+    // THREADS / 64 waves; xor-shuffles inside the wave, then one value per wave through LDS
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) {
         const float other = __shfl_xor(v, o);
@@ -59,18 +62,19 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *scrat
     __syncthreads();
     float r = scratch[0];
 #pragma unroll
-    for (int w = 1; w < kAttnThreads / kWave; w++) r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+    for (int w = 1; w < THREADS / kWave; w++) r = is_max ? fmaxf(r, scratch[w]) : r + scratch[w];
     return r;
 }
 
 // grid = samples.  Sixteen lanes share a tail token (eight head dimensions each) and every lane group
 // has two tokens in flight, so a block covers 128 tail tokens per step.  The softmax keeps a row of up
-// to 16384 entries in registers (two 8-entry vectors per thread): one read, one write.
-constexpr int kRowVecs = 2;
+// to 16384 entries in registers (two or four 8-entry vectors per thread): one read, one write.
 constexpr int kTailUnroll = 2;
 
-__global__ void __launch_bounds__(kAttnThreads) attn_tail_softmax(AttnArgs a)
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS) attn_tail_softmax(AttnArgs a)
 {
+    constexpr int kAttnThreads = THREADS, kAttnGroups = THREADS / 16, kRowVecs = kAttnRowEntries / (THREADS * 8);
     __shared__ float scratch[kAttnThreads / kWave];
     const int64_t sample = blockIdx.x;
     const int64_t kv = sample / a.heads_per_kv;
@@ -139,7 +143,7 @@ __global__ void __launch_bounds__(kAttnThreads) attn_tail_softmax(AttnArgs a)
 #pragma unroll
             for (int i = 0; i < 8; i++) mx = fmaxf(mx, x[v][i]);
         }
-        mx = block_reduce(mx, true, scratch);
+        mx = block_reduce<THREADS>(mx, true, scratch);
         float sum = 0.f;
 #pragma unroll
         for (int v = 0; v < kRowVecs; v++) {
@@ -149,7 +153,7 @@ __global__ void __launch_bounds__(kAttnThreads) attn_tail_softmax(AttnArgs a)
                 sum += x[v][i];
             }
         }
-        sum = block_reduce(sum, false, scratch);
+        sum = block_reduce<THREADS>(sum, false, scratch);
 #pragma unroll
         for (int v = 0; v < kRowVecs; v++) {
             const int64_t i0 = ((int64_t)v * kAttnThreads + tid) * 8;
@@ -170,17 +174,19 @@ __global__ void __launch_bounds__(kAttnThreads) attn_tail_softmax(AttnArgs a)
     // longer rows: three passes over the row (it stays in L2)
     float mx = -INFINITY;
     for (int64_t i = tid; i < a.width; i += kAttnThreads) mx = fmaxf(mx, value(i, row[i]));
-    mx = block_reduce(mx, true, scratch);
+    mx = block_reduce<THREADS>(mx, true, scratch);
     float sum = 0.f;
     for (int64_t i = tid; i < a.width; i += kAttnThreads) sum += expf(value(i, row[i]) - mx);
-    sum = block_reduce(sum, false, scratch);
+    sum = block_reduce<THREADS>(sum, false, scratch);
     for (int64_t i = tid; i < a.width; i += kAttnThreads) row[i] = f32_to_h16(expf(value(i, row[i]) - mx) / sum);
 }
 
 // grid = samples: thread t owns head dimensions 8*(t%16).. of the tokens t/16, t/16 + 64, ...
 // out = fp16( fp16(out from the quantized values) + fp16(sum_j p[v_tokens + j] * v_tail[j]) )
-__global__ void __launch_bounds__(kAttnThreads) attn_tail_output(AttnArgs a)
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS) attn_tail_output(AttnArgs a)
 {
+    constexpr int kAttnGroups = THREADS / 16;
     __shared__ float part[kAttnGroups][129];
     const int64_t sample = blockIdx.x;
     const int64_t kv = sample / a.heads_per_kv;
@@ -301,7 +307,9 @@ extern "C" int kvmix_decode_attention(const kvmix_decode_attn_t *p, void *worksp
     a.inv_sqrt_d = 1.0f / sqrtf((float)p->D);
     hipStream_t st = (hipStream_t)stream;
     if (p->samples > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    hipLaunchKernelGGL(attn_tail_softmax, dim3((unsigned)p->samples), dim3(kAttnThreads), 0, st, a);
+    const bool narrow = p->samples > 256;  // more rows than CUs
+    if (narrow) hipLaunchKernelGGL(attn_tail_softmax<kAttnThreadsNarrow>, dim3((unsigned)p->samples), dim3(kAttnThreadsNarrow), 0, st, a);
+    else hipLaunchKernelGGL(attn_tail_softmax<kAttnThreadsWide>, dim3((unsigned)p->samples), dim3(kAttnThreadsWide), 0, st, a);
     int rc = launch_status();
     if (rc != KVMIX_OK) return rc;
     if (p->v_tokens > 0) {
@@ -311,6 +319,7 @@ extern "C" int kvmix_decode_attention(const kvmix_decode_attn_t *p, void *worksp
                                   p->out_stride, p->out_stride, workspace, workspace_bytes, stream);
         if (rc != KVMIX_OK) return rc;
     }
-    hipLaunchKernelGGL(attn_tail_output, dim3((unsigned)p->samples), dim3(kAttnThreads), 0, st, a);
+    if (narrow) hipLaunchKernelGGL(attn_tail_output<kAttnThreadsNarrow>, dim3((unsigned)p->samples), dim3(kAttnThreadsNarrow), 0, st, a);
+    else hipLaunchKernelGGL(attn_tail_output<kAttnThreadsWide>, dim3((unsigned)p->samples), dim3(kAttnThreadsWide), 0, st, a);
     return launch_status();
 }
