@@ -515,6 +515,73 @@ def e2e_extra(torch, dev, batch=4, prompt_len=2048, new_tokens=512):
     }
 
 
+def hf_generate_extra(torch, dev, batch=4, prompt_len=2048, new_tokens=512):
+    """The reference's own harness in small (Inference-comparision.py:89-201): `generate()` of the
+    stock model with its fp16 cache against `LlamaForCausalLM_KVmix.generate()` with the packed
+    cache, same random-init Llama-2-7B-shaped weights, same prompt; throughput counted over all
+    tokens as the reference prints it (:147-151), plus the memory both caches add to the weights."""
+    import gc
+
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from kvmix_amd.hf import LlamaForCausalLM_KVmix
+
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+                      num_key_value_heads=32, vocab_size=32000, max_position_embeddings=4096)
+    cfg._attn_implementation = "eager"
+    kbits, vbits = layer_bits(32)
+    quant_bits = {i: {"k_bits": kbits[i], "v_bits": vbits[i]} for i in range(32)}
+    cfg.residual_length = 128  # the fixed window of BASELINE configs[4] instead of the ratio rule
+
+    def build(cls, **kw):
+        with torch.device("meta"):
+            m = cls(cfg, **kw)
+        m = m.to(torch.float16).to_empty(device=dev)
+        g = torch.Generator(device=dev).manual_seed(4)
+        with torch.no_grad():
+            for name, w in m.named_parameters():
+                if w.dim() == 1:
+                    w.fill_(1.0)
+                else:
+                    w.normal_(0.0, 0.02, generator=g)
+        m.model.rotary_emb.__init__(config=cfg, device=dev)  # (the inverse frequencies are a buffer, not a parameter)
+        return m.eval()
+
+    gen = torch.Generator(device="cpu").manual_seed(4)
+    prompt = torch.randint(0, cfg.vocab_size, (batch, prompt_len), generator=gen).to(dev)
+    mask = torch.ones_like(prompt)
+    res = {"model": "Llama-2-7B shape, random init, fp16, transformers generate(), eager attention",
+           "batch": batch, "prompt_tokens": prompt_len, "new_tokens": new_tokens}
+    for name, cls, kw in (("stock_fp16_cache", LlamaForCausalLM, {}), ("kvmix_packed_cache", LlamaForCausalLM_KVmix, {"quant_bits": quant_bits})):
+        model = build(cls, **kw)
+        model.generate(prompt[:1, :64], attention_mask=mask[:1, :64], max_new_tokens=8, do_sample=False, pad_token_id=0)  # warm-up
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats(dev)
+        before = torch.cuda.memory_allocated(dev)
+        t0 = time.perf_counter()
+        out = model.generate(prompt, attention_mask=mask, max_new_tokens=new_tokens, min_new_tokens=new_tokens, do_sample=False,
+                             pad_token_id=0)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        res[name] = {"wall_s": round(wall, 3), "all_tokens_per_s": round(out.numel() / wall, 1),
+                     "new_tokens_per_s": round(batch * new_tokens / wall, 1),
+                     "peak_memory_above_weights_MB": round((torch.cuda.max_memory_allocated(dev) - before) / 2 ** 20, 1)}
+        # what the cache itself holds for this context: one more prompt forward, cache kept alive
+        cache = model.new_cache(prompt_len + 1) if hasattr(model, "new_cache") else None
+        torch.cuda.empty_cache()
+        base = torch.cuda.memory_allocated(dev)
+        with torch.no_grad():
+            o = model(prompt, attention_mask=mask, past_key_values=cache, use_cache=True, logits_to_keep=1)
+        cache = o.past_key_values
+        del o
+        torch.cuda.synchronize()
+        res[name]["cache_MB_after_prompt"] = round((torch.cuda.memory_allocated(dev) - base) / 2 ** 20, 1)
+        del model, out, cache
+        gc.collect()
+        torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -529,6 +596,10 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the batch sweep of BASELINE configs[3]")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end Llama-2-7B-shape decode loop")
     ap.add_argument("--e2e-only", action="store_true", help="run only the end-to-end decode loop")
+    ap.add_argument("--hf-batch", type=int, default=4)
+    ap.add_argument("--hf-new-tokens", type=int, default=512)
+    ap.add_argument("--hf-only", action="store_true",
+                    help="run only the transformers generate() comparison (stock fp16 cache against the KVmix wrappers)")
     ap.add_argument("--no-attention-step", action="store_true", help="skip the attention-step comparison")
     ap.add_argument("--attention-step-only", action="store_true", help="run only the attention-step comparison")
     ap.add_argument("--shapes-only", action="store_true",
@@ -552,6 +623,9 @@ def main():
     B, H, D, T, R = args.batch, 32, 128, args.context, 128
     if args.e2e_only:
         print(json.dumps({"e2e_config4_llama2_7b": e2e_extra(torch, dev)}))
+        return
+    if args.hf_only:
+        print(json.dumps({"hf_generate_config4": hf_generate_extra(torch, dev, batch=args.hf_batch, new_tokens=args.hf_new_tokens)}))
         return
     if args.attention_step_only:
         if args.copy_calibration:
@@ -714,6 +788,11 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
             result["e2e_config4_llama2_7b"] = e2e_extra(torch, dev)
         except Exception as ex:  # the headline line must still be printed
             result["e2e_config4_llama2_7b"] = {"error": f"{type(ex).__name__}: {ex}"}
+        torch.cuda.empty_cache()
+        try:
+            result["hf_generate_config4"] = hf_generate_extra(torch, dev)
+        except Exception as ex:
+            result["hf_generate_config4"] = {"error": f"{type(ex).__name__}: {ex}"}
     print(json.dumps(result))
 
 

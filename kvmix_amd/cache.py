@@ -59,12 +59,12 @@ class _Tail:
     def append(self, new: torch.Tensor, reserve: int) -> None:
         B, H, n, D = new.shape
         if self.buf is None:
-            self.buf = torch.zeros((B, H, max(reserve, 2 * n), D), dtype=new.dtype, device=new.device)
+            self.buf = torch.zeros((B, H, max(reserve, n), D), dtype=new.dtype, device=new.device)
         cap = self.buf.shape[2]
         if self.start + self.len + n > cap:
             live = self.view()
-            if 2 * (self.len + n) > cap:  # the tail itself has grown: a longer buffer
-                buf = torch.zeros((B, H, max(2 * cap, 2 * (self.len + n)), D), dtype=new.dtype, device=new.device)
+            if self.len + n > cap:  # the tail itself has outgrown the buffer: a longer one
+                buf = torch.zeros((B, H, max(2 * cap, self.len + n), D), dtype=new.dtype, device=new.device)
                 buf[:, :, :self.len].copy_(live)
                 self.buf = buf
             else:  # room at the front: move the live tokens there (regions may overlap)
@@ -179,13 +179,23 @@ class PackedKVCache:
             raise RuntimeError("KVmix operators run on the GPU only: got a tensor on " + str(key_states.device))
         key_states, value_states = key_states.detach(), value_states.detach()  # the cache is not part of any autograd graph
         n = key_states.shape[2]
-        reserve = 4 * max(self.residual_length or 0, 2 * self.Vgroup_size, n)
-        self._k_tail.append(key_states, reserve)
-        self._v_tail.append(value_states, reserve)
+        steady = max((self.residual_length or 0) + self.Vgroup_size, 2 * self.Vgroup_size)  # a tail between two flushes
+        # Many tokens onto empty tails (a prompt): what the policy flushes is quantized straight from
+        # the incoming tensors and only the rest is kept in fp16, so the tails never hold the prompt.
+        direct = n > 1 and self._k_tail.len == 0 and self._v_tail.len == 0
+        if direct:
+            nk = flush_length(n, self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
+            nv = flush_length(n, self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
+            reserve = max(steady, n - nk, n - nv) + 2 * self.Vgroup_size
+            self._k_tail.append(key_states[:, :, nk:], reserve)
+            self._v_tail.append(value_states[:, :, nv:], reserve)
+        else:
+            reserve = steady + 2 * self.Vgroup_size + n
+            self._k_tail.append(key_states, reserve)
+            self._v_tail.append(value_states, reserve)
+            nk = flush_length(self._k_tail.len, self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
+            nv = flush_length(self._v_tail.len, self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
         self.kv_seq_len += n
-
-        nk = flush_length(self._k_tail.len, self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
-        nv = flush_length(self._v_tail.len, self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
         if nk == 0 and nv == 0:
             return
         self._reserve(key_states, nk, nv)
@@ -195,14 +205,15 @@ class PackedKVCache:
             w0, g0 = self._words(self.k_tokens, self.k_bits, self.k_fmt), self.k_tokens // self.Kgroup_size
             w1, g1 = self._words(self.k_tokens + nk, self.k_bits, self.k_fmt), (self.k_tokens + nk) // self.Kgroup_size
             k_out = (self._k[0][..., w0:w1], self._k[1][..., g0:g1], self._k[2][..., g0:g1])
-            k_chunk = self._k_tail.view()[:, :, :nk]
+            k_chunk = key_states[:, :, :nk] if direct else self._k_tail.view()[:, :, :nk]
         if nv > 0:
             v_out = tuple(t[:, :, self.v_tokens:self.v_tokens + nv] for t in self._v)
-            v_chunk = self._v_tail.view()[:, :, :nv]
+            v_chunk = value_states[:, :, :nv] if direct else self._v_tail.view()[:, :, :nv]
         ops.quantize_kv_flush_into(k_chunk, self.Kgroup_size, self.k_bits, k_out, v_chunk, self.Vgroup_size,
                                    self.v_bits, v_out, self.k_fmt, self.v_fmt)
-        self._k_tail.drop_front(nk)
-        self._v_tail.drop_front(nv)
+        if not direct:
+            self._k_tail.drop_front(nk)
+            self._v_tail.drop_front(nv)
         self.k_tokens += nk
         self.v_tokens += nv
         kc = ks = km = vc = vs = vm = None
