@@ -154,3 +154,23 @@ def test_cache_argument_errors(dev):
         c.append(x.to(dev).float(), x.to(dev).float())
     with pytest.raises(RuntimeError, match="equal shape"):
         c.append(x.to(dev), x.to(dev)[:, :, :, :64])
+
+
+def test_a_prompt_does_not_size_the_tails(dev):
+    """The fp16 tails hold what the policy keeps, not the prompt: a long prompt is quantized straight
+    from the incoming tensors (the cache would otherwise be larger than the fp16 cache it replaces)."""
+    from kvmix_amd.cache import PackedKVCache
+
+    gen = torch.Generator(device=dev).manual_seed(3)
+    k = torch.randn(2, 2, 1500, 128, device=dev, generator=gen).half()
+    v = torch.randn(2, 2, 1500, 128, device=dev, generator=gen).half()
+    fixed = PackedKVCache(4, 2, residual_length=128, capacity=2048)
+    fixed.append(k.transpose(1, 2).contiguous().transpose(1, 2), v, prompt=True)  # (a strided view, as a model hands it over)
+    assert fixed.k_tokens == 1344 and fixed.v_tokens == 1344 and len(fixed.as_tuple()[1][0, 0]) == 156
+    assert fixed._k_tail.buf.shape[2] <= 128 + 32 + 64 and fixed._v_tail.buf.shape[2] <= 128 + 32 + 64
+    for _ in range(300):  # decode steps through several flushes and compactions: the buffers stay that size
+        fixed.append(k[:, :, :1], v[:, :, :1])
+    assert fixed.kv_seq_len == 1800 and fixed._k_tail.buf.shape[2] <= 128 + 32 + 64
+    ratio = PackedKVCache(4, 2, k_residual_ratio=0.2, v_residual_ratio=0.1, capacity=2048)
+    ratio.append(k, v, prompt=True)
+    assert ratio._k_tail.len == 1500 - ratio.k_tokens and ratio._k_tail.buf.shape[2] <= ratio._k_tail.len + 64
