@@ -202,6 +202,21 @@ class KVmixAttention:
                 k_tail, (kc, ks, km), v_tail, (vc, vs, vm) = self._flush(key_states, (None,) * 3, value_states,
                                                                          (None,) * 3, prompt=True)
                 k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
+            if not need_weights and query_states.dtype == torch.float16 and query_states.is_cuda:
+                # nobody reads the probabilities: torch's fused attention, which never holds the
+                # [Q, Q] matrix (fp32 accumulation throughout, where the composition below rounds the
+                # logits and the probabilities to fp16)
+                mask16 = None
+                if attention_mask is not None:
+                    if attention_mask.shape[-2:] != (q_len, kv_seq_len):
+                        raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
+                                         f"{(B, nh, q_len, kv_seq_len)}")
+                    mask16 = attention_mask.clamp(min=torch.finfo(torch.float16).min).to(torch.float16)
+                attn_output = F.scaled_dot_product_attention(query_states, key_states, value_states, attn_mask=mask16,
+                                                             enable_gqa=n_rep > 1)
+                cache = inplace if (use_cache and inplace is not None) else (
+                    (kc, k_tail, ks, km, vc, v_tail, vs, vm, kv_seq_len) if use_cache else None)
+                return attn_output, None, cache
             attn_weights = _grouped_matmul_qk(query_states, key_states, n_rep) / math.sqrt(D)
             if attention_mask is not None:
                 if attention_mask.shape[-2:] != attn_weights.shape[-2:]:

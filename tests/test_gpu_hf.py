@@ -76,7 +76,7 @@ def small_config(kind, layers=4, **extra):
 
     cls = LlamaConfig if kind == "llama" else MistralConfig
     cfg = cls(hidden_size=512, intermediate_size=1024, num_hidden_layers=layers, num_attention_heads=4,
-              num_key_value_heads=2, vocab_size=1000, max_position_embeddings=2048, **extra)
+              num_key_value_heads=2, vocab_size=1000, max_position_embeddings=2048, eos_token_id=None, **extra)  # (no token ends a generation early)
     cfg._attn_implementation = "eager"
     return cfg
 
