@@ -598,6 +598,7 @@ def main():
     ap.add_argument("--e2e-only", action="store_true", help="run only the end-to-end decode loop")
     ap.add_argument("--hf-batch", type=int, default=4)
     ap.add_argument("--hf-new-tokens", type=int, default=512)
+    ap.add_argument("--hf-prompt", type=int, default=2048)
     ap.add_argument("--hf-only", action="store_true",
                     help="run only the transformers generate() comparison (stock fp16 cache against the KVmix wrappers)")
     ap.add_argument("--no-attention-step", action="store_true", help="skip the attention-step comparison")
@@ -625,7 +626,7 @@ def main():
         print(json.dumps({"e2e_config4_llama2_7b": e2e_extra(torch, dev)}))
         return
     if args.hf_only:
-        print(json.dumps({"hf_generate_config4": hf_generate_extra(torch, dev, batch=args.hf_batch, new_tokens=args.hf_new_tokens)}))
+        print(json.dumps({"hf_generate_config4": hf_generate_extra(torch, dev, batch=args.hf_batch, prompt_len=args.hf_prompt, new_tokens=args.hf_new_tokens)}))
         return
     if args.attention_step_only:
         if args.copy_calibration:

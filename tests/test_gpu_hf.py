@@ -253,3 +253,23 @@ def test_recipe_profile_then_generate(dev):
     # cache-less forward being the stock one, ranks the layers the same way
     again = profile_model(model, prompts, [torch.ones_like(p) for p in prompts], [p.clone() for p in prompts], 10)
     assert again == quant_bits
+
+
+def test_cache_reuse_sampling_and_attentions(dev):
+    stock, model = build_pair("llama", dev, BITS)
+    ids = torch.randint(0, 1000, (2, 150), generator=torch.Generator().manual_seed(1)).to(dev)
+    fresh = model.generate(ids, max_new_tokens=40, do_sample=False, pad_token_id=0)
+    cache = model.new_cache(64)
+    first = model.generate(ids, max_new_tokens=40, do_sample=False, pad_token_id=0, past_key_values=cache)
+    cache.reset()
+    assert cache.get_seq_length() == 0
+    again = model.generate(ids, max_new_tokens=40, do_sample=False, pad_token_id=0, past_key_values=cache)
+    assert torch.equal(fresh, first) and torch.equal(fresh, again)  # a reset cache behaves like a new one
+    sampled = model.generate(ids, max_new_tokens=10, do_sample=True, top_k=5, pad_token_id=0)
+    assert sampled.shape == (2, 160)
+    cache = model.new_cache()
+    with torch.no_grad():
+        model(ids, past_key_values=cache, use_cache=True)
+        step = model(ids[:, :1], past_key_values=cache, use_cache=True, output_attentions=True)
+    assert len(step.attentions) == 4 and tuple(step.attentions[0].shape) == (2, 4, 1, 151)  # the four-launch step returns its probabilities
+    assert float((step.attentions[0].float().sum(-1) - 1).abs().max()) < 2e-3
