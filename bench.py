@@ -434,9 +434,9 @@ def attention_step_extra(torch, dev):
             def fn(i):
                 kq, vq, kt, vt = sets[i % nsets]
                 return ops.decode_attention(q, kq, vq, kt, vt, kg, kb, 32, vb, single_pass=single)
-            iters = max(30, 2 * nsets)
+            iters = max(100, 2 * nsets)
             with torch.cuda.stream(side):
-                for i in range(nsets):
+                for i in range(max(nsets, 20)):
                     fn(i)
                 torch.cuda.synchronize()
                 graph = torch.cuda.CUDAGraph()
