@@ -385,7 +385,6 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
         const int64_t j_begin = t0 > a.k_tokens ? t0 - a.k_tokens : 0;
         const int64_t j_end = t1 - a.k_tokens < k_len ? t1 - a.k_tokens : k_len;
         const uint16_t *kt = a.k_tail + kv * a.kt_bs + sub * 8;
-#pragma unroll 4
         for (int64_t j0 = j_begin; j0 < j_end; j0 += kFusedThreads / 16) {
             const int64_t j = j0 + grp;
             const bool in = j < j_end;
