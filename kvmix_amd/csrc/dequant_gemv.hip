@@ -654,21 +654,67 @@ gemv_cols3(GemvArgs a)
         }
     };
 
+    if (kq % U == 0 && kbeg + kq <= K) {
+        // Every section is a whole number of steps (head dimensions of 64, 128, 256 are): the rows are
+        // walked with three running pointers -- one 64-bit add per load instead of a clamp, a
+        // multiply and an add -- and the last step prefetches nothing, so no row past the section is
+        // ever addressed.
+        const uint32_t *cq = cp + (uint32_t)kbeg * c_rs;
+        const uint16_t *sq = sp + (uint32_t)kbeg * s_rs;
+        const uint16_t *zq = zp + (uint32_t)kbeg * s_rs;
+        auto next_row = [&](int u) {
+            cw[u] = *reinterpret_cast<const Words<UPL> *>(cq);
+            sw[u] = *reinterpret_cast<const HalfN *>(sq);
+            zw[u] = *reinterpret_cast<const HalfN *>(zq);
+            cq += c_rs;
+            sq += s_rs;
+            zq += s_rs;
+        };
+        auto step_x = [&](int k0) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        load_row(u, kbeg + u);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll 1
-    for (int st = 0; st < steps; st++) {
-        const int k0 = kbeg + st * U;
-        load_x(k0);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int u = 0; u < U; u++) {
+#pragma unroll
+                for (int h = 0; h < NREP; h++) xr[u][h] = xs[h * (K + 1) + k0 + u];
+            }
+        };
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            compute_row(u, k0 + u);
-            load_row(u, k0 + U + u);
+            next_row(u);
             __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll 1
+        for (int st = 0; st < steps - 1; st++) {
+            const int k0 = kbeg + st * U;
+            step_x(k0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                compute_row(u, k0 + u);
+                next_row(u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        step_x(kbeg + (steps - 1) * U);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; u++) compute_row(u, kbeg + (steps - 1) * U + u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            load_row(u, kbeg + u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll 1
+        for (int st = 0; st < steps; st++) {
+            const int k0 = kbeg + st * U;
+            load_x(k0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                compute_row(u, k0 + u);
+                load_row(u, k0 + U + u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
 
