@@ -531,6 +531,7 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
 //   rows).  Tiles as in gemv_cols: TU = (64/RQ)*4 words per wave, last tile shifted left.
 //   block = (64, 2..4); grid = (tiles/waves, samples, M), XCD-swizzled; dynamic LDS = (K+1)*4.
 // ---------------------------------------------------------------------------------------
+constexpr float kCols3ZeroDown = 8.0779356694631608874e-28f;  // 2^-90: the zero term is accumulated with x * 2^90
 // 2^(59 - offset of code i inside its word or inside word >> 24): undoes the fp32-pattern scaling
 __device__ __forceinline__ constexpr float cols3_out_scale(int i)
 {
@@ -564,7 +565,7 @@ gemv_cols3(GemvArgs a)
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
     for (int i = wy * kWave + lane; i < NREP * (K + 1); i += blockDim.y * kWave) {
         const int h = i / (K + 1), k = i % (K + 1);
-        xs[i] = k < K ? h16_to_f32(xp[h * a.x_bs + k]) : 0.f;
+        xs[i] = k < K ? h16_to_f32(xp[h * a.x_bs + k]) * 1237940039285380274899124224.0f : 0.f;  // x * 2^90, see compute_row
     }
     __syncthreads();
 
@@ -645,9 +646,11 @@ gemv_cols3(GemvArgs a)
             f[9] = __uint_as_float(hi & 0x38u);
             f[10] = __uint_as_float(hi & 0xC0u);
 #pragma unroll
+            // (x arrives multiplied by 2^90: the zero term carries the factor too and loses it at the end;
+            // it stays finite up to |sum x * zero| = 2^37, far beyond what an fp16 result can hold)
             for (int h = 0; h < NREP; h++) {
                 zsum[h][j] = fmaf(xv[h], (float)sz.y, zsum[h][j]);
-                const float mq = (xv[h] * 1237940039285380274899124224.0f) * (float)sz.x;  // 2^90
+                const float mq = fmaf(xv[h], (float)sz.x, 0.f);  // (a multiply; written as an fma so that the fp16 operand needs no conversion)
 #pragma unroll
                 for (int i = 0; i < VALS; i++) acc[j][h][i] = fmaf(mq, f[i], acc[j][h][i]);
             }
@@ -659,16 +662,19 @@ gemv_cols3(GemvArgs a)
         // walked with three running pointers -- one 64-bit add per load instead of a clamp, a
         // multiply and an add -- and the last step prefetches nothing, so no row past the section is
         // ever addressed.
-        const uint32_t *cq = cp + (uint32_t)kbeg * c_rs;
-        const uint16_t *sq = sp + (uint32_t)kbeg * s_rs;
-        const uint16_t *zq = zp + (uint32_t)kbeg * s_rs;
+        // (uniform bases and 32-bit byte offsets per lane: the form a load with a scalar base takes)
+        const uint8_t *cb = reinterpret_cast<const uint8_t *>(a.code + kv * a.c_bs);
+        const uint8_t *sb = reinterpret_cast<const uint8_t *>(reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs);
+        const uint8_t *zb = reinterpret_cast<const uint8_t *>(reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs);
+        uint32_t co = ((uint32_t)unit0 + (uint32_t)kbeg * c_rs) * 4u;
+        uint32_t so = ((uint32_t)unit0 + (uint32_t)kbeg * s_rs) * 2u;
+        const uint32_t c_step = c_rs * 4u, s_step = s_rs * 2u;
         auto next_row = [&](int u) {
-            cw[u] = *reinterpret_cast<const Words<UPL> *>(cq);
-            sw[u] = *reinterpret_cast<const HalfN *>(sq);
-            zw[u] = *reinterpret_cast<const HalfN *>(zq);
-            cq += c_rs;
-            sq += s_rs;
-            zq += s_rs;
+            cw[u] = *reinterpret_cast<const Words<UPL> *>(cb + co);
+            sw[u] = *reinterpret_cast<const HalfN *>(sb + so);
+            zw[u] = *reinterpret_cast<const HalfN *>(zb + so);
+            co += c_step;
+            so += s_step;
         };
         auto step_x = [&](int k0) {
 #pragma unroll
@@ -729,7 +735,7 @@ gemv_cols3(GemvArgs a)
                 for (int j = 0; j < UPL; j++) {
 #pragma unroll
                     for (int i = 0; i < VALS; i++)
-                        part[((wy * NREP + h) * TOT + j * VALS + i) * kWave + lane] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j]);
+                        part[((wy * NREP + h) * TOT + j * VALS + i) * kWave + lane] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j] * kCols3ZeroDown);
                 }
             }
         }
@@ -742,7 +748,7 @@ gemv_cols3(GemvArgs a)
 #pragma unroll
         for (int j = 0; j < UPL; j++) {
 #pragma unroll
-            for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j]);
+            for (int i = 0; i < VALS; i++) flat[j * VALS + i] = fmaf(acc[j][h][i], cols3_out_scale(i), zsum[h][j] * kCols3ZeroDown);
         }
         for (int o = 1; o < ks; o++) {
 #pragma unroll
