@@ -1639,11 +1639,18 @@ gemv_cols_mfma2(GemvArgs a)
     uint16_t xh;
     uint32_t w[KB][4][WL];
 
+    // (with one tile per wave -- the only setting in use -- an item is a chunk: no division per load)
+    constexpr bool kOneTile = KVMIX_MFMA2_MAX_TPW == 1;
+    const int g_first = tile0 * TG + TG <= ngroups ? tile0 * TG : ngroups - TG;
     auto tile_g0 = [&](int it) {
+        if constexpr (kOneTile) return g_first;
         const int g = (tile0 + (nch > 0 ? it / nch : 0) * ntw) * TG;
         return g + TG <= ngroups ? g : ngroups - TG;
     };
-    auto chunk_k0 = [&](int it) { return (ch0 + (nch > 0 ? it % nch : 0)) * CH; };
+    auto chunk_k0 = [&](int it) {
+        if constexpr (kOneTile) return (ch0 + it) * CH;
+        return (ch0 + (nch > 0 ? it % nch : 0)) * CH;
+    };
     auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
     auto load_small = [&](int it) {
         const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
@@ -1817,7 +1824,7 @@ gemv_cols_mfma2(GemvArgs a)
             __builtin_amdgcn_sched_barrier(0);
         }
         wave_lds_fence();  // the next chunk overwrites the tile
-        if (it % nch == nch - 1) finish_tile(it);
+        if (kOneTile ? it == items - 1 : it % nch == nch - 1) finish_tile(it);
     }
 }
 
