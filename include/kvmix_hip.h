@@ -250,7 +250,7 @@ int kvmix_decode_attention(const kvmix_decode_attn_t *step, void *workspace, siz
  * result differs from kvmix_decode_attention's by up to about 2^-10 of the largest value magnitude.
  *
  * Supported (kvmix_decode_attention_fused_supported returns 1, else the call returns
- * KVMIX_ERR_UNSUPPORTED): D = 128; keys 1/2/4-bit in groups of 32 or the reference's 3-bit words;
+ * KVMIX_ERR_UNSUPPORTED): D = 128; keys 1/2/4-bit or dense 3-bit in groups of 32 or the reference's 3-bit words;
  * values 1/2/4-bit or dense 3-bit in groups of 32; 1, 2, 4 or 8 query heads per kv head.
  * workspace: at least kvmix_decode_attention_fused_workspace_bytes() bytes of device scratch.
  */

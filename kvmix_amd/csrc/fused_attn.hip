@@ -14,8 +14,8 @@
 // once.  The result therefore differs from the four-launch step of decode_attn.hip by up to about
 // 2^-10 of the largest value magnitude.
 //
-// Layout handled: D = 128; keys with 1/2/4 bits in groups of 32 tokens or the reference's 3-bit
-// words (11 codes, own scale and zero); values with 1/2/4 bits or dense 3 bits in groups of 32
+// Layout handled: D = 128; keys with 1/2/4 bits or dense 3 bits in groups of 32 tokens or the
+// reference's 3-bit words (11 codes, own scale and zero); values with 1/2/4 bits or dense 3 bits in groups of 32
 // head dimensions; up to eight query heads per kv head (one block each; they share the slab through L2).
 #include "kvmix_common.h"
 
@@ -37,7 +37,7 @@ struct FusedArgs {
     int64_t q_bs, kc_bs, kc_rs, ksz_bs, ksz_rs, vc_bs, vc_rs, vsz_bs, vsz_rs;
     int64_t kt_bs, kt_ts, vt_bs, vt_ts, mask_bs;
     int64_t k_tokens, v_tokens, k_slots, v_slots, k_len, v_len;
-    int k_mode, v_mode;       // 1, 2, 4 = bits; 3 = the reference's 3-bit words (keys) / dense 3-bit (values)
+    int k_mode, v_mode;       // 1, 2, 4 = bits; 3 = the reference's 3-bit words (keys) / dense 3-bit (values); 30 = dense 3-bit keys
     int slab;                 // positions per block
     int slabs;
     int heads_per_kv, heads;
@@ -144,6 +144,31 @@ __device__ __forceinline__ int fold_lanes(float *v, int lane, int &left)
     }
 }
 
+// 32 codes of one quantization group of a value row -> acc[i] += m * code i (pattern-scaled)
+template <int MODE>
+__device__ __forceinline__ void fma_value_group(const Words<(MODE == 3 ? 3 : MODE)> &g, float m, float *acc)
+{
+    if (MODE == 3) {
+        // dense 3-bit: 32 codes in three consecutive words; four runs of 24 bits hold eight codes each
+        const uint32_t r[4] = {g.v[0] & 0xffffffu, ((g.v[0] >> 24) | (g.v[1] << 8)) & 0xffffffu,
+                               ((g.v[1] >> 16) | (g.v[2] << 16)) & 0xffffffu, g.v[2] >> 8};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[8 * k + i] = fmaf(m, __uint_as_float(r[k] & (7u << (3 * i))), acc[8 * k + i]);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < MODE; j++) fma_fields<MODE>(g.v[j], m, &acc[j * (32 / MODE)]);
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ constexpr float value_unscale(int i)
+{
+    return MODE == 3 ? field_unscale(3 * (i % 8)) : field_unscale(field_offset(MODE, i % (32 / MODE)));
+}
+
 // Logits of the slab's quantized positions.  kKeyLanes lanes share a key row (one head dimension):
 // a lane owns 32 consecutive positions = one quantization group (16 / 8 / 4 bytes of codes, one
 // scale, one zero), or four of the reference's 3-bit words; a block covers 32 head dimensions per
@@ -152,7 +177,7 @@ __device__ __forceinline__ int fold_lanes(float *v, int lane, int &left)
 template <int MODE, int NREP>
 __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv, int64_t t0, const float *qs, float *red)
 {
-    constexpr int WORDS = MODE == 3 ? 4 : MODE;
+    constexpr int WORDS = MODE == 3 ? 4 : (MODE == 30 ? 3 : MODE);  // (30: dense 3-bit, three words per group of 32)
     constexpr int LPP = MODE == 3 ? 44 : 32;
     constexpr int UNIT = MODE == 3 ? 11 : 32;          // positions per (scale, zero)
     constexpr int NSZ = MODE == 3 ? 4 : 1;
@@ -172,7 +197,7 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
         for (int i = 0; i < LPP; i++) acc[h][i] = 0.f;
     }
     if (units > 0) {
-        const int64_t word0 = MODE == 3 ? first / 11 : first * MODE / 32;
+        const int64_t word0 = MODE == 3 ? first / 11 : (MODE == 30 ? first / 32 * 3 : first * MODE / 32);
         const uint32_t *codes = a.k_code + kv * a.kc_bs + word0;
         const int64_t sz0 = kv * a.ksz_bs + first / UNIT;
 #pragma unroll
@@ -216,8 +241,12 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
                 } else {
                     const float m = x * h16_to_f32(sc[0]) * kPatternUp;
                     zacc[h][0] = fmaf(x, h16_to_f32(zr[0]), zacc[h][0]);
+                    if constexpr (MODE == 30) {
+                        fma_value_group<3>(w, m, acc[h]);
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < WORDS; j++) fma_fields<MODE>(w.v[j], m, &acc[h][j * (32 / MODE)]);
+                        for (int j = 0; j < WORDS; j++) fma_fields<MODE>(w.v[j], m, &acc[h][j * (32 / MODE)]);
+                    }
                 }
             }
         }
@@ -228,6 +257,7 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
 #pragma unroll
         for (int i = 0; i < LPP; i++) {
             if (MODE == 3) acc[h][i] = fmaf(acc[h][i], ref3_unscale(i % 11), zacc[h][i / 11]);
+            else if (MODE == 30) acc[h][i] = fmaf(acc[h][i], value_unscale<3>(i), zacc[h][0]);
             else acc[h][i] = fmaf(acc[h][i], field_unscale(field_offset(MODE, i % (32 / MODE))), zacc[h][0]);
         }
         int left;
@@ -237,31 +267,6 @@ __device__ __forceinline__ void slab_key_partials(const FusedArgs &a, int64_t kv
             if (i < left) red[(wave * NREP + h) * kRedStride + sub * (LPP + 1) + at + i] = acc[h][i];
         }
     }
-}
-
-// 32 codes of one quantization group of a value row -> acc[i] += m * code i (pattern-scaled)
-template <int MODE>
-__device__ __forceinline__ void fma_value_group(const Words<(MODE == 3 ? 3 : MODE)> &g, float m, float *acc)
-{
-    if (MODE == 3) {
-        // dense 3-bit: 32 codes in three consecutive words; four runs of 24 bits hold eight codes each
-        const uint32_t r[4] = {g.v[0] & 0xffffffu, ((g.v[0] >> 24) | (g.v[1] << 8)) & 0xffffffu,
-                               ((g.v[1] >> 16) | (g.v[2] << 16)) & 0xffffffu, g.v[2] >> 8};
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) acc[8 * k + i] = fmaf(m, __uint_as_float(r[k] & (7u << (3 * i))), acc[8 * k + i]);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < MODE; j++) fma_fields<MODE>(g.v[j], m, &acc[j * (32 / MODE)]);
-    }
-}
-
-template <int MODE>
-__device__ __forceinline__ constexpr float value_unscale(int i)
-{
-    return MODE == 3 ? field_unscale(3 * (i % 8)) : field_unscale(field_offset(MODE, i % (32 / MODE)));
 }
 
 // acc[h][i] += sum over the slab's quantized value tokens of p[h][t] * value[t][32 * grp + i]:
@@ -364,6 +369,7 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
         case 4: slab_key_partials<4, NREP>(a, kv, t0, qs, red); break;
         case 2: slab_key_partials<2, NREP>(a, kv, t0, qs, red); break;
         case 1: slab_key_partials<1, NREP>(a, kv, t0, qs, red); break;
+        case 30: slab_key_partials<30, NREP>(a, kv, t0, qs, red); break;
         default: slab_key_partials<3, NREP>(a, kv, t0, qs, red); break;
         }
         __syncthreads();
@@ -544,6 +550,7 @@ using namespace kvmix;
 static int fused_key_mode(const kvmix_decode_attn_t *p)
 {
     if (p->k_tokens == 0) return 4;  // no quantized keys: any mode, nothing is read
+    if (p->k_fmt == KVMIX_FMT_DENSE3) return p->k_bits == 3 && p->k_group == 32 ? 30 : 0;
     if (p->k_fmt != KVMIX_FMT_REF) return 0;
     if (p->k_bits == 3) return p->k_group == 11 ? 3 : 0;
     return (p->k_bits == 1 || p->k_bits == 2 || p->k_bits == 4) && p->k_group == 32 ? p->k_bits : 0;
@@ -563,7 +570,7 @@ static int64_t fused_width(const kvmix_decode_attn_t *p)
     return a > b ? a : b;
 }
 
-static int fused_slab(const kvmix_decode_attn_t *p) { return p->k_tokens > 0 && p->k_bits == 3 ? kSlabRef3 : kSlabG32; }
+static int fused_slab(const kvmix_decode_attn_t *p) { return p->k_tokens > 0 && fused_key_mode(p) == 3 ? kSlabRef3 : kSlabG32; }
 
 static int64_t fused_slabs(const kvmix_decode_attn_t *p)
 {
@@ -610,7 +617,7 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
         if (!p->k_code || !p->k_scale || !p->k_zero) return KVMIX_ERR_NULL;
         const int64_t unit = k_mode == 3 ? 11 : 32;
         if (p->k_tokens % unit != 0) return KVMIX_ERR_SHAPE;
-        const int64_t words = k_mode == 3 ? p->k_tokens / 11 : p->k_tokens * k_mode / 32;
+        const int64_t words = k_mode == 3 ? p->k_tokens / 11 : p->k_tokens * (k_mode == 30 ? 3 : k_mode) / 32;
         if (p->k_code_row_stride < words || p->k_sz_row_stride < p->k_tokens / unit) return KVMIX_ERR_SHAPE;
     }
     if (p->v_tokens > 0) {

@@ -455,8 +455,8 @@ def decode_attention(q: torch.Tensor, k_packed, v_packed, k_tail: torch.Tensor, 
     if single_pass:
         st.out, st.out_stride = out.data_ptr(), D
         if not L.kvmix_decode_attention_fused_supported(ctypes.byref(st)):
-            raise RuntimeError("the single-pass attention step does not take this layout (head_dim 128, keys 1/2/4-bit "
-                               "group 32 or reference 3-bit, values 1/2/4-bit or dense 3-bit group 32)")
+            raise RuntimeError("the single-pass attention step does not take this layout (head_dim 128, keys 1/2/4-bit or "
+                               "dense 3-bit group 32 or reference 3-bit, values 1/2/4-bit or dense 3-bit group 32)")
         ws_bytes = L.kvmix_decode_attention_fused_workspace_bytes(ctypes.byref(st))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         with torch.cuda.device(q.device):

@@ -136,7 +136,8 @@ def test_single_pass_attention_host_validation_needs_no_gpu(lib):
     assert sup(desc(D=64)) == 0
     assert sup(desc(heads_per_kv=3)) == 0
     assert sup(desc(k_tokens=64, k_group=64)) == 0                       # key groups other than 32
-    assert sup(desc(k_tokens=64, k_bits=3, k_group=32, k_fmt=_lib.FMT_DENSE3)) == 0   # dense 3-bit keys
+    assert sup(desc(k_tokens=64, k_bits=3, k_group=32, k_fmt=_lib.FMT_DENSE3)) == 1   # dense 3-bit keys
+    assert sup(desc(k_tokens=64, k_bits=4, k_group=32, k_fmt=_lib.FMT_DENSE3)) == 0
     assert sup(desc(k_tokens=66, k_bits=3, k_group=11)) == 1             # the reference's 3-bit words
     assert sup(desc(v_tokens=32, v_bits=3)) == 0                         # 3-bit values only in the dense format
     assert sup(desc(v_tokens=32, v_bits=3, v_fmt=_lib.FMT_DENSE3)) == 1

@@ -132,9 +132,28 @@ def test_single_pass_refuses_what_it_does_not_take(dev):
 
     assert not ops.single_pass_supported(64, 1, 4, ops.FMT_REF, 32, 4, ops.FMT_REF, 32)
     assert not ops.single_pass_supported(128, 3, 4, ops.FMT_REF, 32, 4, ops.FMT_REF, 32)
-    assert not ops.single_pass_supported(128, 1, 3, ops.FMT_DENSE3, 32, 4, ops.FMT_REF, 32)
+    assert ops.single_pass_supported(128, 1, 3, ops.FMT_DENSE3, 32, 4, ops.FMT_REF, 32)
+    assert not ops.single_pass_supported(128, 1, 3, ops.FMT_REF, 32, 4, ops.FMT_REF, 32)   # reference 3-bit words come in groups of 11
     assert not ops.single_pass_supported(128, 1, 4, ops.FMT_REF, 64, 4, ops.FMT_REF, 32)
     q = torch.zeros(1, 2, 1, 64, dtype=torch.float16, device=dev)
     tail = torch.zeros(1, 2, 5, 64, dtype=torch.float16, device=dev)
     with pytest.raises(RuntimeError, match="single-pass"):
         ops.decode_attention(q, None, None, tail, tail, 32, 4, 32, 4, single_pass=True)
+
+
+def test_single_pass_with_dense_three_bit_keys(dev):
+    """Dense 3-bit keys (32 codes in three words, group 32): the single pass against the four-launch step."""
+    from kvmix_amd import ops
+
+    gen = torch.Generator(device=dev).manual_seed(12)
+    for (B, nkv, rep, tk, tv, n, v_bits) in [(2, 2, 2, 1504, 1472, 1600, 3), (1, 4, 1, 512, 0, 530, 4), (3, 1, 4, 96, 128, 140, 2)]:
+        D = 128
+        i32 = lambda *shape: torch.randint(-2 ** 31, 2 ** 31 - 1, shape, dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
+        f16 = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=gen) * scale).half()
+        kq = (i32(B, nkv, D, tk * 3 // 32), f16(B, nkv, D, tk // 32, scale=0.05).abs(), f16(B, nkv, D, tk // 32, scale=0.3))
+        vq = (i32(B, nkv, tv, D * v_bits // 32), f16(B, nkv, tv, D // 32, scale=0.2).abs(), f16(B, nkv, tv, D // 32)) if tv else None
+        k_tail, v_tail, q = f16(B, nkv, n - tk, D), f16(B, nkv, n - tv, D), f16(B, nkv * rep, 1, D)
+        fmt = dict(k_fmt=ops.FMT_DENSE3, v_fmt=ops.FMT_DENSE3 if v_bits == 3 else ops.FMT_REF)
+        out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, 32, 3, 32, v_bits, **fmt)
+        out_s, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, 32, 3, 32, v_bits, single_pass=True, **fmt)
+        check(out_s, out_f, v_magnitude(vq, v_tail, v_bits))
