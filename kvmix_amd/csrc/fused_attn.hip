@@ -15,8 +15,9 @@
 // 2^-10 of the largest value magnitude.
 //
 // Layout handled: D = 128; keys with 1/2/4 bits or dense 3 bits in groups of 32 tokens or the
-// reference's 3-bit words (11 codes, own scale and zero); values with 1/2/4 bits or dense 3 bits in groups of 32
-// head dimensions; up to eight query heads per kv head (one block each; they share the slab through L2).
+// reference's 3-bit words (11 codes, own scale and zero); values with 1/2/4 bits or dense 3 bits in
+// groups of 32 head dimensions; up to eight query heads per kv head (one block each; they share the
+// slab through L2).
 #include "kvmix_common.h"
 
 namespace kvmix {
