@@ -6,8 +6,9 @@
  * kernels on `stream` and returns without synchronising.  Return value 0 is
  * success; negative values are the KVMIX_ERR_* codes below (kvmix_strerror()
  * gives the text, which for argument errors is the reference's TORCH_CHECK text).
- * The library keeps no global mutable state: calls on different streams or from
- * different threads are independent.
+ * Calls on different streams or from different threads are independent: the library's
+ * only process-wide state is set up once per device under a lock or an atomic flag (a
+ * kernel attribute) and never changes afterwards.
  *
  * Packed formats (`fmt`):
  *   KVMIX_FMT_REF    the reference's layout.  bits 1/2/4: 32/bits codes per

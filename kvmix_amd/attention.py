@@ -212,6 +212,16 @@ class KVmixAttention:
                         raise ValueError(f"Attention mask shape {attention_mask.shape} does not match weights shape "
                                          f"{(B, nh, q_len, kv_seq_len)}")
                     mask16 = attention_mask.clamp(min=torch.finfo(torch.float16).min).to(torch.float16)
+                    # A query row whose every position is masked (a left-padding position): the reference adds
+                    # the mask to its fp16 logits in the promoted dtype of the two and clamps
+                    # (models/modeling_llama_KVmix.py:259-262).  With a half mask every entry of such a row ends
+                    # at the lowest finite half, with a float mask of the lowest finite float the logit is
+                    # absorbed: the softmax is uniform either way.  The fused routine adds in fp32 and would
+                    # keep the logits' differences; a zero query makes them equal.  (A float mask holding
+                    # -65504 keeps the differences in the reference too and is left alone.)
+                    absorbed = torch.finfo(torch.float16).min if attention_mask.dtype == torch.float16 else -1e30
+                    dead = attention_mask.amax(dim=-1, keepdim=True) <= absorbed
+                    query_states = query_states.masked_fill(dead, 0)
                 attn_output = F.scaled_dot_product_attention(query_states, key_states, value_states, attn_mask=mask16,
                                                              enable_gqa=n_rep > 1)
                 cache = inplace if (use_cache and inplace is not None) else (

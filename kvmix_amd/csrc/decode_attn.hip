@@ -80,7 +80,9 @@ __global__ void __launch_bounds__(THREADS) attn_tail_softmax(AttnArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int tid = threadIdx.x;
     uint16_t *row = a.probs + sample * a.p_bs;
-    const int64_t k_len = a.k_len_dev ? *a.k_len_dev : a.k_len;
+    // (a device-side counter that ran past the window is cut to it: nothing is read out of bounds)
+    int64_t k_len = a.k_len_dev ? *a.k_len_dev : a.k_len;
+    k_len = k_len < 0 ? 0 : (k_len > a.k_slots ? a.k_slots : k_len);
     const int D = a.D;
 
     // 1. logits of the tail window: row[k_tokens + j] = fp16(q . k_tail[j]) or -inf past the live tokens
@@ -192,7 +194,8 @@ __global__ void __launch_bounds__(THREADS) attn_tail_output(AttnArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int tid = threadIdx.x;
     const int sub = tid % 16, grp = tid / 16;
-    const int64_t v_len = a.v_len_dev ? *a.v_len_dev : a.v_len;
+    int64_t v_len = a.v_len_dev ? *a.v_len_dev : a.v_len;
+    v_len = v_len < 0 ? 0 : (v_len > a.v_slots ? a.v_slots : v_len);
     const uint16_t *prow = a.probs + sample * a.p_bs + a.v_tokens;
     const uint16_t *vt = a.v_tail + kv * a.vt_bs;
     uint16_t *op = a.out + sample * a.o_bs;

@@ -37,6 +37,9 @@
 
 #include "kvmix_common.h"
 
+#include <atomic>
+#include <mutex>
+
 #ifndef KVMIX_COLS3_HEADS_U
 #define KVMIX_COLS3_HEADS_U 4
 #endif
@@ -89,6 +92,8 @@
 #endif
 
 namespace kvmix {
+
+constexpr int kMaxDevices = 64;  // per-device set-up state is kept for device ordinals below this
 
 struct GemvArgs {
     const __half *x;
@@ -2008,12 +2013,14 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
         constexpr int DEPTH = 1;  // chunks in flight per wave (deeper costs occupancy and was slower)
         if (lds > 64 * 1024) {
             // above the default per-block limit: raise it for this kernel, once per device
-            static bool raised[64] = {};
+            // (the attribute is idempotent: two threads that both find the flag clear set it twice)
+            static std::atomic<bool> raised[kMaxDevices];
             int dev = 0;
-            if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !raised[dev]) {
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices ||
+                !raised[dev].load(std::memory_order_acquire)) {
                 (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_rows_mfma<MODE, NREP, DEPTH>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-                raised[dev] = true;
+                if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
             }
         }
         hipLaunchKernelGGL((gemv_rows_mfma<MODE, NREP, DEPTH>), grid, block, lds, st, a);

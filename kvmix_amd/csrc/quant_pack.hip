@@ -710,12 +710,13 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
     int rc = check_format(group, bits, fmt, n, &vpw);
     if (rc != KVMIX_OK) return rc;
     const bool ref3 = bits == 3 && fmt == KVMIX_FMT_REF;
-    if (!ref3 && group != 32) return KVMIX_ERR_UNSUPPORTED;
     if (scale_mode != KVMIX_SCALE_RECIPROCAL && scale_mode != KVMIX_SCALE_DIVIDE) return KVMIX_ERR_FORMAT;
     if (outer == 0 || n == 0 || D == 0) {
+        // (before the group check: an empty key half of kvmix_quant_pack_kv_flush may name any group)
         empty = true;
         return KVMIX_OK;
     }
+    if (!ref3 && group != 32) return KVMIX_ERR_UNSUPPORTED;
     if (!k || !code || !scale || !zero) return KVMIX_ERR_NULL;
     const int64_t words = vpw ? n / vpw : n * 3 / 32;
     groups = n / group;

@@ -154,10 +154,16 @@ class _KVmixAttentionForward:
             attention_mask = torch.full((q_len, seen + q_len), torch.finfo(torch.float32).min, dtype=torch.float32,
                                         device=query_states.device).triu_(seen + 1)[None, None]
         if attention_mask is not None:
+            # A prompt's mask stays in the model's dtype, as transformers builds it for the reference: the
+            # prompt branch adds it to fp16 logits in fp16 (models/modeling_llama_KVmix.py:259-262), which is
+            # what makes the rows of left-padding positions uniform.  A single-token step adds it to fp32
+            # logits (:68-75,189-192), and the library's step takes fp32.
+            mask_dtype = query_states.dtype if q_len > 1 else torch.float32
             if attention_mask.dtype == torch.bool:
-                attention_mask = torch.zeros(attention_mask.shape, dtype=torch.float32, device=attention_mask.device
-                                             ).masked_fill_(~attention_mask, torch.finfo(torch.float32).min)
-            attention_mask = attention_mask.to(torch.float32)
+                attention_mask = torch.zeros(attention_mask.shape, dtype=mask_dtype, device=attention_mask.device
+                                             ).masked_fill_(~attention_mask, torch.finfo(mask_dtype).min)
+            elif attention_mask.dtype != mask_dtype:
+                attention_mask = attention_mask.clamp(min=torch.finfo(mask_dtype).min).to(mask_dtype)
         packed = None if past_key_values is None else past_key_values.packed(self.layer_idx)
         attn_output, attn_weights, _ = self.kvmix(query_states, key_states, value_states, packed,
                                                   attention_mask=attention_mask, use_cache=packed is not None,

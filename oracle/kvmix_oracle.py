@@ -436,20 +436,58 @@ def _matmul_f16(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     return np.matmul(a.astype(np.float32), b.astype(np.float32)).astype(np.float16)
 
 
+def attention_prompt(q, k, v, attention_mask=None):
+    """The dense attention of the prompt branch (models/modeling_llama_KVmix.py:253-264):
+    fp16 logits q.K^T / sqrt(D) (a half tensor divided by a Python number stays half), the mask added
+    in the promoted dtype of the two (a half mask: the sum is rounded to half, so a fully masked row
+    ends with every entry at the lowest finite half and its softmax is uniform; a float mask: the sum
+    is float), clamped to that dtype's lowest finite value, softmax in fp32, probabilities rounded to
+    fp16, fp16 product with V.  q [B,nh,T,D], k, v [B,nh_kv,T,D] f16; mask None or [B,1,T,T] f16/f32.
+    Returns (attn_output [B,nh,T,D] f16, probs f16)."""
+    B, nh, T, D = q.shape
+    rep = nh // k.shape[1]
+    w = _matmul_f16(q, repeat_kv(k, rep).transpose(0, 1, 3, 2))
+    w = (w.astype(np.float32) / np.float32(math.sqrt(D))).astype(np.float16)
+    if attention_mask is None:
+        w = w.astype(np.float32)
+    elif attention_mask.dtype == np.float16:
+        with np.errstate(over="ignore"):
+            w = (w.astype(np.float32) + attention_mask.astype(np.float32)).astype(np.float16)
+        w = np.maximum(w, np.finfo(np.float16).min).astype(np.float32)
+    else:
+        w = np.maximum(w.astype(np.float32) + attention_mask.astype(np.float32), np.finfo(np.float32).min)
+    p = _softmax_f32(w).astype(np.float16)
+    return _matmul_f16(p, repeat_kv(v, rep)), p
+
+
 def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_ratio,
-                          group_size=32, attention_mask=None, fixed_window=None):
+                          group_size=32, attention_mask=None, fixed_window=None,
+                          k_dense3=False, v_dense3=False, compute_output=True):
     """One decode step of LlamaAttention_KVmix.forward after RoPE.
 
     q [B,nh,1,D] f16; k_new, v_new [B,nh_kv,1,D] f16; cache = the reference's 9-tuple
     (Kcode, K_tail, Kscale, Kmin, Vcode, V_tail, Vscale, Vmin, kv_seq_len), entries may
     be None.  Returns (attn_output [B,nh,1,D] f16, probs f16, new cache).
     fixed_window=R replaces the ratio rule by: when the tail reaches R tokens, flush
-    floor(R/g)*g of the oldest ones (the benchmark's fixed residual window)."""
+    floor(R/g)*g of the oldest ones (the benchmark's fixed residual window).
+    k_dense3 / v_dense3 (with 3 bits): that side is kept in the dense 3-bit stream -- an
+    extension without reference counterpart -- in groups of group_size; the flow around the
+    quantizer and the product is the reference's.
+    compute_output=False only brings the cache up to date (append + flush) and returns
+    (None, None, new cache): the cache never depends on the attention arithmetic."""
     kc, k_tail, ks, km, vc, v_tail, vs, vm, seen = cache
     B, nh, _, D = q.shape
     n_rep = nh // k_new.shape[1]
-    kg = 11 if k_bits == 3 else group_size
+    k_dense3 = bool(k_dense3) and k_bits == 3
+    v_dense3 = bool(v_dense3) and v_bits == 3
+    kg = 11 if (k_bits == 3 and not k_dense3) else group_size
     vg = group_size
+
+    def quant(chunk, g, bits, dense3):
+        return quantize_pack_dense3(chunk, g) if dense3 else quantize_pack_last_dim(chunk, g, bits)
+
+    def gemm(g, x, c, s, m, bits, dense3):
+        return quantized_gemm_dense3(g, x, c, s, m) if dense3 else quantized_gemm(g, x, c, s, m, bits)
     k_tail = k_new if k_tail is None else np.concatenate([k_tail, k_new], axis=2)
     v_tail = v_new if v_tail is None else np.concatenate([v_tail, v_new], axis=2)
 
@@ -462,7 +500,7 @@ def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_rat
     if nk > 0:
         chunk = np.ascontiguousarray(k_tail[:, :, :nk, :].transpose(0, 1, 3, 2))
         k_tail = k_tail[:, :, nk:, :]
-        c, s, m = quantize_pack_last_dim(chunk, kg, k_bits)
+        c, s, m = quant(chunk, kg, k_bits, k_dense3)
         kc = c if kc is None else np.concatenate([kc, c], axis=3)
         ks = s if ks is None else np.concatenate([ks, s], axis=3)
         km = m if km is None else np.concatenate([km, m], axis=3)
@@ -470,15 +508,16 @@ def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_rat
     if nv > 0:
         chunk = np.ascontiguousarray(v_tail[:, :, :nv, :])
         v_tail = v_tail[:, :, nv:, :]
-        c, s, m = quantize_pack_last_dim(chunk, vg, v_bits)
+        c, s, m = quant(chunk, vg, v_bits, v_dense3)
         vc = c if vc is None else np.concatenate([vc, c], axis=2)
         vs = s if vs is None else np.concatenate([vs, s], axis=2)
         vm = m if vm is None else np.concatenate([vm, m], axis=2)
 
+    if not compute_output:
+        return None, None, (kc, k_tail, ks, km, vc, v_tail, vs, vm, seen + 1)
     att_q = None
     if kc is not None:
-        att_q = quantized_gemm(kg, q, repeat_kv(kc, n_rep), repeat_kv(ks, n_rep),
-                               repeat_kv(km, n_rep), k_bits)
+        att_q = gemm(kg, q, repeat_kv(kc, n_rep), repeat_kv(ks, n_rep), repeat_kv(km, n_rep), k_bits, k_dense3)
     att_f = _matmul_f16(q, repeat_kv(k_tail, n_rep).transpose(0, 1, 3, 2))
     if att_q is not None:
         w = np.concatenate([att_q.astype(np.float32), att_f.astype(np.float32)], axis=-1)
@@ -492,9 +531,8 @@ def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_rat
         out = _matmul_f16(p, repeat_kv(v_tail, n_rep))
     else:
         lv = v_tail.shape[2]
-        out_q = quantized_gemm(vg, np.ascontiguousarray(p[..., : p.shape[-1] - lv]),
-                               repeat_kv(vc, n_rep), repeat_kv(vs, n_rep), repeat_kv(vm, n_rep),
-                               v_bits)
+        out_q = gemm(vg, np.ascontiguousarray(p[..., : p.shape[-1] - lv]),
+                     repeat_kv(vc, n_rep), repeat_kv(vs, n_rep), repeat_kv(vm, n_rep), v_bits, v_dense3)
         out_f = _matmul_f16(p[..., p.shape[-1] - lv:], repeat_kv(v_tail, n_rep))
         out = (out_q.astype(np.float32) + out_f.astype(np.float32)).astype(np.float16)
     return out, p, (kc, k_tail, ks, km, vc, v_tail, vs, vm, seen + 1)

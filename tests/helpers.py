@@ -38,3 +38,48 @@ def gemv_close(got, want, abs_sum):
     tol = GEMV_RTOL * np.abs(want) + GEMV_ABS_TERM * np.asarray(abs_sum, np.float64)
     bad = err > tol
     return not bad.any(), float((err / np.maximum(tol, 1e-30)).max())
+
+
+def unpack_codes_torch(code, bits, dense3=False):
+    """Packed words [..., W] int32 -> integer codes [..., n] on the tensor's device, with torch integer
+    ops only (a checker that shares nothing with the HIP kernels or the C oracle).
+    Reference layouts: bits 1/2/4, 32/bits codes per word, code i at bit i*bits; bits 3, eleven codes per
+    word (ten 3-bit fields, then a 2-bit field at bit 30).  dense3: 32 codes in three words, code i at
+    bits [3i, 3i+3) of the 96-bit little-endian stream."""
+    import torch
+
+    dev = code.device
+    if dense3:
+        w = code.reshape(code.shape[:-1] + (code.shape[-1] // 3, 3)).to(torch.int64) & 0xFFFFFFFF
+        w0, w1, w2 = w[..., 0], w[..., 1], w[..., 2]
+        out = torch.empty(w0.shape + (32,), dtype=torch.int32, device=dev)
+        for i in range(32):
+            lo = 3 * i
+            if lo + 3 <= 32:
+                v = w0 >> lo
+            elif lo < 32:
+                v = (w0 >> lo) | (w1 << (32 - lo))
+            elif lo + 3 <= 64:
+                v = w1 >> (lo - 32)
+            elif lo < 64:
+                v = (w1 >> (lo - 32)) | (w2 << (64 - lo))
+            else:
+                v = w2 >> (lo - 64)
+            out[..., i] = (v & 7).to(torch.int32)
+        return out.reshape(code.shape[:-1] + (code.shape[-1] // 3 * 32,))
+    if bits == 3:
+        shifts = torch.tensor([3 * i for i in range(10)] + [30], device=dev, dtype=torch.int32)
+        masks = torch.tensor([7] * 10 + [3], device=dev, dtype=torch.int32)
+    else:
+        shifts = torch.arange(0, 32, bits, device=dev, dtype=torch.int32)
+        masks = torch.full((32 // bits,), (1 << bits) - 1, device=dev, dtype=torch.int32)
+    q = (code.unsqueeze(-1) >> shifts) & masks
+    return q.reshape(code.shape[:-1] + (code.shape[-1] * shifts.numel(),))
+
+
+def dequantize_torch(code, scale, zero, bits, group, dense3=False):
+    """fp32 dequantized tensor [..., n] = scale * code + zero (scale, zero per group along the last dimension)."""
+    import torch
+
+    q = unpack_codes_torch(code, bits, dense3).to(torch.float32)
+    return scale.float().repeat_interleave(group, -1) * q + zero.float().repeat_interleave(group, -1)

@@ -88,6 +88,34 @@ def test_prompt_then_decode(oracle, dev):
         np.testing.assert_allclose(out_g.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
 
 
+def test_prompt_left_padding_rows_are_uniform_in_both_prompt_forms(dev):
+    """A left-padded prompt: the pad query positions see nothing but masked keys.  The reference's fp16
+    logits of such a row all end at the lowest finite value (mask added, then clamped;
+    models/modeling_llama_KVmix.py:259-262), so the row's output is the plain mean of V over all
+    positions.  Both prompt forms (probabilities asked for or not) must give that, and must agree
+    on the other rows."""
+    from kvmix_amd.attention import KVmixAttention
+
+    rng = np.random.default_rng(11)
+    B, nh, nkv, D, T, pad = 2, 4, 2, 128, 96, 17
+    att = KVmixAttention(4, 2, group_size=32)
+    K = to_t(kv_like(rng, (B, nkv, T, D)), dev)
+    V = to_t(kv_like(rng, (B, nkv, T, D)), dev)
+    Q = to_t((4 * rng.standard_normal((B, nh, T, D))).astype(np.float16), dev)
+    low = np.finfo(np.float32).min
+    mask = np.triu(np.full((T, T), low, np.float32), 1)[None, None].repeat(B, 0)
+    mask[1, :, :, :pad] = low  # sequence 1 is left-padded: its first `pad` keys are masked for every query
+    mask = to_t(mask, dev)
+    out_w, p, _ = att(Q, K, V, None, attention_mask=mask, use_cache=False, need_weights=True)
+    out_f, none, _ = att(Q, K, V, None, attention_mask=mask, use_cache=False, need_weights=False)
+    assert none is None and p is not None
+    mean_v = V[1].float().mean(dim=1).repeat_interleave(nh // nkv, dim=0)  # [nh, D]
+    for out in (out_w, out_f):
+        got = out[1, :, :pad].float()
+        assert torch.allclose(got, mean_v[:, None, :].expand_as(got), rtol=2e-2, atol=2e-2)
+    assert torch.allclose(out_w.float(), out_f.float(), rtol=2e-2, atol=3e-2)
+
+
 def test_mask_shape_error(dev):
     from kvmix_amd.attention import KVmixAttention
 

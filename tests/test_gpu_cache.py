@@ -48,6 +48,64 @@ def test_inplace_decode_follows_the_oracle(oracle, dev, k_bits, v_bits, nkv, win
     assert cache_o[0] is not None and cache_o[4] is not None
 
 
+@pytest.mark.parametrize("k_bits,v_bits,g", [(4, 2, 64), (2, 4, 128), (3, 1, 64)])
+def test_inplace_decode_with_other_group_sizes(oracle, dev, k_bits, v_bits, g):
+    """config.group_size other than 32 (the reference takes any): the flushes go through the generic
+    quantizer, also in the steps where both tails flush at once, and the products through the
+    generic kernel; cache bit for bit, outputs within tolerance, 300 steps."""
+    from kvmix_amd.attention import KVmixAttention
+
+    rng = np.random.default_rng(g + k_bits)
+    B, nh, nkv, D, window = 2, 4, 2, 128, 2 * g
+    att = KVmixAttention(k_bits, v_bits, group_size=g, residual_length=window)
+    cache_o = (None,) * 8 + (0,)
+    cache_i = att.new_cache(capacity=256)
+    both = 0
+    for step in range(300):
+        k = kv_like(rng, (B, nkv, 1, D))
+        v = kv_like(rng, (B, nkv, 1, D))
+        q = rng.standard_normal((B, nh, 1, D)).astype(np.float16)
+        before = (cache_o[0], cache_o[4])
+        out_o, p_o, cache_o = oracle.attention_decode_step(q, k, v, cache_o, k_bits, v_bits, 0.0, 0.0, group_size=g,
+                                                           fixed_window=window)
+        both += (cache_o[0] is not before[0]) and (cache_o[4] is not before[1])
+        if step == 0:
+            cache_i.append(to_t(k, dev), to_t(v, dev))
+            continue
+        out_i, p_i, _ = att(to_t(q, dev), to_t(k, dev), to_t(v, dev), cache_i)
+        same_cache(cache_i.as_tuple(), cache_o)
+        np.testing.assert_allclose(out_i.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
+    assert both >= 1 or k_bits == 3  # (group-11 keys and group-64 values rarely flush in the same step)
+
+
+@pytest.mark.parametrize("k_dense3,nkv", [(False, 4), (True, 2)])
+def test_inplace_dense3_values_follow_the_oracle_glue(oracle, dev, k_dense3, nkv):
+    """3-bit values in the dense stream (and 3-bit keys in either format) against the oracle's decode
+    step carrying the same formats: cache bit for bit and outputs, 150 steps with a 64-token window."""
+    from kvmix_amd import ops
+    from kvmix_amd.attention import KVmixAttention
+
+    rng = np.random.default_rng(31 + nkv)
+    B, nh, D, g, window = 2, 4, 128, 32, 64
+    att = KVmixAttention(3, 3, group_size=g, residual_length=window)
+    cache_i = att.new_cache(capacity=64, k_fmt=ops.FMT_DENSE3 if k_dense3 else ops.FMT_REF, v_fmt=ops.FMT_DENSE3)
+    cache_o = (None,) * 8 + (0,)
+    for step in range(150):
+        k = kv_like(rng, (B, nkv, 1, D))
+        v = kv_like(rng, (B, nkv, 1, D))
+        q = rng.standard_normal((B, nh, 1, D)).astype(np.float16)
+        out_o, p_o, cache_o = oracle.attention_decode_step(q, k, v, cache_o, 3, 3, 0.0, 0.0, group_size=g,
+                                                           fixed_window=window, k_dense3=k_dense3, v_dense3=True)
+        if step == 0:
+            cache_i.append(to_t(k, dev), to_t(v, dev))
+            continue
+        out_i, p_i, _ = att(to_t(q, dev), to_t(k, dev), to_t(v, dev), cache_i)
+        same_cache(cache_i.as_tuple(), cache_o)
+        np.testing.assert_allclose(p_i.cpu().numpy().astype(np.float64), p_o.astype(np.float64), rtol=5e-3, atol=2e-5)
+        np.testing.assert_allclose(out_i.cpu().numpy().astype(np.float64), out_o.astype(np.float64), rtol=5e-3, atol=5e-3)
+    assert cache_o[0] is not None and cache_o[4] is not None
+
+
 def test_inplace_prompt_then_decode(oracle, dev):
     """Prompt through an empty in-place cache, then decode steps whose first flush covers several
     groups; tail buffers wrap and compact on the way."""

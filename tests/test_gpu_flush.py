@@ -59,3 +59,66 @@ def test_fused_flush_empty_half():
     vc2, vs2, vm2 = ops.quantize_pack_last_dim_cuda(v, 32, 4)
     assert kc.shape == (1, 2, 64, 0)
     assert torch.equal(vc, vc2) and torch.equal(vs, vs2) and torch.equal(vm, vm2)
+
+
+def test_flush_at_config1_size_against_the_oracle():
+    """One flush of BASELINE configs[1] at full size (batch 8, 32 heads, head_dim 128, 128-token window):
+    121 key tokens into the reference's 3-bit words with 128 value tokens into the dense 3-bit stream,
+    and 128 / 128 tokens at 4 and 2 bits, written in place at an offset of larger cache buffers;
+    codes, scales and zeros bit for bit against the oracle, nothing else in the buffers touched."""
+    from kvmix_amd import ops
+    from oracle import kvmix_oracle as O
+
+    B, H, D, cap = 8, 32, 128, 8192
+    rng = np.random.default_rng(17)
+    for k_bits, v_bits, nk in ((3, 3, 121), (4, 2, 128), (2, 4, 128)):
+        k_group = 11 if k_bits == 3 else 32
+        v_fmt = ops.FMT_DENSE3 if v_bits == 3 else ops.FMT_REF
+        k_np = kv_like(rng, (B, H, nk, D), outlier_axis=3)
+        v_np = kv_like(rng, (B, H, 128, D), outlier_axis=3)
+        kvpw = 11 if k_bits == 3 else 32 // k_bits
+        vwords = D * 3 // 32 if v_bits == 3 else D * v_bits // 32
+        k0 = 7936 if k_bits != 3 else 7942          # tokens already in the cache (whole groups)
+        kc = torch.full((B, H, D, cap // kvpw), -1, dtype=torch.int32, device="cuda")
+        ks = torch.full((B, H, D, cap // k_group), 7.0, dtype=torch.float16, device="cuda")
+        km = torch.full_like(ks, 7.0)
+        vc = torch.full((B, H, cap, vwords), -1, dtype=torch.int32, device="cuda")
+        vs = torch.full((B, H, cap, D // 32), 7.0, dtype=torch.float16, device="cuda")
+        vm = torch.full_like(vs, 7.0)
+        w0, g0, v0 = k0 // kvpw, k0 // k_group, 7936
+        k_out = (kc[..., w0:w0 + nk // kvpw], ks[..., g0:g0 + nk // k_group], km[..., g0:g0 + nk // k_group])
+        v_out = (vc[:, :, v0:v0 + 128], vs[:, :, v0:v0 + 128], vm[:, :, v0:v0 + 128])
+        ops.quantize_kv_flush_into(torch.from_numpy(k_np).cuda(), k_group, k_bits, k_out, torch.from_numpy(v_np).cuda(), 32,
+                                   v_bits, v_out, ops.FMT_REF, v_fmt)
+        torch.cuda.synchronize()
+        oc, osc, omn = O.quantize_pack_last_dim(np.ascontiguousarray(k_np.transpose(0, 1, 3, 2)), k_group, k_bits)
+        if v_bits == 3:
+            ovc, ovs, ovm = O.quantize_pack_dense3(v_np, 32)
+        else:
+            ovc, ovs, ovm = O.quantize_pack_last_dim(v_np, 32, v_bits)
+        for got, want in zip(k_out + v_out, (oc, osc, omn, ovc, ovs, ovm)):
+            assert same_bits(got.cpu().numpy(), want), (k_bits, v_bits)
+        # the rest of the buffers still holds the fill pattern
+        for buf, lo, hi, axis, fill in ((kc, w0, w0 + nk // kvpw, 3, -1), (ks, g0, g0 + nk // k_group, 3, 7.0),
+                                        (km, g0, g0 + nk // k_group, 3, 7.0), (vc, v0, v0 + 128, 2, -1),
+                                        (vs, v0, v0 + 128, 2, 7.0), (vm, v0, v0 + 128, 2, 7.0)):
+            before, after = buf.narrow(axis, 0, lo), buf.narrow(axis, hi, buf.shape[axis] - hi)
+            assert bool((before == fill).all()) and bool((after == fill).all())
+
+
+def test_flush_with_group_64_keys_when_both_tails_flush(dev=None):
+    """A group size other than 32 (the reference allows any): the key half goes through the generic
+    quantizer, the value half through the flush entry point with an empty key half -- which must not
+    be refused for the key group it names."""
+    from kvmix_amd import ops
+    from oracle import kvmix_oracle as O
+
+    rng = np.random.default_rng(23)
+    B, H, D, n = 2, 3, 128, 128
+    k_np = kv_like(rng, (B, H, n, D), outlier_axis=3)
+    v_np = kv_like(rng, (B, H, n, D), outlier_axis=3)
+    kc, ks, km, vc, vs, vm = ops.quantize_kv_flush(torch.from_numpy(k_np).cuda(), 64, 4, torch.from_numpy(v_np).cuda(), 64, 2)
+    oc, osc, omn = O.quantize_pack_last_dim(np.ascontiguousarray(k_np.transpose(0, 1, 3, 2)), 64, 4)
+    ovc, ovs, ovm = O.quantize_pack_last_dim(v_np, 64, 2)
+    for got, want in zip((kc, ks, km, vc, vs, vm), (oc, osc, omn, ovc, ovs, ovm)):
+        assert same_bits(got.cpu().numpy(), want)

@@ -325,6 +325,81 @@ def test_full_size_properties_gqa_32k(dev):
     assert ((out - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
 
 
+def test_full_size_properties_config1_b8_t8192(oracle, dev):
+    """BASELINE configs[1]'s two 3-bit legs at full size (batch 8, 32 heads, head_dim 128, 8192 tokens,
+    128-token window): q.K^T over keys in the reference's 3-bit words (8063 = 11 * 733 quantized
+    tokens) and p.V over values in the dense 3-bit stream (8064 tokens; no reference counterpart).
+    Properties that need no CPU run at this size -- exact integer column sums, exact one-hot rows,
+    torch's fp32 matmul of the dequantized operand on a two-batch slice -- and the oracle itself on
+    one (batch, head) pair."""
+    import KVmix
+    from helpers import dequantize_torch, unpack_codes_torch
+    from kvmix_amd import ops
+
+    torch.manual_seed(5)
+    B, H, D = 8, 32, 128
+    Tqk, Tqv = 8063, 8064
+    # keys, reference 3-bit words: all-ones query, scale 1, zero 0 -> column sums of the codes (<= 128 * 7)
+    kcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tqk // 11), dtype=torch.int64, device=dev).to(torch.int32)
+    ones = torch.ones(B, H, D, Tqk // 11, dtype=torch.float16, device=dev)
+    x1 = torch.ones(B, H, 1, D, dtype=torch.float16, device=dev)
+    out = KVmix.quantized_gemm(11, x1, kcode, ones, torch.zeros_like(ones), 3)
+    assert out.shape == (B, H, 1, Tqk)
+    assert torch.equal(out[:, :, 0].to(torch.int32), unpack_codes_torch(kcode, 3).sum(2))
+    # one-hot query: one dequantized channel row, exact after the fp16 rounding
+    ks = (torch.rand(B, H, D, Tqk // 11, device=dev) + 0.5).half()
+    kz = torch.randn(B, H, D, Tqk // 11, device=dev).half()
+    e = torch.zeros(B, H, 1, D, dtype=torch.float16, device=dev)
+    e[..., 101] = 1
+    out = KVmix.quantized_gemm(11, e, kcode, ks, kz, 3)
+    want = dequantize_torch(kcode[:, :, 101], ks[:, :, 101], kz[:, :, 101], 3, 11).half()
+    assert torch.equal(out[:, :, 0], want)
+    # random queries against torch's fp32 matmul on two batch entries, and the oracle on one (batch, head)
+    q = torch.randn(B, H, 1, D, device=dev).half()
+    out = KVmix.quantized_gemm(11, q, kcode, ks, kz, 3)
+    deq = dequantize_torch(kcode[:2], ks[:2], kz[:2], 3, 11)                      # [2, H, D, Tqk]
+    ref = torch.matmul(q[:2].float(), deq)
+    ab = torch.matmul(q[:2].float().abs(), deq.abs())
+    assert ((out[:2].float() - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
+    b, h = 7, 30
+    _, w64, a64 = oracle.quantized_gemm(11, q[b:b + 1, h:h + 1].cpu().numpy(), kcode[b:b + 1, h:h + 1].cpu().numpy(),
+                                        ks[b:b + 1, h:h + 1].cpu().numpy(), kz[b:b + 1, h:h + 1].cpu().numpy(), 3,
+                                        want_f64=True)
+    ok, worst = gemv_close(out[b:b + 1, h:h + 1].cpu().numpy(), w64, a64)
+    assert ok, worst
+    del kcode, ones, ks, kz, deq, ref, ab
+
+    # values, dense 3-bit stream
+    vcode = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tqv, D * 3 // 32), dtype=torch.int64, device=dev).to(torch.int32)
+    vs = (torch.rand(B, H, Tqv, D // 32, device=dev) + 0.5).half()
+    vz = torch.randn(B, H, Tqv, D // 32, device=dev).half()
+    p = torch.zeros(B, H, 1, Tqv, dtype=torch.float16, device=dev)
+    rows = torch.randint(0, Tqv, (H,), device=dev)
+    for hh in range(H):
+        p[:, hh, 0, rows[hh]] = 1
+    out = ops.quantized_gemm(32, p, vcode, vs, vz, 3, fmt=ops.FMT_DENSE3)
+    for hh in range(H):
+        r = int(rows[hh])
+        want = dequantize_torch(vcode[:, hh, r], vs[:, hh, r], vz[:, hh, r], 3, 32, dense3=True).half()
+        assert torch.equal(out[:, hh, 0], want), hh
+    # all-ones probabilities over the first 256 tokens, scale 1, zero 0: exact sums (<= 256 * 7, exact in fp16)
+    one = torch.ones_like(vs[:, :, :256])
+    out = ops.quantized_gemm(32, torch.ones(B, H, 1, 256, dtype=torch.float16, device=dev), vcode[:, :, :256], one,
+                             torch.zeros_like(one), 3, fmt=ops.FMT_DENSE3)
+    assert torch.equal(out[:, :, 0].to(torch.int32), unpack_codes_torch(vcode[:, :, :256], 3, dense3=True).sum(2))
+    pr = torch.softmax(torch.randn(B, H, 1, Tqv, device=dev), -1).half()
+    out = ops.quantized_gemm(32, pr, vcode, vs, vz, 3, fmt=ops.FMT_DENSE3)
+    deq = dequantize_torch(vcode[:2], vs[:2], vz[:2], 3, 32, dense3=True)       # [2, H, Tqv, D]
+    ref = torch.matmul(pr[:2].float(), deq)
+    ab = torch.matmul(pr[:2].float().abs(), deq.abs())
+    assert ((out[:2].float() - ref).abs() <= 1e-3 * ref.abs() + 2e-5 * ab).all()
+    _, w64, a64 = oracle.quantized_gemm_dense3(32, pr[b:b + 1, h:h + 1].cpu().numpy(), vcode[b:b + 1, h:h + 1].cpu().numpy(),
+                                               vs[b:b + 1, h:h + 1].cpu().numpy(), vz[b:b + 1, h:h + 1].cpu().numpy(),
+                                               want_f64=True)
+    ok, worst = gemv_close(out[b:b + 1, h:h + 1].cpu().numpy(), w64, a64)
+    assert ok, worst
+
+
 @pytest.mark.parametrize("bits", [1, 2])
 def test_full_size_properties_batch128_t4096(dev, bits):
     """BASELINE configs[3] at its largest batch: 128 x 32 heads, 4064 quantized tokens, 1/2 bits."""

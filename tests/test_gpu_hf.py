@@ -38,12 +38,8 @@ class RatioOracle(OracleAttention):
         from kvmix_amd.cache import flush_length
 
         o = self.o
-        B, nh, T, D = q.shape
-        rep = nh // k.shape[1]
-        w = o._matmul_f16(q, o.repeat_kv(k, rep).transpose(0, 1, 3, 2)).astype(np.float32) / np.float32(math.sqrt(D))
-        w = np.maximum(w + mask.astype(np.float32), np.finfo(np.float32).min)
-        p = o._softmax_f32(w.astype(np.float32)).astype(np.float16)
-        out = o._matmul_f16(p, o.repeat_kv(v, rep))
+        T = k.shape[2]
+        out, _ = o.attention_prompt(q, k, v, mask)
         kg = 11 if self.k_bits == 3 else self.group
         nk = flush_length(T, self.k_ratio, kg, None, prompt=True)
         nv = flush_length(T, self.v_ratio, self.group, None, prompt=True)
@@ -51,9 +47,9 @@ class RatioOracle(OracleAttention):
         vc, vs, vm = o.quantize_pack_last_dim(np.ascontiguousarray(v[:, :, :nv]), self.group, self.v_bits)
         return out, (kc, k[:, :, nk:], ks, km, vc, v[:, :, nv:], vs, vm, T)
 
-    def step(self, q, k, v, cache):
+    def step(self, q, k, v, cache, compute_output=True):
         return self.o.attention_decode_step(q, k, v, cache, self.k_bits, self.v_bits, self.k_ratio, self.v_ratio,
-                                            group_size=self.group)
+                                            group_size=self.group, v_dense3=self.v_dense3, compute_output=compute_output)
 
 
 class Tap:
@@ -175,7 +171,9 @@ def test_left_padded_batch(oracle, dev, kind, extra):
     for li, tap in enumerate(taps):
         orc, state = RatioOracle(oracle, model.quant_bits[li]), None
         for step, (q, k, v, out_g, m) in enumerate(tap.calls):
-            assert m is not None and m.dtype == np.float32 and m.shape == (B, 1, q.shape[2], T + step)
+            # (the prompt's mask arrives in the model's dtype, a single-token step's in fp32)
+            assert m is not None and m.dtype == (np.float16 if step == 0 else np.float32)
+            assert m.shape == (B, 1, q.shape[2], T + step)
             if state is None:
                 out_o, state = orc.prompt(q, k, v, m)
             else:

@@ -1,5 +1,6 @@
-"""The single-pass attention step (ops.decode_attention(single_pass=True)) against the four-launch
-step, which the other tests tie to the oracle.  The two differ by design in the roundings after
+"""The single-pass attention step (ops.decode_attention(single_pass=True)): every key and value format
+and head grouping against fp64 attention over the cache dequantized with torch integer ops, and
+random layouts against the four-launch step, which the other tests tie to the oracle.  The two differ by design in the roundings after
 the softmax (single pass: fp32 probabilities, one rounding of the output; four launches: the
 reference's fp16 probabilities and fp16 halves), i.e. by about 2^-10 of the largest value
 magnitude; the tolerance below is 2e-3 of that magnitude plus 2e-3 relative."""
@@ -103,28 +104,48 @@ def test_single_pass_with_device_side_lengths(dev):
         assert torch.equal(got, want)
 
 
-def test_single_pass_against_exact_attention(dev):
-    """Against fp64 attention over the dequantized cache, with the one rounding the single-pass step
-    keeps from the reference (logits to fp16 before scaling): a few 1e-3 of the value magnitude."""
+KEY_KINDS = {"k1": (1, False), "k2": (2, False), "k4": (4, False), "kref3": (3, False), "kdense3": (3, True)}
+VALUE_KINDS = {"v1": (1, False), "v2": (2, False), "v4": (4, False), "vdense3": (3, True)}
+
+
+@pytest.mark.parametrize("k_kind", list(KEY_KINDS))
+@pytest.mark.parametrize("v_kind", list(VALUE_KINDS))
+def test_single_pass_against_exact_attention(dev, k_kind, v_kind):
+    """Every key and value format, with 1, 4 and 8 query heads per kv head and a padding mask, against
+    fp64 attention over the cache dequantized with torch integer ops (no kernel of the library), with the
+    one rounding the single-pass step keeps from the reference (logits to fp16 before scaling): a few
+    1e-3 of the value magnitude."""
+    from helpers import unpack_codes_torch
     from kvmix_amd import ops
 
-    gen = torch.Generator(device=dev).manual_seed(10)
-    B, nkv, rep, n, tk, tv = 2, 2, 4, 1700, 1536, 1600
-    q, kq, vq, k_tail, v_tail, kg, _, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, 4, 4, tk, tv, n)
-    out, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, 4, 32, 4, single_pass=True, **fmt)
-
-    def unpack4(code):  # [..., W] int32 -> [..., W*8] codes, low nibble first
-        c = code.to(torch.int64) & 0xffffffff
-        return torch.stack([(c >> (4 * i)) & 15 for i in range(8)], -1).flatten(-2).double()
-
-    K = unpack4(kq[0]) * kq[1].double().repeat_interleave(32, -1) + kq[2].double().repeat_interleave(32, -1)  # [B,nkv,D,tk]
-    V = unpack4(vq[0]) * vq[1].double().repeat_interleave(32, -1) + vq[2].double().repeat_interleave(32, -1)  # [B,nkv,tv,D]
-    K = torch.cat([K.transpose(2, 3), k_tail.double()], 2).repeat_interleave(rep, 1)
-    V = torch.cat([V, v_tail.double()], 2).repeat_interleave(rep, 1)
-    logits = (q.double() @ K.transpose(2, 3)).half().double() / 128 ** 0.5
-    want = torch.softmax(logits, -1) @ V
-    err = float((out.double() - want).abs().max())
-    assert err <= 4e-3 * float(V.abs().max()), err
+    (k_bits, k_dense3), (v_bits, v_dense3) = KEY_KINDS[k_kind], VALUE_KINDS[v_kind]
+    gen = torch.Generator(device=dev).manual_seed(10 + 7 * k_bits + v_bits + k_dense3)
+    D, B, nkv = 128, 2, 2
+    kg = 11 if (k_bits == 3 and not k_dense3) else 32
+    i32 = lambda *shape: torch.randint(-2 ** 31, 2 ** 31 - 1, shape, dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
+    f16 = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=gen) * scale).half()
+    for rep, n, tk, tv in ((1, 1700, (1536 // kg) * kg, 1600), (4, 900, (700 // kg) * kg, 832), (8, 2300, (2200 // kg) * kg, 2176)):
+        kw = tk * 3 // 32 if k_dense3 else (tk // 11 if k_bits == 3 else tk * k_bits // 32)
+        vw = D * 3 // 32 if v_dense3 else D * v_bits // 32
+        kq = (i32(B, nkv, D, kw), f16(B, nkv, D, tk // kg, scale=0.05).abs(), f16(B, nkv, D, tk // kg, scale=0.3))
+        vq = (i32(B, nkv, tv, vw), f16(B, nkv, tv, D // 32, scale=0.2).abs(), f16(B, nkv, tv, D // 32))
+        k_tail, v_tail, q = f16(B, nkv, n - tk, D), f16(B, nkv, n - tv, D), f16(B, nkv * rep, 1, D)
+        mask = torch.zeros(B, 1, 1, n, device=dev)
+        mask[B - 1, :, :, :n // 3] = torch.finfo(torch.float32).min  # the last sequence is left-padded
+        fmt = dict(k_fmt=ops.FMT_DENSE3 if k_dense3 else ops.FMT_REF, v_fmt=ops.FMT_DENSE3 if v_dense3 else ops.FMT_REF)
+        assert ops.single_pass_supported(D, rep, k_bits, fmt["k_fmt"], kg, v_bits, fmt["v_fmt"], 32)
+        out, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask,
+                                      single_pass=True, **fmt)
+        K = unpack_codes_torch(kq[0], k_bits, k_dense3).double() * kq[1].double().repeat_interleave(kg, -1) \
+            + kq[2].double().repeat_interleave(kg, -1)
+        V = unpack_codes_torch(vq[0], v_bits, v_dense3).double() * vq[1].double().repeat_interleave(32, -1) \
+            + vq[2].double().repeat_interleave(32, -1)                                                # [B,nkv,tv,D]
+        K = torch.cat([K.transpose(2, 3), k_tail.double()], 2).repeat_interleave(rep, 1)
+        V = torch.cat([V, v_tail.double()], 2).repeat_interleave(rep, 1)
+        logits = (q.double() @ K.transpose(2, 3)).half().double() / D ** 0.5 + mask.double()
+        want = torch.softmax(logits, -1) @ V
+        err = float((out.double() - want).abs().max())
+        assert err <= 4e-3 * float(V.abs().max()), (k_kind, v_kind, rep, err)
 
 
 def test_single_pass_refuses_what_it_does_not_take(dev):

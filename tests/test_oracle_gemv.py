@@ -207,3 +207,88 @@ def test_flush_rule(oracle):
     assert oracle.flush_length(416, 0.2, 32) == 320
     assert oracle.flush_length(13, 0.2, 11) == 11
     assert oracle.flush_length(5, 0.3, 32) == 0
+
+
+def test_prompt_attention_against_float64_and_fully_masked_rows(oracle):
+    """attention_prompt: causal rows against dense float64 attention; a row whose every position is
+    masked gives the plain mean of V when the mask is half (every fp16 logit ends at the lowest finite
+    half) or holds the lowest finite float (the logit is absorbed), but keeps its logits' differences
+    when a float mask holds -65504 -- the three cases of models/modeling_llama_KVmix.py:259-262."""
+    rng = np.random.default_rng(12)
+    B, nh, nkv, T, D, pad = 2, 4, 2, 40, 64, 9
+    q = rng.standard_normal((B, nh, T, D)).astype(np.float16)
+    k = rng.standard_normal((B, nkv, T, D)).astype(np.float16)
+    v = rng.standard_normal((B, nkv, T, D)).astype(np.float16)
+    rep = nh // nkv
+    mean_v = np.repeat(v.astype(np.float64), rep, 1).mean(2)                       # [B, nh, D]
+    for dtype, low in ((np.float16, np.finfo(np.float16).min), (np.float32, np.finfo(np.float32).min),
+                       (np.float32, np.float32(np.finfo(np.float16).min))):
+        mask = np.triu(np.full((T, T), low, dtype), 1)[None, None].repeat(B, 0)
+        mask[1, :, :, :pad] = low
+        out, p = oracle.attention_prompt(q, k, v, mask)
+        assert out.dtype == np.float16 and p.dtype == np.float16 and p.shape == (B, nh, T, T)
+        # rows with at least one open position: dense float64 attention over the open positions
+        m64 = np.where(mask.astype(np.float64) < -1e4, -np.inf, 0.0)
+        w = np.einsum("bhqd,bhtd->bhqt", q.astype(np.float64), np.repeat(k.astype(np.float64), rep, 1)) / np.sqrt(D) + m64
+        with np.errstate(invalid="ignore"):
+            e = np.exp(w - w.max(-1, keepdims=True))
+            want = np.einsum("bhqt,bhtd->bhqd", e / e.sum(-1, keepdims=True), np.repeat(v.astype(np.float64), rep, 1))
+        live = np.ones((B, T), bool)
+        live[1, :pad] = False
+        np.testing.assert_allclose(out.astype(np.float64)[live.nonzero()[0], :, live.nonzero()[1]],
+                                   want[live.nonzero()[0], :, live.nonzero()[1]], rtol=1e-2, atol=1e-2)
+        dead = out[1, :, :pad].astype(np.float64)
+        uniform = np.allclose(dead, mean_v[1][:, None, :], rtol=1e-2, atol=1e-2)
+        absorbed = dtype == np.float16 or low == np.finfo(np.float32).min
+        assert uniform == absorbed, (dtype, low)
+
+
+@pytest.mark.parametrize("k_dense3,v_dense3", [(True, True), (False, True), (True, False)])
+def test_decode_steps_with_dense3_sides_match_dense_attention(oracle, k_dense3, v_dense3):
+    """The decode step with 3-bit sides kept in the dense stream: the cache holds what one-shot dense
+    3-bit quantization of the flushed tokens gives, and the step equals dense float64 attention over
+    the dequantized cache (the same pin as for the reference's formats)."""
+    rng = np.random.default_rng(13)
+    B, nh, nkv, D, g, window = 1, 4, 2, 128, 32, 64
+    rep = nh // nkv
+    cache = (None,) * 8 + (0,)
+    hist_k, hist_v = [], []
+    for step in range(140):
+        k = kv_like(rng, (B, nkv, 1, D))
+        v = kv_like(rng, (B, nkv, 1, D))
+        q = rng.standard_normal((B, nh, 1, D)).astype(np.float16)
+        hist_k.append(k)
+        hist_v.append(v)
+        out, p, cache = oracle.attention_decode_step(q, k, v, cache, 3, 3 if v_dense3 else 4, 0.0, 0.0, group_size=g,
+                                                     fixed_window=window, k_dense3=k_dense3, v_dense3=v_dense3)
+        kc, k_tail, ks, km, vc, v_tail, vs, vm, seen = cache
+        kg = g if k_dense3 else 11
+        Kd = k_tail.astype(np.float64)
+        if kc is not None:
+            kq = oracle.dequantize_dense3_np(kc, ks, km, g) if k_dense3 else oracle.dequantize_np(kc, ks, km, 3, 11)
+            Kd = np.concatenate([kq.astype(np.float64).transpose(0, 1, 3, 2), Kd], 2)
+        Vd = v_tail.astype(np.float64)
+        if vc is not None:
+            vq = oracle.dequantize_dense3_np(vc, vs, vm, g) if v_dense3 else oracle.dequantize_np(vc, vs, vm, 4, g)
+            Vd = np.concatenate([vq.astype(np.float64), Vd], 2)
+        assert Kd.shape[2] == step + 1 and Vd.shape[2] == step + 1
+        want, pw = dense_attention(q.astype(np.float64), np.repeat(Kd, rep, 1), np.repeat(Vd, rep, 1))
+        np.testing.assert_allclose(p.astype(np.float64), pw, rtol=4e-3, atol=2e-4)
+        np.testing.assert_allclose(out.astype(np.float64), want, rtol=4e-3, atol=4e-3)
+    kc, _, ks, km, vc, _, vs, vm, _ = cache
+    assert kc is not None and vc is not None
+    allk, allv = np.concatenate(hist_k, 2), np.concatenate(hist_v, 2)
+    if k_dense3:
+        c, s, m = oracle.quantize_pack_dense3(np.ascontiguousarray(allk[:, :, :64].transpose(0, 1, 3, 2)), g)
+        assert same_bits(kc[..., : c.shape[-1]], c) and same_bits(ks[..., :2], s) and same_bits(km[..., :2], m)
+    if v_dense3:
+        c, s, m = oracle.quantize_pack_dense3(np.ascontiguousarray(allv[:, :, :64]), g)
+        assert same_bits(vc[:, :, :64], c) and same_bits(vs[:, :, :64], s) and same_bits(vm[:, :, :64], m)
+    # compute_output=False leaves the cache exactly as the full step does
+    a = oracle.attention_decode_step(q, k, v, cache, 3, 3 if v_dense3 else 4, 0.0, 0.0, group_size=g, fixed_window=window,
+                                     k_dense3=k_dense3, v_dense3=v_dense3)[2]
+    b = oracle.attention_decode_step(q, k, v, cache, 3, 3 if v_dense3 else 4, 0.0, 0.0, group_size=g, fixed_window=window,
+                                     k_dense3=k_dense3, v_dense3=v_dense3, compute_output=False)
+    assert b[0] is None and b[1] is None
+    for x, y in zip(a, b[2]):
+        assert (x is None and y is None) or (isinstance(x, int) and x == y) or same_bits(x, y)
