@@ -8,7 +8,8 @@
  * gives the text, which for argument errors is the reference's TORCH_CHECK text).
  * Calls on different streams or from different threads are independent: the library's
  * only process-wide state is set up once per device under a lock or an atomic flag (a
- * kernel attribute) and never changes afterwards.
+ * kernel attribute, the address of kvmix_quantized_gemv_static's buffer) and never
+ * changes afterwards.  The one exception is the content of that buffer, see there.
  *
  * Packed formats (`fmt`):
  *   KVMIX_FMT_REF    the reference's layout.  bits 1/2/4: 32/bits codes per
@@ -43,6 +44,7 @@ extern "C" {
 #define KVMIX_ERR_FORMAT (-10)     /* unknown fmt */
 #define KVMIX_ERR_WORKSPACE (-11)  /* workspace smaller than kvmix_gemv_workspace_bytes() */
 #define KVMIX_ERR_LAUNCH (-12)     /* hipGetLastError() after a launch was not hipSuccess */
+#define KVMIX_ERR_STATIC_SCRATCH (-13) /* kvmix_quantized_gemv_static: problem beyond the built-in buffer */
 
 #define KVMIX_F16 0
 #define KVMIX_F32 1
@@ -175,6 +177,30 @@ int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride, int64
                          int64_t M, int64_t K, int64_t N, void *out, int64_t out_batch_stride,
                          int64_t out_row_stride, void *workspace, size_t workspace_bytes,
                          kvmix_stream_t stream);
+
+/*
+ * kvmix_quantized_gemv for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments minus the workspace, same kernels, same results bit for bit: the split-K partial
+ * sums go to a buffer of KVMIX_GEMV_STATIC_SCRATCH_BYTES that is part of the library's device
+ * image (every device the library runs on holds it until the process ends).  The call allocates
+ * and frees nothing.  A problem whose kvmix_gemv_workspace_bytes() exceeds the buffer is refused
+ * with KVMIX_ERR_STATIC_SCRATCH before anything is launched.  The buffer covers every q.K^T product
+ * and every p.V product with N <= 128 (at most 1.06 MiB of partial sums, reached near 120 output
+ * rows of 128k tokens; launches of 1024 and more output rows need none); with N = 256 a few shapes
+ * around 120 output rows of 64k and more tokens need up to 2.11 MiB and are refused.
+ * All calls on one device share the buffer: two calls that overlap on one device (different
+ * streams, or threads) race on it; calls on one stream are ordered and safe.  Nothing in the
+ * buffer has to start at zero (every partial sum is written before it is read).  The first call
+ * on a device looks the buffer's address up (hipGetSymbolAddress): make it outside a capture.
+ */
+#define KVMIX_GEMV_STATIC_SCRATCH_BYTES (2u << 20)
+int kvmix_quantized_gemv_static(int group, const void *x, int64_t x_batch_stride, int64_t x_row_stride,
+                                const uint32_t *code, int64_t code_batch_stride, int64_t code_row_stride,
+                                const void *scale, const void *zero, int64_t sz_batch_stride,
+                                int64_t sz_row_stride, int bits, int fmt, int64_t samples, int heads_per_kv,
+                                int64_t M, int64_t K, int64_t N, void *out, int64_t out_batch_stride,
+                                int64_t out_row_stride, kvmix_stream_t stream);
 
 /*
  * One decode step of attention over the packed cache and its fp16 residual tails: what

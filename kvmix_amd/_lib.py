@@ -14,6 +14,7 @@ OK = 0
 F16, F32 = 0, 1
 FMT_REF, FMT_DENSE3, FMT_REF3_WRAP = 0, 1, 2
 SCALE_RECIPROCAL, SCALE_DIVIDE = 0, 1
+GEMV_STATIC_SCRATCH_BYTES = 2 << 20  # KVMIX_GEMV_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "kvmix_version",
@@ -23,6 +24,7 @@ EXPORTS = (
     "kvmix_quant_pack_kv_flush",
     "kvmix_gemv_workspace_bytes",
     "kvmix_quantized_gemv",
+    "kvmix_quantized_gemv_static",
     "kvmix_decode_attention_workspace_bytes",
     "kvmix_decode_attention",
     "kvmix_decode_attention_fused_supported",
@@ -116,6 +118,9 @@ def load() -> ctypes.CDLL:
     L.kvmix_quantized_gemv.restype = i32
     L.kvmix_quantized_gemv.argtypes = [i32, vp, i64, i64, vp, i64, i64, vp, vp, i64, i64, i32, i32,
                                        i64, i32, i64, i64, i64, vp, i64, i64, vp, sz, vp]
+    L.kvmix_quantized_gemv_static.restype = i32
+    L.kvmix_quantized_gemv_static.argtypes = [i32, vp, i64, i64, vp, i64, i64, vp, vp, i64, i64, i32, i32,
+                                              i64, i32, i64, i64, i64, vp, i64, i64, vp]
     L.kvmix_decode_attention_workspace_bytes.restype = sz
     L.kvmix_decode_attention_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
     L.kvmix_decode_attention.restype = i32

@@ -2296,6 +2296,40 @@ extern "C" size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t
     return splits > 1 ? (size_t)(samples * M) * (size_t)splits * (size_t)N * sizeof(float) : 0;
 }
 
+// Workspace of kvmix_quantized_gemv_static: the split-K partial sums of the p.V kernels.  Every
+// device the library runs on holds its own copy of this array until the process ends.  In host
+// code the name stands for the symbol, not for device memory: the address on a device comes from
+// hipGetSymbolAddress (static_scratch below) and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[KVMIX_GEMV_STATIC_SCRATCH_BYTES];
+
+// the array's address on the current device, looked up once per device; nullptr on failure
+static void *static_scratch()
+{
+    static std::mutex lock;
+    static void *ptr[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> hold(lock);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    return ptr[dev];
+}
+
+static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
+                          int64_t x_row_stride, const uint32_t *code,
+                          int64_t code_batch_stride, int64_t code_row_stride,
+                          const void *scale, const void *zero, int64_t sz_batch_stride,
+                          int64_t sz_row_stride, int bits, int fmt, int64_t samples,
+                          int heads_per_kv, int64_t M, int64_t K, int64_t N, void *out,
+                          int64_t out_batch_stride, int64_t out_row_stride, void *workspace,
+                          size_t workspace_bytes, bool workspace_is_static, kvmix_stream_t stream);
+
 extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride,
                                     int64_t x_row_stride, const uint32_t *code,
                                     int64_t code_batch_stride, int64_t code_row_stride,
@@ -2304,6 +2338,38 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
                                     int heads_per_kv, int64_t M, int64_t K, int64_t N, void *out,
                                     int64_t out_batch_stride, int64_t out_row_stride, void *workspace,
                                     size_t workspace_bytes, kvmix_stream_t stream)
+{
+    return quantized_gemv(group, x, x_batch_stride, x_row_stride, code, code_batch_stride, code_row_stride, scale,
+                          zero, sz_batch_stride, sz_row_stride, bits, fmt, samples, heads_per_kv, M, K, N, out,
+                          out_batch_stride, out_row_stride, workspace, workspace_bytes, false, stream);
+}
+
+extern "C" int kvmix_quantized_gemv_static(int group, const void *x, int64_t x_batch_stride,
+                                           int64_t x_row_stride, const uint32_t *code,
+                                           int64_t code_batch_stride, int64_t code_row_stride,
+                                           const void *scale, const void *zero, int64_t sz_batch_stride,
+                                           int64_t sz_row_stride, int bits, int fmt, int64_t samples,
+                                           int heads_per_kv, int64_t M, int64_t K, int64_t N, void *out,
+                                           int64_t out_batch_stride, int64_t out_row_stride,
+                                           kvmix_stream_t stream)
+{
+    // the documented bound, not the launch plan's exact need: what is refused depends on sizes only
+    if (kvmix_gemv_workspace_bytes(samples, M, K, N) > KVMIX_GEMV_STATIC_SCRATCH_BYTES) return KVMIX_ERR_STATIC_SCRATCH;
+    void *ws = static_scratch();
+    if (!ws) return KVMIX_ERR_STATIC_SCRATCH;
+    return quantized_gemv(group, x, x_batch_stride, x_row_stride, code, code_batch_stride, code_row_stride, scale,
+                          zero, sz_batch_stride, sz_row_stride, bits, fmt, samples, heads_per_kv, M, K, N, out,
+                          out_batch_stride, out_row_stride, ws, KVMIX_GEMV_STATIC_SCRATCH_BYTES, true, stream);
+}
+
+static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
+                          int64_t x_row_stride, const uint32_t *code,
+                          int64_t code_batch_stride, int64_t code_row_stride,
+                          const void *scale, const void *zero, int64_t sz_batch_stride,
+                          int64_t sz_row_stride, int bits, int fmt, int64_t samples,
+                          int heads_per_kv, int64_t M, int64_t K, int64_t N, void *out,
+                          int64_t out_batch_stride, int64_t out_row_stride, void *workspace,
+                          size_t workspace_bytes, bool workspace_is_static, kvmix_stream_t stream)
 {
     if (fmt != KVMIX_FMT_REF && fmt != KVMIX_FMT_DENSE3) return KVMIX_ERR_FORMAT;
     if (bits != 1 && bits != 2 && bits != 3 && bits != 4) return KVMIX_ERR_BITS;
@@ -2381,7 +2447,8 @@ extern "C" int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_st
                                      rows_max_waves(rows_use_mfma(mode, N, K, code_row_stride), nrep));
         if (p.splits > 1) {
             const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
-            if (!workspace || workspace_bytes < need) return KVMIX_ERR_WORKSPACE;
+            if (!workspace || workspace_bytes < need)
+                return workspace_is_static ? KVMIX_ERR_STATIC_SCRATCH : KVMIX_ERR_WORKSPACE;
         }
         switch (mode) {
         case 1: launch_rows<1>(a, samples, st); break;
