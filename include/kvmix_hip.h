@@ -324,6 +324,41 @@ typedef struct kvmix_rope_append {
 
 int kvmix_rope_append(const kvmix_rope_append_t *step, kvmix_stream_t stream);
 
+/*
+ * Measurement support, no counterpart in the reference and not called by any operator: a kernel
+ * that only reads, in the access patterns of the GEMV kernels, to establish what streaming rate
+ * the GPU reaches without arithmetic (the ceiling the GEMV figures are compared with), and how
+ * that rate falls when arithmetic is added to the same loop.
+ *   pattern 0 ("slab", the p.V pattern): `count` blocks of `waves` waves (1..16), block i reads the
+ *       a0 contiguous bytes at buf + i * a0 in chunks of 64 * bytes_per_lane * in_flight bytes
+ *       handed round-robin to its waves; a0 must be a multiple of the chunk.  Reads count * a0 bytes.
+ *   pattern 1 ("rows", the q.K^T pattern): buf is [count slices][a0 rows][a1 row bytes]; a wave
+ *       owns a column piece of 64 * bytes_per_lane bytes and walks it down the a0 rows of its
+ *       slice, in_flight rows at a time; `waves` (1..4) neighbouring pieces per block.
+ *       Reads count * a0 * a1 bytes.
+ *   pattern 2 ("rows and side arrays", what a 4-bit q.K^T launch reads): pattern 1 with 8 bytes per
+ *       lane and 16 rows in flight (bytes_per_lane and in_flight are ignored), plus per 16 rows one
+ *       16-byte load per lane from each of two side arrays [count][a0][a1 / 8] that follow the code
+ *       array in buf (64-byte pieces per row and wave, as the scales and zeros are read).
+ *       Reads count * a0 * a1 * 1.25 bytes.
+ * bytes_per_lane in {4, 8, 16}, in_flight in {4, 8, 16}; sink: 4 writable bytes (never written
+ * for a buffer that does not xor to one particular pattern).
+ * flags: KVMIX_PROBE_NT non-temporal loads (pattern 2: of the code array); pattern 2 only:
+ * KVMIX_PROBE_NT_SIDE the side arrays too, KVMIX_PROBE_XCD_ORDER consecutive logical blocks on one XCD,
+ * KVMIX_PROBE_ROTATING the kernels' order of issue (four rows consumed, four refilled) instead of
+ * 18 loads in a burst, KVMIX_PROBE_ALU(n) n = 0..15 rounds of synthetic arithmetic per four rows (a
+ * round: 16 integer vector operations, four of them 32-bit multiplies, and one 4x4x4 matrix-core
+ * operation), KVMIX_PROBE_LDS_KIB(k) k KiB of unused LDS per block to hold the resident waves down.
+ */
+#define KVMIX_PROBE_NT 1
+#define KVMIX_PROBE_NT_SIDE 2
+#define KVMIX_PROBE_XCD_ORDER 4
+#define KVMIX_PROBE_ROTATING 8
+#define KVMIX_PROBE_ALU(n) (((n) & 15) << 4)
+#define KVMIX_PROBE_LDS_KIB(k) (((k) & 255) << 8)
+int kvmix_probe_stream_read(const void *buf, int pattern, int64_t a0, int64_t a1, int count, int waves,
+                            int bytes_per_lane, int in_flight, int flags, void *sink, kvmix_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ EXPORTS = (
     "kvmix_decode_attention_fused_workspace_bytes",
     "kvmix_decode_attention_fused",
     "kvmix_rope_append",
+    "kvmix_probe_stream_read",
 )
 
 _lib = None
@@ -133,6 +134,8 @@ def load() -> ctypes.CDLL:
     L.kvmix_decode_attention_fused.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
     L.kvmix_rope_append.restype = i32
     L.kvmix_rope_append.argtypes = [ctypes.POINTER(RopeAppend), vp]
+    L.kvmix_probe_stream_read.restype = i32
+    L.kvmix_probe_stream_read.argtypes = [vp, i32, i64, i64, i32, i32, i32, i32, i32, vp, vp]
     _lib = L
     return L
 

@@ -8,7 +8,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libkvmix_hip.so")
-SOURCES = ["abi.hip", "quant_pack.hip", "dequant_gemv.hip", "decode_attn.hip", "fused_attn.hip", "rope_append.hip"]
+SOURCES = ["abi.hip", "quant_pack.hip", "dequant_gemv.hip", "decode_attn.hip", "fused_attn.hip", "rope_append.hip", "stream_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -87,6 +87,18 @@
 #ifndef KVMIX_ROWS_SINGLE_BLOCK_CHUNKS
 #define KVMIX_ROWS_SINGLE_BLOCK_CHUNKS 2  // p.V: keep one block per output row up to this many chunks per wave
 #endif
+#ifndef KVMIX_MFMA2_SPLIT4
+#define KVMIX_MFMA2_SPLIT4 1  // gemv_cols_mfma2, 4 bits: two dword loads per row instead of one dwordx2 + lane exchange
+#endif
+#ifndef KVMIX_STREAM_NT
+#define KVMIX_STREAM_NT 1  // non-temporal loads for the packed operands
+#endif
+#ifndef KVMIX_COLS_NT_CODES
+#define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal
+#endif
+#ifndef KVMIX_COLS_NT_SZ
+#define KVMIX_COLS_NT_SZ 0  // q.K^T kernels: scales and zeros non-temporal
+#endif
 #ifndef KVMIX_TARGET_WAVES
 #define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
 #endif
@@ -115,6 +127,39 @@ struct GemvArgs {
     int ksplit;  // gemv_cols_mfma2: waves that share a tile and slice K
 };
 
+// Buffer addressing for the streaming loops: address = descriptor base (scalar registers) + a per-lane
+// byte offset that never changes (one vector register) + a byte offset that is the same for the whole
+// wave (a scalar register: the row).  A flat global load needs the full 64-bit address in two vector
+// registers per load, formed by vector-ALU adds; here the row arithmetic runs on the scalar unit and costs
+// the vector ALU nothing.  Offsets are 32-bit: the host only sends problems whose (batch, kv-head)
+// slice stays below 2^32 bytes to the kernels that use this.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const void *base)
+{
+    // raw buffer, no stride, no bounds (num_records = 2^32 - 1 bytes), 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)0xffffffffu, 0x00020000);
+}
+template <typename T, bool NT>
+__device__ __forceinline__ T ld_buffer(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_bytes, uint32_t wave_bytes)
+{
+    constexpr int AUX = (NT && KVMIX_STREAM_NT) ? 2 : 0;  // bit 1 of the cache policy = non-temporal
+    T out;
+    if constexpr (sizeof(T) == 16) {
+        const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, wave_bytes, AUX);
+        __builtin_memcpy(&out, &v, 16);
+    } else if constexpr (sizeof(T) == 8) {
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_bytes, wave_bytes, AUX);
+        __builtin_memcpy(&out, &v, 8);
+    } else if constexpr (sizeof(T) == 4) {
+        const auto v = __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes, wave_bytes, AUX);
+        __builtin_memcpy(&out, &v, 4);
+    } else {
+        static_assert(sizeof(T) == 2, "unsupported size for a buffer load");
+        const auto v = __builtin_amdgcn_raw_buffer_load_b16(rsrc, lane_bytes, wave_bytes, AUX);
+        __builtin_memcpy(&out, &v, 2);
+    }
+    return out;
+}
+
 // MODE: 1, 2, 4 = reference layout with that many bits (group 32 in the fast kernels),
 //       3 = the reference's 3-bit layout (11 codes per word, group 11),
 //       30 = dense 3-bit stream (32 codes in 3 words, group 32).
@@ -136,6 +181,69 @@ struct __attribute__((packed, aligned(4))) Words {
 struct __attribute__((packed, aligned(2))) Half8 {
     uint16_t v[8];
 };
+
+// Packed codes are read exactly once per launch: they are loaded non-temporally (the `nt` bit of
+// global_load), which keeps the stream from displacing itself and its neighbours in the caches on
+// the way.  Measured on MI355X with a kernel that only reads: 6.0-6.2 TB/s with plain loads against
+// 6.7-6.9 TB/s with non-temporal ones for contiguous slabs (the p.V pattern), 6.1 against 6.4-6.6 TB/s
+// for row pieces (the q.K^T pattern).  The scales and zeros of the q.K^T kernels stay on plain loads:
+// their 64-byte row pieces share cache lines with the neighbouring wave's, which the L2 has to keep.
+// T: a trivially copyable type of 1, 2, 4, 8, 12 or 16 bytes whose alignment (2 or at least 4) is all
+// that is assumed of the address.
+typedef uint32_t nt_u4a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t nt_u2a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t nt_u1a4 __attribute__((aligned(4)));
+typedef uint16_t nt_h8a2 __attribute__((ext_vector_type(8), aligned(2)));
+typedef uint16_t nt_h4a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint16_t nt_h2a2 __attribute__((ext_vector_type(2), aligned(2)));
+
+template <typename V, bool NT, typename T>
+__device__ __forceinline__ void ld_stream_as(T &out, const void *p)
+{
+    static_assert(sizeof(V) == sizeof(T), "size");
+    V v;
+    if constexpr (NT && KVMIX_STREAM_NT)
+        v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    else
+        v = *reinterpret_cast<const V *>(p);
+    __builtin_memcpy(&out, &v, sizeof(T));
+}
+
+template <typename T, bool NT = true>
+__device__ __forceinline__ T ld_stream(const void *p)
+{
+    constexpr int N = sizeof(T);
+    constexpr int A = alignof(T);
+    T out;
+    if constexpr (A >= 4 && N == 16) {
+        ld_stream_as<nt_u4a4, NT>(out, p);
+    } else if constexpr (A >= 4 && N == 8) {
+        ld_stream_as<nt_u2a4, NT>(out, p);
+    } else if constexpr (A >= 4 && N == 4) {
+        ld_stream_as<nt_u1a4, NT>(out, p);
+    } else if constexpr (A >= 4 && N == 12) {
+        struct __attribute__((packed, aligned(4))) Lo {
+            uint32_t v[2];
+        } lo;
+        uint32_t hi;
+        ld_stream_as<nt_u2a4, NT>(lo, p);
+        ld_stream_as<nt_u1a4, NT>(hi, reinterpret_cast<const uint8_t *>(p) + 8);
+        __builtin_memcpy(&out, &lo, 8);
+        __builtin_memcpy(reinterpret_cast<uint8_t *>(&out) + 8, &hi, 4);
+    } else if constexpr (A == 2 && N == 16) {
+        ld_stream_as<nt_h8a2, NT>(out, p);
+    } else if constexpr (A == 2 && N == 8) {
+        ld_stream_as<nt_h4a2, NT>(out, p);
+    } else if constexpr (A == 2 && N == 4) {
+        ld_stream_as<nt_h2a2, NT>(out, p);
+    } else if constexpr (N == 2) {
+        ld_stream_as<uint16_t, NT>(out, p);
+    } else {
+        static_assert(N == 1, "unsupported size for a streamed load");
+        ld_stream_as<uint8_t, NT>(out, p);
+    }
+    return out;
+}
 
 // Integer codes are fed to the multiplier as fp16 SUBNORMALS: a 16-bit pattern p < 2048 read
 // as binary16 is exactly p * 2^-24 (the first two binades share one ulp).  Masking a field of
@@ -413,12 +521,12 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
             const uint32_t off0 = (uint32_t)kfirst * c_rs + lane_word0;
 #pragma unroll
             for (int u = 0; u < U; u++)
-                w[u] = *reinterpret_cast<const Words<LW> *>(cp + (off0 + (uint32_t)u * c_rs));
+                w[u] = ld_stream<Words<LW>, KVMIX_COLS_NT_CODES>(cp + (off0 + (uint32_t)u * c_rs));
         } else {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int k = kfirst + u < K ? kfirst + u : K - 1;
-                w[u] = *reinterpret_cast<const Words<LW> *>(cp + ((uint32_t)k * c_rs + lane_word0));
+                w[u] = ld_stream<Words<LW>, KVMIX_COLS_NT_CODES>(cp + ((uint32_t)k * c_rs + lane_word0));
             }
         }
     };
@@ -448,8 +556,8 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
             const int row = idx / SEGS, seg = idx % SEGS;
             const int rowc = kc + (row < rows ? row : rows - 1);
             const uint32_t off = (uint32_t)rowc * s_rs + (uint32_t)(t0 + seg * 8);
-            s8[it] = *reinterpret_cast<const Half8 *>(sp + off);
-            z8[it] = *reinterpret_cast<const Half8 *>(zp + off);
+            s8[it] = ld_stream<Half8, KVMIX_COLS_NT_SZ>(sp + off);
+            z8[it] = ld_stream<Half8, KVMIX_COLS_NT_SZ>(zp + off);
         }
         uint16_t xh[(KC + kWave - 1) / kWave];
 #pragma unroll
@@ -616,9 +724,9 @@ gemv_cols3(GemvArgs a)
     HalfN sw[U], zw[U];
     auto load_row = [&](int u, int k) {
         const uint32_t kc = (uint32_t)(k < kend ? k : K - 1);
-        cw[u] = *reinterpret_cast<const Words<UPL> *>(cp + kc * c_rs);
-        sw[u] = *reinterpret_cast<const HalfN *>(sp + kc * s_rs);
-        zw[u] = *reinterpret_cast<const HalfN *>(zp + kc * s_rs);
+        cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cp + kc * c_rs);
+        sw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(sp + kc * s_rs);
+        zw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(zp + kc * s_rs);
     };
     // x of the U rows of a step is read from LDS in one go at the head of the step: read row by row,
     // each read's latency sits in front of that row's arithmetic
@@ -675,9 +783,9 @@ gemv_cols3(GemvArgs a)
         uint32_t so = ((uint32_t)unit0 + (uint32_t)kbeg * s_rs) * 2u;
         const uint32_t c_step = c_rs * 4u, s_step = s_rs * 2u;
         auto next_row = [&](int u) {
-            cw[u] = *reinterpret_cast<const Words<UPL> *>(cb + co);
-            sw[u] = *reinterpret_cast<const HalfN *>(sb + so);
-            zw[u] = *reinterpret_cast<const HalfN *>(zb + so);
+            cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cb + co);
+            sw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(sb + so);
+            zw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(zb + so);
             co += c_step;
             so += s_step;
         };
@@ -875,8 +983,8 @@ __global__ void __launch_bounds__(NREP > 1 ? 64 * kRowsHeadsWaves : 64 * kRowsMa
         int kr = k0 + row0;  // a window cut by the end of the range is read one window early
         kr = kr + RPS <= ke32 ? kr : ke32 - RPS;  // (in bounds: the host routes K < 8 elsewhere)
         kr = kr < 0 ? 0 : kr;
-        s8 = *reinterpret_cast<const Half8 *>(sp + (uint32_t)kr * LPR);
-        z8 = *reinterpret_cast<const Half8 *>(zp + (uint32_t)kr * LPR);
+        s8 = ld_stream<Half8>(sp + (uint32_t)kr * LPR);
+        z8 = ld_stream<Half8>(zp + (uint32_t)kr * LPR);
 #pragma unroll
         for (int h = 0; h < NREP; h++) {
 #pragma unroll
@@ -889,7 +997,7 @@ __global__ void __launch_bounds__(NREP > 1 ? 64 * kRowsHeadsWaves : 64 * kRowsMa
         for (int t = 0; t < HT; t++) {
             int k = k0 + (t0 + t) * RPW + r;
             k = k < ke32 ? k : ke32 - 1;
-            w[t] = *reinterpret_cast<const Words<WORDS> *>(cp + (uint32_t)k * c_rs);
+            w[t] = ld_stream<Words<WORDS>>(cp + (uint32_t)k * c_rs);
         }
     };
     auto stage = [&](int k0) {
@@ -1152,8 +1260,8 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : ke32 - CH; };
     auto load_small = [&](int d, int k0) {
         const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
-        s8[d] = *reinterpret_cast<const Half8 *>(sp + kr * LPR);
-        z8[d] = *reinterpret_cast<const Half8 *>(zp + kr * LPR);
+        s8[d] = ld_stream<Half8>(sp + kr * LPR);
+        z8[d] = ld_stream<Half8>(zp + kr * LPR);
 #pragma unroll
         for (int h = 0; h < NREP; h++) xh[d][h] = *reinterpret_cast<const Half2x *>(xp + h * a.x_bs + kr);
     };
@@ -1161,7 +1269,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
 #pragma unroll
         for (int k = 0; k < 4; k++)
-            w[d][t][k] = *reinterpret_cast<const Elem *>(base + (t * RKB + RL * k) * (EPR * EB));
+            w[d][t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
     };
     auto stage = [&](int d, int k0) {
         const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
@@ -1431,15 +1539,15 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     auto load_small = [&](int it) {
         const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
         const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
-        s8 = *reinterpret_cast<const Half8 *>(sbase + off);
-        z8 = *reinterpret_cast<const Half8 *>(zbase + off);
+        s8 = ld_stream<Half8, KVMIX_COLS_NT_SZ>(sbase + off);
+        z8 = ld_stream<Half8, KVMIX_COLS_NT_SZ>(zbase + off);
 #pragma unroll
         for (int h = 0; h < NREP; h++) xh[h] = xp[h * a.x_bs + d];
     };
     auto load_codes = [&](int it, int t) {
         const Elem *base = cbase + ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_re + (uint32_t)tile_g0(it) * 4);
 #pragma unroll
-        for (int k = 0; k < 4; k++) w[t][k] = base[(uint32_t)k * c_re];
+        for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem, KVMIX_COLS_NT_CODES>(base + (uint32_t)k * c_re);
     };
     auto stage = [&](int it) {
         const int k0 = chunk_k0(it);
@@ -1581,6 +1689,11 @@ gemv_cols_mfma2(GemvArgs a)
     constexpr int FPB = 8 / BITS;
     constexpr int TG = 32;             // groups per tile
     constexpr int WL = BITS == 4 ? 2 : 1;  // registers per lane and row (1 bit: a ushort in one register)
+    // 4 bits: the lane's two elements are element `lane` of each 256-byte half of the tile row (two dword
+    // loads), so that a quad of lanes holds the four elements of ONE group in either half: set s works on
+    // half s with every lane's own register, no exchange between lanes.  Group g of the tile is then set
+    // g / 16, quad g % 16.  (2 bits, 1 bit: neighbouring elements, sets 0 / 1 = the quad's first / second group.)
+    constexpr bool SPLIT = BITS == 4 && KVMIX_MFMA2_SPLIT4;
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
@@ -1612,13 +1725,15 @@ gemv_cols_mfma2(GemvArgs a)
     const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
-    // (byte pointer: a lane's two elements are 2 * BITS bytes)
-    const uint8_t *cbase = reinterpret_cast<const uint8_t *>(a.code + kv * a.c_bs) + lane * (2 * BITS);
+    // buffer descriptors of this (batch, kv-head) slice; a lane's two elements are 2 * BITS bytes
+    const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.code + kv * a.c_bs);
+    const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.scale + kv * a.s_bs);
+    const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.zero + kv * a.s_bs);
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
     const int sub = lane % 4;   // staging: row lane/4 of the chunk, groups 8*sub .. 8*sub+7
     const int srow = lane / 4;
-    const uint16_t *sbase = reinterpret_cast<const uint16_t *>(a.scale) + kv * a.s_bs + 8 * sub;
-    const uint16_t *zbase = reinterpret_cast<const uint16_t *>(a.zero) + kv * a.s_bs + 8 * sub;
+    const uint32_t c_lane = SPLIT ? (uint32_t)lane * 4u : (uint32_t)lane * (2 * BITS);  // bytes
+    const uint32_t s_lane = 2u * ((uint32_t)srow * s_rs + 8u * (uint32_t)sub);    // bytes
     const int j4 = lane % 4;    // position in the quad
 
     f32x4_t acc[2][NPOS];
@@ -1638,7 +1753,7 @@ gemv_cols_mfma2(GemvArgs a)
     auto cell = [](int t, int s, int l) { return (2 * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
     // staged row srow is k-slot srow%4 of k-step srow/4; its group g = 8*sub + jj is set g%2 of quad g/2,
     // i.e. operand lanes 4*(g/2) + i = 16*sub + 4*(jj/2) + i
-    const int aoff = cell(srow / 4, 0, 16 * sub) + srow % 4;
+    const int aoff = SPLIT ? cell(srow / 4, sub / 2, 32 * (sub % 2)) + srow % 4 : cell(srow / 4, 0, 16 * sub) + srow % 4;
 
     Half8 s8, z8;
     uint16_t xh;
@@ -1658,21 +1773,24 @@ gemv_cols_mfma2(GemvArgs a)
     };
     auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
     auto load_small = [&](int it) {
-        const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
-        const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
-        s8 = *reinterpret_cast<const Half8 *>(sbase + off);
-        z8 = *reinterpret_cast<const Half8 *>(zbase + off);
-        xh = xp[d];
+        const uint32_t d0 = (uint32_t)chunk_base(chunk_k0(it));
+        const uint32_t off = 2u * (d0 * s_rs + (uint32_t)tile_g0(it));  // bytes, the same for every lane
+        s8 = ld_buffer<Half8, KVMIX_COLS_NT_SZ>(srsrc, s_lane, off);
+        z8 = ld_buffer<Half8, KVMIX_COLS_NT_SZ>(zrsrc, s_lane, off);
+        xh = xp[d0 + (uint32_t)srow];
     };
     auto load_codes = [&](int it, int t) {
         // (a group of 32 codes is BITS words)
-        const uint8_t *base = cbase + 4u * ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
+        const uint32_t base = 4u * ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             if constexpr (BITS == 1) {
-                w[t][k][0] = *reinterpret_cast<const uint16_t *>(base + 4u * (uint32_t)k * c_rs);
+                w[t][k][0] = ld_buffer<uint16_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+            } else if constexpr (SPLIT) {
+                w[t][k][0] = ld_buffer<uint32_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                w[t][k][1] = ld_buffer<uint32_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane + 256u, base + 4u * (uint32_t)k * c_rs);
             } else {
-                const Words<WL> v = *reinterpret_cast<const Words<WL> *>(base + 4u * (uint32_t)k * c_rs);
+                const Words<WL> v = ld_buffer<Words<WL>, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
 #pragma unroll
                 for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
             }
@@ -1693,8 +1811,12 @@ gemv_cols_mfma2(GemvArgs a)
             const float v2 = v1 - __uint_as_float(b1);
             const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
 #pragma unroll
-            for (int pt = 0; pt < 3; pt++)
-                atile[aoff + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+            for (int pt = 0; pt < 3; pt++) {
+                if constexpr (SPLIT)  // operand lane 32 * (sub % 2) + 4 * jj + pt of set sub / 2
+                    atile[aoff + (((4 * jj + pt) / 16) * 17 + (4 * jj + pt) % 16) * 4] = (uint16_t)(part[pt] >> 16);
+                else
+                    atile[aoff + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+            }
         }
     };
     // first element (8 codes) of the group set s works on, as this lane sees it: for 4 bits the
@@ -1710,7 +1832,9 @@ gemv_cols_mfma2(GemvArgs a)
             uint32_t hi = 0;  // 2 bits / 1 bit: byte offset (0 or 2 / 0 or 1) of the element inside the register
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                if constexpr (BITS == 4) {
+                if constexpr (SPLIT) {
+                    src[k] = w[t][k][s];
+                } else if constexpr (BITS == 4) {
                     const uint32_t other = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][1], 0x44, 0xf, 0xf, false)
                                                   : __builtin_amdgcn_mov_dpp(w[t][k][1], 0xEE, 0xf, 0xf, false);
                     const bool own = s == 0 ? j4 < 2 : j4 >= 2;
@@ -1785,14 +1909,14 @@ gemv_cols_mfma2(GemvArgs a)
             uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)tile_g0(it) * 32;
 #pragma unroll
             for (int s = 0; s < 2; s++) {
-                const float zt = zl[2 * q + s];
+                const float zt = SPLIT ? zl[16 * s + q] : zl[2 * q + s];
                 // element of the quad's 8 that this lane's accumulators of set s belong to
                 const int elem = s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1)));
                 Out8 o;
 #pragma unroll
                 for (int p = 0; p < NPOS; p++)
                     o.v[p] = f32_to_h16(fmaf(sum[s][p], __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
-                *reinterpret_cast<Out8 *>(orow + (8 * q + elem) * 8) = o;
+                *reinterpret_cast<Out8 *>(orow + (SPLIT ? 64 * s + lane : 8 * q + elem) * 8) = o;
             }
         }
         wave_lds_fence();
