@@ -96,6 +96,9 @@
 #ifndef KVMIX_COLS_NT_CODES
 #define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal
 #endif
+#ifndef KVMIX_COLS3_NT_SZ
+#define KVMIX_COLS3_NT_SZ 1  // q.K^T, reference 3-bit words, one head per pass: scales and zeros (as large as the codes) non-temporal
+#endif
 #ifndef KVMIX_COLS_NT_SZ
 #define KVMIX_COLS_NT_SZ 0  // q.K^T kernels: scales and zeros non-temporal
 #endif
@@ -725,8 +728,8 @@ gemv_cols3(GemvArgs a)
     auto load_row = [&](int u, int k) {
         const uint32_t kc = (uint32_t)(k < kend ? k : K - 1);
         cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cp + kc * c_rs);
-        sw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(sp + kc * s_rs);
-        zw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(zp + kc * s_rs);
+        sw[u] = ld_stream<HalfN, (KVMIX_COLS3_NT_SZ && NREP == 1)>(sp + kc * s_rs);
+        zw[u] = ld_stream<HalfN, (KVMIX_COLS3_NT_SZ && NREP == 1)>(zp + kc * s_rs);
     };
     // x of the U rows of a step is read from LDS in one go at the head of the step: read row by row,
     // each read's latency sits in front of that row's arithmetic
@@ -784,8 +787,8 @@ gemv_cols3(GemvArgs a)
         const uint32_t c_step = c_rs * 4u, s_step = s_rs * 2u;
         auto next_row = [&](int u) {
             cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cb + co);
-            sw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(sb + so);
-            zw[u] = ld_stream<HalfN, KVMIX_COLS_NT_SZ>(zb + so);
+            sw[u] = ld_stream<HalfN, (KVMIX_COLS3_NT_SZ && NREP == 1)>(sb + so);
+            zw[u] = ld_stream<HalfN, (KVMIX_COLS3_NT_SZ && NREP == 1)>(zb + so);
             co += c_step;
             so += s_step;
         };
