@@ -75,6 +75,9 @@
 #ifndef KVMIX_COLS_MFMA2_1BIT
 #define KVMIX_COLS_MFMA2_1BIT 1  // 1-bit q.K^T through the two-element kernel too
 #endif
+#ifndef KVMIX_MFMA2_RESIDENT_WAVES
+#define KVMIX_MFMA2_RESIDENT_WAVES 3072  // gemv_cols_mfma2: 3 waves on each of 1024 SIMDs
+#endif
 #ifndef KVMIX_MFMA2_MAX_TPW
 #define KVMIX_MFMA2_MAX_TPW 1  // gemv_cols_mfma2: tiles a wave walks at most (measured: one tile per wave and more waves beats several tiles per wave at every size tried)
 #endif
@@ -94,7 +97,7 @@
 #define KVMIX_STREAM_NT 1  // non-temporal loads for the packed operands
 #endif
 #ifndef KVMIX_COLS_NT_CODES
-#define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal
+#define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal (the matrix-core kernels: 2 and 4 bits only -- a wave's 1-bit row piece is 64 or 128 bytes and shares its cache lines with the neighbours')
 #endif
 #ifndef KVMIX_COLS3_NT_SZ
 #define KVMIX_COLS3_NT_SZ 1  // q.K^T, reference 3-bit words, one head per pass: scales and zeros (as large as the codes) non-temporal
@@ -1550,7 +1553,7 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     auto load_codes = [&](int it, int t) {
         const Elem *base = cbase + ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_re + (uint32_t)tile_g0(it) * 4);
 #pragma unroll
-        for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem, KVMIX_COLS_NT_CODES>(base + (uint32_t)k * c_re);
+        for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem, (KVMIX_COLS_NT_CODES && BITS >= 2)>(base + (uint32_t)k * c_re);
     };
     auto stage = [&](int it) {
         const int k0 = chunk_k0(it);
@@ -1680,7 +1683,9 @@ __global__ void __launch_bounds__(64 * kColsWaves)
 constexpr int kColsMfma2Row = 74 * 4;                   // bf16 elements per (k-step, set) row
 constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets
 
-template <int BITS>
+// NTC: the codes are loaded non-temporally (the host asks for it while the launch is no more than a few rounds of
+// resident waves: measured faster up to 8k waves, slower at 16k, where rows of neighbouring tiles meet in the L2)
+template <int BITS, bool NTC>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(KVMIX_MFMA2_OCC4)))
 gemv_cols_mfma2(GemvArgs a)
 {
@@ -1788,12 +1793,12 @@ gemv_cols_mfma2(GemvArgs a)
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             if constexpr (BITS == 1) {
-                w[t][k][0] = ld_buffer<uint16_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                w[t][k][0] = ld_buffer<uint16_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
             } else if constexpr (SPLIT) {
-                w[t][k][0] = ld_buffer<uint32_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
-                w[t][k][1] = ld_buffer<uint32_t, KVMIX_COLS_NT_CODES>(crsrc, c_lane + 256u, base + 4u * (uint32_t)k * c_rs);
+                w[t][k][0] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                w[t][k][1] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane + 256u, base + 4u * (uint32_t)k * c_rs);
             } else {
-                const Words<WL> v = ld_buffer<Words<WL>, KVMIX_COLS_NT_CODES>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                const Words<WL> v = ld_buffer<Words<WL>, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
 #pragma unroll
                 for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
             }
@@ -2283,12 +2288,14 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     hipLaunchKernelGGL((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a);
 }
 
-template <int BITS>
-static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
+template <int BITS, bool NTC>
+static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
 {
     const int64_t tiles = (a.N / 32 + 31) / 32;
     const int64_t batch = samples * a.M;
-    int64_t tpw = batch * tiles / kTargetWaves;  // tiles per wave: about one resident round of waves
+    // tiles per wave: as many as it takes for ONE round of resident waves (three per SIMD with this kernel's
+    // registers) to cover the problem -- a partial second round runs with most of the chip idle
+    int64_t tpw = (batch * tiles + KVMIX_MFMA2_RESIDENT_WAVES - 1) / KVMIX_MFMA2_RESIDENT_WAVES;
     tpw = tpw < 1 ? 1 : (tpw > KVMIX_MFMA2_MAX_TPW ? KVMIX_MFMA2_MAX_TPW : tpw);
     // few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
     const int64_t chunks = (a.K + 15) / 16;
@@ -2299,7 +2306,7 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
         a.splits = 1;
         const dim3 grid((unsigned)tiles, (unsigned)samples, (unsigned)a.M);  // one tile per block of ks waves
         const size_t lds = (size_t)ks * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-        hipLaunchKernelGGL((gemv_cols_mfma2<BITS>), grid, dim3(kWave, ks), lds, st, a);
+        hipLaunchKernelGGL((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, ks), lds, st, a);
         return;
     }
     const int64_t slots = (tiles + tpw - 1) / tpw;
@@ -2307,7 +2314,19 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     a.splits = (int)tpw;
     const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
     const size_t lds = (size_t)wpb * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-    hipLaunchKernelGGL((gemv_cols_mfma2<BITS>), grid, dim3(kWave, wpb), lds, st, a);
+    hipLaunchKernelGGL((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, wpb), lds, st, a);
+}
+
+template <int BITS>
+static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
+{
+    // non-temporal code loads: 2 and 4 bits (a wave's 1-bit row piece is 128 bytes and shares its cache lines
+    // with the neighbours'), and only while the launch is at most three rounds of resident waves
+    const int64_t tiles = (a.N / 32 + 31) / 32;
+    if (BITS >= 2 && samples * a.M * tiles <= 3 * (int64_t)KVMIX_MFMA2_RESIDENT_WAVES)
+        launch_cols_mfma2_nt<BITS, true>(a, samples, st);
+    else
+        launch_cols_mfma2_nt<BITS, false>(a, samples, st);
 }
 
 template <int MODE>
