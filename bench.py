@@ -404,6 +404,53 @@ def sweep_extra(torch, _lib, lib, dev, stream):
     return res
 
 
+def stream_ceiling_extra(torch, _lib, lib, dev):
+    """What a kernel that only reads reaches on this GPU (kvmix_probe_stream_read: no arithmetic), in the
+    access patterns of the GEMV kernels, over 1 GiB regions of a 4 GiB buffer taken in turn (nothing is
+    served from the Infinity Cache).  The GEMV figures are to be read against these, not against 8 TB/s alone:
+      slab       contiguous slab per block (the p.V pattern), 1024 blocks of 8 waves, 16 bytes per lane
+      rows       512-byte row pieces down 128 rows of a [512][128][4032 B] array (the q.K^T 4-bit pattern)
+      rows_side  the same plus the two side arrays read as the scales and zeros are (what a 4-bit q.K^T
+                 launch at B=16, T=8192 reads), blocks in XCD-aware order
+    each with plain and with non-temporal loads."""
+    GiB = 1 << 30
+    buf = torch.empty(4 * GiB, dtype=torch.uint8, device=dev)
+    buf.view(torch.int64).random_()
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    NT, SIDE_NT, XCD = 1, 2, 4
+
+    def run(pattern, a0, a1, count, waves, bpl, u, flags, nbytes, reps=20):
+        regions = (4 * GiB) // nbytes
+
+        def go(i):
+            rc = lib.kvmix_probe_stream_read(buf.data_ptr() + (i % regions) * nbytes, pattern, a0, a1, count, waves, bpl, u,
+                                             flags, sink.data_ptr(), st)
+            if rc != 0:
+                raise RuntimeError(_lib.strerror(rc))
+        for i in range(5):
+            go(i)
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(reps):
+            go(i)
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) * 1e3 / reps
+        return {"us": round(us, 1), "MB": round(nbytes / 1e6, 1), "GBps": round(nbytes / us / 1e3, 1)}
+
+    res = {}
+    slab = (GiB // 1024) // (64 * 16 * 8) * (64 * 16 * 8)
+    for name, flags in (("plain", 0), ("nontemporal", NT)):
+        res[f"slab_{name}"] = run(0, slab, 0, 1024, 8, 16, 8, flags, slab * 1024)
+        res[f"rows_{name}"] = run(1, 128, 4032, 512, 4, 8, 16, flags, 512 * 128 * 4032)
+        res[f"rows_side_{name}"] = run(2, 128, 4032, 512, 4, 8, 16, flags | XCD, 512 * 128 * (4032 + 2 * 504))
+    del buf
+    torch.cuda.empty_cache()
+    return res
+
+
 def attention_step_extra(torch, dev):
     """The whole attention step of one layer (logits over packed keys + fp16 tail, softmax, output
     over packed values + fp16 tail) in its two forms: four launches with the reference's roundings,
@@ -605,6 +652,9 @@ def main():
     ap.add_argument("--attention-step-only", action="store_true", help="run only the attention-step comparison")
     ap.add_argument("--shapes-only", action="store_true",
                     help="skip the step: only the B=16/T=8192 target shape and the GQA configuration (for profiling)")
+    ap.add_argument("--stream-ceiling", action="store_true",
+                    help="run only the streaming-read probe (what a kernel without arithmetic reaches)")
+    ap.add_argument("--no-stream-ceiling", action="store_true", help="skip the streaming-read probe")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 1 GiB device copies (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
@@ -622,6 +672,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, D, T, R = args.batch, 32, 128, args.context, 128
+    if args.stream_ceiling:
+        res = stream_ceiling_extra(torch, _lib, lib, dev)
+        print(json.dumps({"hbm_read_ceiling_GBps": max(v["GBps"] for v in res.values()), "stream_ceiling": res}))
+        return
     if args.e2e_only:
         print(json.dumps({"e2e_config4_llama2_7b": e2e_extra(torch, dev)}))
         return
@@ -716,11 +770,16 @@ def main():
     dom = max(per_kernel.items(), key=lambda kv: kv[1]["launches_per_step"] * kv[1]["avg_us"])
     dname, d = dom
     achieved = d["bytes_per_launch"] / d["avg_us"] / 1e3
-    traffic = None
+    # HBM traffic of the dominant kernel: NOT measured in this run -- read from the committed counter summary
+    # (two rocprofv3 --pmc passes, FETCH_SIZE and WRITE_SIZE scaled by a plain copy; profiles/bench_step_kernels_config1.md)
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(dname)
+            tj = json.load(open(tpath))
+            traffic = tj.get(dname)
+            traffic_source = ("profiles/hbm_traffic.json (static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                              + str(tj.get("_measured", "date not recorded")) + "; not re-measured in this run)")
         except Exception:
             traffic = None
     gemv_us = sum(v["launches_per_step"] * v["avg_us"] for k, v in per_kernel.items() if k.startswith("gemv"))
@@ -759,6 +818,7 @@ def main():
         "roofline": {"kernel": dname, "device_kernel": DEVICE_KERNEL.get(dname, ""),
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "bytes_per_launch": int(d["bytes_per_launch"]), "avg_launch_us": round(d["avg_us"], 2)},
     }
     print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H, D, T, R)
@@ -772,6 +832,10 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
         for L in layers:
             L.__dict__.clear()
         torch.cuda.empty_cache()
+        if not args.no_stream_ceiling:
+            res = stream_ceiling_extra(torch, _lib, lib, dev)
+            result["hbm_read_ceiling_GBps"] = max(v["GBps"] for v in res.values())
+            result["stream_ceiling"] = res
         result["target_shape_B16_T8192"] = target_shape_extra(torch, _lib, lib, dev,
                                                               torch.cuda.current_stream().cuda_stream)
         torch.cuda.empty_cache()

@@ -179,6 +179,26 @@ int kvmix_quantized_gemv(int group, const void *x, int64_t x_batch_stride, int64
                          kvmix_stream_t stream);
 
 /*
+ * Which kernel a kvmix_quantized_gemv call of these sizes is dispatched to, without launching
+ * anything and without a GPU (no counterpart in the reference; for tests that pin the dispatch of
+ * the benchmark shapes, and for reading profiles).  code_row_stride / sz_row_stride as in the call
+ * (words / elements between two rows of one slice).  kernel: the kernel's name with its template
+ * arguments; grid, block, lds_bytes: its launch geometry; splits: blocks along K of a p.V kernel
+ * (more than one brings the reduction launch) or tiles a q.K^T wave walks; ksplit: waves that
+ * share a q.K^T tile; launches: kernel launches of the call (0: nothing to do).
+ * Returns the code kvmix_quantized_gemv would return for these sizes.
+ */
+typedef struct kvmix_gemv_plan {
+    char kernel[64];
+    unsigned grid[3], block[3];
+    uint64_t lds_bytes;
+    int splits, ksplit, launches;
+} kvmix_gemv_plan_t;
+int kvmix_quantized_gemv_plan(int group, int bits, int fmt, int64_t samples, int heads_per_kv, int64_t M,
+                              int64_t K, int64_t N, int64_t code_row_stride, int64_t sz_row_stride,
+                              kvmix_gemv_plan_t *plan);
+
+/*
  * kvmix_quantized_gemv for callers that cannot allocate device memory (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments minus the workspace, same kernels, same results bit for bit: the split-K partial

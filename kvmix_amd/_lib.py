@@ -25,6 +25,7 @@ EXPORTS = (
     "kvmix_gemv_workspace_bytes",
     "kvmix_quantized_gemv",
     "kvmix_quantized_gemv_static",
+    "kvmix_quantized_gemv_plan",
     "kvmix_decode_attention_workspace_bytes",
     "kvmix_decode_attention",
     "kvmix_decode_attention_fused_supported",
@@ -88,6 +89,13 @@ class RopeAppend(ctypes.Structure):
                 ("batch", _i64), ("heads", _i32), ("kv_heads", _i32), ("D", _i64)]
 
 
+class GemvPlan(ctypes.Structure):
+    """kvmix_gemv_plan_t"""
+    _fields_ = [("kernel", ctypes.c_char * 64), ("grid", ctypes.c_uint * 3), ("block", ctypes.c_uint * 3),
+                ("lds_bytes", ctypes.c_uint64), ("splits", ctypes.c_int), ("ksplit", ctypes.c_int),
+                ("launches", ctypes.c_int)]
+
+
 class KVmixLibraryMissing(ImportError):
     pass
 
@@ -122,6 +130,8 @@ def load() -> ctypes.CDLL:
     L.kvmix_quantized_gemv_static.restype = i32
     L.kvmix_quantized_gemv_static.argtypes = [i32, vp, i64, i64, vp, i64, i64, vp, vp, i64, i64, i32, i32,
                                               i64, i32, i64, i64, i64, vp, i64, i64, vp]
+    L.kvmix_quantized_gemv_plan.restype = i32
+    L.kvmix_quantized_gemv_plan.argtypes = [i32, i32, i32, i64, i32, i64, i64, i64, i64, i64, ctypes.POINTER(GemvPlan)]
     L.kvmix_decode_attention_workspace_bytes.restype = sz
     L.kvmix_decode_attention_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
     L.kvmix_decode_attention.restype = i32
@@ -138,6 +148,21 @@ def load() -> ctypes.CDLL:
     L.kvmix_probe_stream_read.argtypes = [vp, i32, i64, i64, i32, i32, i32, i32, i32, vp, vp]
     _lib = L
     return L
+
+
+def gemv_plan(group: int, bits: int, fmt: int, samples: int, heads_per_kv: int, M: int, K: int, N: int,
+              code_row_stride: int = None, sz_row_stride: int = None) -> dict:
+    """kvmix_quantized_gemv_plan for dense rows (or the given row strides): the kernel a call of these
+    sizes gets, as a dict.  Needs no GPU."""
+    if code_row_stride is None:
+        code_row_stride = N * 3 // 32 if (bits == 3 and fmt == FMT_DENSE3) else (N // 11 if bits == 3 else N * bits // 32)
+    if sz_row_stride is None:
+        sz_row_stride = N // group
+    plan = GemvPlan()
+    check(load().kvmix_quantized_gemv_plan(group, bits, fmt, samples, heads_per_kv, M, K, N, code_row_stride,
+                                           sz_row_stride, ctypes.byref(plan)))
+    return {"kernel": plan.kernel.decode(), "grid": tuple(plan.grid), "block": tuple(plan.block),
+            "lds_bytes": plan.lds_bytes, "splits": plan.splits, "ksplit": plan.ksplit, "launches": plan.launches}
 
 
 def strerror(code: int) -> str:

@@ -38,6 +38,8 @@
 #include "kvmix_common.h"
 
 #include <atomic>
+#include <cstdarg>
+#include <cstdio>
 #include <mutex>
 
 #ifndef KVMIX_COLS3_HEADS_U
@@ -2069,6 +2071,32 @@ __global__ void __launch_bounds__(GenericCfg<MODE>::THREADS) gemv_generic(GemvAr
 
 constexpr int64_t kTargetWaves = KVMIX_TARGET_WAVES;
 
+// kvmix_quantized_gemv_plan: the dispatch below runs as usual, but every launch is recorded instead of made
+static thread_local kvmix_gemv_plan_t *t_plan = nullptr;
+
+static void plan_record(const dim3 &grid, const dim3 &block, size_t lds, const char *fmt, ...)
+{
+    kvmix_gemv_plan_t *p = t_plan;
+    if (p->launches++ > 0) return;  // (a second launch is the split-K reduction: counted, not described)
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(p->kernel, sizeof(p->kernel), fmt, ap);
+    va_end(ap);
+    p->grid[0] = grid.x, p->grid[1] = grid.y, p->grid[2] = grid.z;
+    p->block[0] = block.x, p->block[1] = block.y, p->block[2] = block.z;
+    p->lds_bytes = lds;
+}
+
+// launch `kernel(args)` -- or, while a plan is being recorded, note its name (a printf format and its
+// arguments: the template parameters) and geometry
+#define KVMIX_LAUNCH(kernel, grid, block, lds, st, args, ...)              \
+    do {                                                                   \
+        if (t_plan)                                                        \
+            plan_record(grid, block, lds, __VA_ARGS__);                    \
+        else                                                               \
+            hipLaunchKernelGGL(kernel, grid, block, lds, st, args);       \
+    } while (0)
+
 static bool rows_shape_ok(int64_t N) { return N == 64 || N == 128 || N == 256; }
 
 struct RowsPlan {
@@ -2143,7 +2171,7 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
         // one A tile per wave and MFMA set; the block reduction (waves*NREP*128 floats) reuses it
         const size_t lds = (size_t)p.waves * rows_mfma_sets(NREP) * kRowsMfmaTile * sizeof(uint16_t);
         constexpr int DEPTH = 1;  // chunks in flight per wave (deeper costs occupancy and was slower)
-        if (lds > 64 * 1024) {
+        if (lds > 64 * 1024 && !t_plan) {
             // above the default per-block limit: raise it for this kernel, once per device
             // (the attribute is idempotent: two threads that both find the flag clear set it twice)
             static std::atomic<bool> raised[kMaxDevices];
@@ -2155,22 +2183,22 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
                 if (dev >= 0 && dev < kMaxDevices) raised[dev].store(true, std::memory_order_release);
             }
         }
-        hipLaunchKernelGGL((gemv_rows_mfma<MODE, NREP, DEPTH>), grid, block, lds, st, a);
+        KVMIX_LAUNCH((gemv_rows_mfma<MODE, NREP, DEPTH>), grid, block, lds, st, a, "gemv_rows_mfma<%d,%d,%d>", MODE, NREP, DEPTH);
         if (a.splits > 1) {
             const dim3 g2((unsigned)((a.N + 255) / 256), (unsigned)samples, (unsigned)a.M);
-            hipLaunchKernelGGL(reduce_splits, g2, dim3(256), 0, st, a);
+            KVMIX_LAUNCH(reduce_splits, g2, dim3(256), 0, st, a, "reduce_splits");
         }
         return;
     }
     const size_t lds = sizeof(float) * (size_t)p.waves * (size_t)NREP * (size_t)(512 + a.N);
     switch (a.N / 32) {
-    case 2: hipLaunchKernelGGL((gemv_rows<MODE, 2, NREP>), grid, block, lds, st, a); break;
-    case 4: hipLaunchKernelGGL((gemv_rows<MODE, 4, NREP>), grid, block, lds, st, a); break;
-    default: hipLaunchKernelGGL((gemv_rows<MODE, 8, NREP>), grid, block, lds, st, a); break;
+    case 2: KVMIX_LAUNCH((gemv_rows<MODE, 2, NREP>), grid, block, lds, st, a, "gemv_rows<%d,2,%d>", MODE, NREP); break;
+    case 4: KVMIX_LAUNCH((gemv_rows<MODE, 4, NREP>), grid, block, lds, st, a, "gemv_rows<%d,4,%d>", MODE, NREP); break;
+    default: KVMIX_LAUNCH((gemv_rows<MODE, 8, NREP>), grid, block, lds, st, a, "gemv_rows<%d,8,%d>", MODE, NREP); break;
     }
     if (a.splits > 1) {
         const dim3 g2((unsigned)((a.N + 255) / 256), (unsigned)samples, (unsigned)a.M);
-        hipLaunchKernelGGL(reduce_splits, g2, dim3(256), 0, st, a);
+        KVMIX_LAUNCH(reduce_splits, g2, dim3(256), 0, st, a, "reduce_splits");
     }
 }
 
@@ -2219,7 +2247,7 @@ static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
     const int64_t tiles = (units + TU - 1) / TU;
     const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, wpb), 0, st, a);
+    KVMIX_LAUNCH((gemv_cols<MODE, RQ, UPL>), grid, dim3(kWave, wpb), 0, st, a, "gemv_cols<%d,%d,%d>", MODE, RQ, UPL);
 }
 
 // smallest tile (in units) any gemv_cols configuration of this mode needs
@@ -2255,13 +2283,13 @@ static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int k
         // one tile per block: its ks waves slice K and leave their sums behind the x vector in LDS
         const dim3 grid((unsigned)tiles, (unsigned)(samples / NREP), (unsigned)a.M);
         const size_t lds = sizeof(float) * ((size_t)NREP * (size_t)(a.K + 1) + (size_t)ks * NREP * UPL * 11 * kWave);
-        hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, ks), lds, st, a);
+        KVMIX_LAUNCH((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, ks), lds, st, a, "gemv_cols3<%d,%d,%d,%d>", RQ, UPL, U, NREP);
         return;
     }
     const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
-    hipLaunchKernelGGL((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, wpb),
-                       sizeof(float) * (size_t)NREP * (size_t)(a.K + 1), st, a);
+    KVMIX_LAUNCH((gemv_cols3<RQ, UPL, U, NREP>), grid, dim3(kWave, wpb), sizeof(float) * (size_t)NREP * (size_t)(a.K + 1), st,
+                 a, "gemv_cols3<%d,%d,%d,%d>", RQ, UPL, U, NREP);
 }
 
 // (gemv_cols_mfma: whole 512-code tiles, at least one whole 32-row chunk)
@@ -2285,7 +2313,7 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     a.splits = (int)tpw;
     const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
     const size_t lds = (size_t)wpb * (rows_mfma_sets(NREP) * kColsMfmaTile * sizeof(uint16_t) + NREP * 16 * sizeof(float));
-    hipLaunchKernelGGL((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a);
+    KVMIX_LAUNCH((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma<%d,%d>", BITS, NREP);
 }
 
 template <int BITS, bool NTC>
@@ -2306,7 +2334,7 @@ static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
         a.splits = 1;
         const dim3 grid((unsigned)tiles, (unsigned)samples, (unsigned)a.M);  // one tile per block of ks waves
         const size_t lds = (size_t)ks * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-        hipLaunchKernelGGL((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, ks), lds, st, a);
+        KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, ks), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
         return;
     }
     const int64_t slots = (tiles + tpw - 1) / tpw;
@@ -2314,7 +2342,7 @@ static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
     a.splits = (int)tpw;
     const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
     const size_t lds = (size_t)wpb * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-    hipLaunchKernelGGL((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, wpb), lds, st, a);
+    KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
 }
 
 template <int BITS>
@@ -2422,7 +2450,10 @@ static void launch_generic(GemvArgs &a, int64_t samples, hipStream_t st)
     const int ub = 1 << ub_log2;
     const size_t lds = ub < THREADS ? (size_t)THREADS * (VALS + 1) * sizeof(float) : 0;
     const dim3 grid((unsigned)((units + ub - 1) / ub), (unsigned)samples, (unsigned)a.M);
-    hipLaunchKernelGGL(gemv_generic<MODE>, grid, dim3(THREADS), lds, st, a, ub_log2);
+    if (t_plan)
+        plan_record(grid, dim3(THREADS), lds, "gemv_generic<%d>", MODE);
+    else
+        hipLaunchKernelGGL(gemv_generic<MODE>, grid, dim3(THREADS), lds, st, a, ub_log2);
 }
 
 }  // namespace kvmix
@@ -2533,8 +2564,10 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
     // first group's scale for the whole word)
     if (group % unit_vals != 0) return KVMIX_ERR_UNSUPPORTED;
     if (samples == 0 || M == 0 || N == 0) return KVMIX_OK;
-    if (!out) return KVMIX_ERR_NULL;
-    if (K > 0 && (!x || !code || !scale || !zero)) return KVMIX_ERR_NULL;
+    if (!t_plan) {
+        if (!out) return KVMIX_ERR_NULL;
+        if (K > 0 && (!x || !code || !scale || !zero)) return KVMIX_ERR_NULL;
+    }
     const int64_t words = N / unit_vals * unit_words, groups = N / group;
     if (code_row_stride < words || sz_row_stride < groups || x_row_stride < K || out_row_stride < N)
         return KVMIX_ERR_SHAPE;
@@ -2593,7 +2626,7 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
                                      rows_max_waves(rows_use_mfma(mode, N, K, code_row_stride), nrep));
         if (p.splits > 1) {
             const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
-            if (!workspace || workspace_bytes < need)
+            if (!t_plan && (!workspace || workspace_bytes < need))
                 return workspace_is_static ? KVMIX_ERR_STATIC_SCRATCH : KVMIX_ERR_WORKSPACE;
         }
         switch (mode) {
@@ -2608,5 +2641,25 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
         KVMIX_DISPATCH(launch_generic)
     }
 #undef KVMIX_DISPATCH
+    if (t_plan) {
+        t_plan->splits = a.splits;
+        t_plan->ksplit = a.ksplit;
+        return KVMIX_OK;
+    }
     return launch_status();
+}
+
+extern "C" int kvmix_quantized_gemv_plan(int group, int bits, int fmt, int64_t samples, int heads_per_kv, int64_t M,
+                                         int64_t K, int64_t N, int64_t code_row_stride, int64_t sz_row_stride,
+                                         kvmix_gemv_plan_t *plan)
+{
+    if (!plan) return KVMIX_ERR_NULL;
+    *plan = kvmix_gemv_plan_t{};
+    t_plan = plan;
+    // contiguous slices: the batch strides only enter the kernels, not the dispatch
+    const int rc = quantized_gemv(group, nullptr, M * K, K, nullptr, K * code_row_stride, code_row_stride, nullptr, nullptr,
+                                  K * sz_row_stride, sz_row_stride, bits, fmt, samples, heads_per_kv, M, K, N, nullptr, M * N,
+                                  N, nullptr, 0, false, nullptr);
+    t_plan = nullptr;
+    return rc;
 }

@@ -1,0 +1,89 @@
+"""Which kernel each benchmark shape is dispatched to (kvmix_quantized_gemv_plan: no launch, no GPU).
+
+A change of the dispatch rules that moves one of the measured shapes onto another kernel (the
+generic fallback above all) has to show up here, not only as a slower bench line.
+"""
+import ctypes
+
+import pytest
+
+from kvmix_amd import _lib
+
+REF, DENSE3 = _lib.FMT_REF, _lib.FMT_DENSE3
+
+
+def plan(bits, fmt, batch, kv_heads, rep, tokens, head_dim, side, group=32):
+    """side 'qk': x is the query (K = head_dim rows, N = tokens); 'pv': x is a row of probabilities."""
+    samples = batch * kv_heads * rep
+    if bits == 3 and fmt == REF:
+        group = 11
+    if side == "qk":
+        return _lib.gemv_plan(group, bits, fmt, samples, rep, 1, head_dim, tokens)
+    return _lib.gemv_plan(group, bits, fmt, samples, rep, 1, tokens, head_dim)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_target_shape_b16_t8k(bits):
+    # 2/4-bit Llama-2-7B KV at 8k context, batch 16 (8064 quantized tokens + the fp16 window)
+    qk = plan(bits, REF, 16, 32, 1, 8064, 128, "qk")
+    assert qk["kernel"].startswith(f"gemv_cols_mfma2<{bits},") and qk["launches"] == 1
+    assert qk["grid"][1] == 512 and qk["block"] == (64, 4, 1)
+    pv = plan(bits, REF, 16, 32, 1, 8064, 128, "pv")
+    assert pv["kernel"] == f"gemv_rows_mfma<{bits},1,1>" and pv["launches"] == 1 and pv["splits"] == 1
+
+
+def test_config0_single_layer_b1_t4096():
+    qk = plan(4, REF, 1, 32, 1, 3968, 128, "qk")
+    assert qk["kernel"].startswith("gemv_cols_mfma2<4,")
+    pv = plan(4, REF, 1, 32, 1, 3968, 128, "pv")
+    # 32 slices: one block of sixteen waves each, no second launch for a reduction
+    assert pv["kernel"] == "gemv_rows_mfma<4,1,1>" and pv["block"] == (64, 16, 1) and pv["launches"] == 1
+
+
+def test_config1_mixed_bits_b8_t8192():
+    assert plan(4, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<4,")
+    assert plan(2, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<2,")
+    # the reference's 3-bit keys: 11 codes a word, 8063 = 733 * 11 tokens
+    assert plan(3, REF, 8, 32, 1, 8063, 128, "qk")["kernel"].startswith("gemv_cols3<")
+    assert plan(3, DENSE3, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols<30,")
+    for bits, mode in ((4, 4), (2, 2)):
+        assert plan(bits, REF, 8, 32, 1, 8064, 128, "pv")["kernel"] == f"gemv_rows_mfma<{mode},1,1>"
+    assert plan(3, DENSE3, 8, 32, 1, 8064, 128, "pv")["kernel"] == "gemv_rows_mfma<30,1,1>"
+
+
+def test_config2_gqa_b16_t32k():
+    # four query heads share a key/value head: one block serves all four from one pass over the codes
+    qk = plan(3, REF, 16, 8, 4, 32637, 128, "qk")
+    assert qk["kernel"].startswith("gemv_cols3<") and qk["kernel"].endswith(",4>")
+    assert qk["grid"][1] == 16 * 8
+    pv = plan(2, REF, 16, 8, 4, 32640, 128, "pv")
+    assert pv["kernel"] == "gemv_rows_mfma<2,4,1>" and pv["grid"][1] == 16 * 8
+
+
+@pytest.mark.parametrize("batch", [1, 16, 64, 128])
+@pytest.mark.parametrize("bits", [1, 2])
+def test_config3_sweep_t4096_residual32(bits, batch):
+    qk = plan(bits, REF, batch, 32, 1, 4064, 128, "qk")["kernel"]
+    if bits == 1 and batch <= 16:
+        assert qk == "gemv_cols_mfma<1,1>"   # several tiles per wave: ahead while one round of waves covers the launch
+    else:
+        # non-temporal code loads (second argument) for 2-bit launches of up to three resident rounds of waves
+        assert qk == f"gemv_cols_mfma2<{bits},{int(bits == 2 and batch <= 64)}>"
+    assert plan(bits, REF, batch, 32, 1, 4064, 128, "pv")["kernel"] == f"gemv_rows_mfma<{bits},1,1>"
+
+
+def test_only_odd_shapes_reach_the_generic_kernel():
+    assert plan(4, REF, 2, 4, 1, 96, 128, "qk")["kernel"] == "gemv_generic<4>"   # three groups a row
+    assert plan(4, REF, 2, 4, 1, 4, 128, "pv")["kernel"] == "gemv_generic<4>"    # four rows
+    assert plan(4, REF, 2, 4, 1, 8064, 128, "qk", group=64)["kernel"] == "gemv_generic<4>"
+    empty = plan(4, REF, 2, 4, 1, 0, 128, "pv")
+    assert empty["launches"] <= 1
+
+
+def test_plan_reports_the_call_s_own_errors():
+    p = _lib.GemvPlan()
+    L = _lib.load()
+    assert L.kvmix_quantized_gemv_plan(32, 5, 0, 1, 1, 1, 128, 128, 16, 4, ctypes.byref(p)) == -1   # KVMIX_ERR_BITS
+    assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 100, 16, 4, ctypes.byref(p)) == -3   # ..._STEPS_GROUP
+    assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 128, 8, 4, ctypes.byref(p)) == -8    # ..._SHAPE
+    assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 128, 16, 4, None) == -7              # ..._NULL
