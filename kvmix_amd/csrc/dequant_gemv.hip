@@ -2258,8 +2258,8 @@ static int64_t cols_min_units()
     return MODE == 3 ? 64 : 16 * ColsUpl<MODE>::value;
 }
 
-#ifndef KVMIX_COLS3_KSPLIT
-#define KVMIX_COLS3_KSPLIT 1  // gemv_cols3: wide tiles shared by two K-slicing waves when there are half as many tiles as waves wanted
+#ifndef KVMIX_COLS3_KSLICE4
+#define KVMIX_COLS3_KSLICE4 1
 #endif
 #ifndef KVMIX_COLS3_WIDE_WAVES
 #define KVMIX_COLS3_WIDE_WAVES 4096
@@ -2402,13 +2402,16 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
         if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
+        else if (KVMIX_COLS3_KSLICE4 && units >= 128 && 2 * ((units + 127) / 128) * 128 <= 3 * units && a.K >= 64 &&
+                 a.K <= 4096 && (waves(128) * 4 <= 1024 || waves(128) * 4 >= 2304))
+            // tiles of 128 words (512 bytes of codes per row), each shared by four waves that slice K: measured
+            // ahead of the one-wave-per-tile configurations below (T = 2.3k..32k, B = 1..128: by 2..35 %) with
+            // streaming loads: longer pieces per row, shorter chains of loads per wave.  Not where that makes
+            // between one and two waves per SIMD (measured behind there), nor where the last tile, moved back
+            // to end at N, would mostly repeat its neighbour.
+            launch_cols3_cfg<2, 4, 1>(a, samples, st, 4);
         else if (units >= 256 && waves(256) >= KVMIX_COLS3_WIDE_WAVES)
             launch_cols3_cfg<1, 4, 1>(a, samples, st);
-        else if (KVMIX_COLS3_KSPLIT && units >= 256 && a.K >= 64 && a.K <= 4096 && waves(256) * 2 >= KVMIX_COLS3_WIDE_WAVES)
-            // half as many wide tiles as that: the widest tile all the same (1 KiB of codes per row and
-            // wave), two waves per tile slicing K (measured: +6 % at B = 32, T = 8k; no gain from four
-            // waves per tile at smaller batches, which keep the narrower tiles below)
-            launch_cols3_cfg<1, 4, 1>(a, samples, st, 2);
         else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
             launch_cols3_cfg<2, 4, 1>(a, samples, st);
         else

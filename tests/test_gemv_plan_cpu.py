@@ -44,7 +44,9 @@ def test_config1_mixed_bits_b8_t8192():
     assert plan(4, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<4,")
     assert plan(2, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<2,")
     # the reference's 3-bit keys: 11 codes a word, 8063 = 733 * 11 tokens
-    assert plan(3, REF, 8, 32, 1, 8063, 128, "qk")["kernel"].startswith("gemv_cols3<")
+    ref3 = plan(3, REF, 8, 32, 1, 8063, 128, "qk")
+    # 128-word tiles, four waves a tile, each with a quarter of the channel rows
+    assert ref3["kernel"] == "gemv_cols3<2,4,8,1>" and ref3["ksplit"] == 4 and ref3["grid"][:2] == (6, 256)
     assert plan(3, DENSE3, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols<30,")
     for bits, mode in ((4, 4), (2, 2)):
         assert plan(bits, REF, 8, 32, 1, 8064, 128, "pv")["kernel"] == f"gemv_rows_mfma<{mode},1,1>"

@@ -92,7 +92,11 @@ def test_reference_3bit_kernel_edges(oracle, dev):
     run_case(oracle, dev, 3, 11, B=1, nh=8, nkv=2, K=50, N=11 * 64, seed=54)     # smallest fast tile, GQA
     run_case(oracle, dev, 3, 11, B=1, nh=2, nkv=2, K=128, N=11 * 131, seed=55, M=2)
     run_case(oracle, dev, 3, 11, B=8, nh=8, nkv=8, K=128, N=11 * 733, seed=56)   # wide tiles (4 words per lane)
-    run_case(oracle, dev, 3, 11, B=32, nh=32, nkv=32, K=64, N=11 * 300, seed=57)  # wide tiles, two waves per tile slicing K
+    run_case(oracle, dev, 3, 11, B=32, nh=32, nkv=32, K=64, N=11 * 300, seed=57)  # four waves per tile slicing K, 16 rows each
+    run_case(oracle, dev, 3, 11, B=1, nh=2, nkv=2, K=100, N=11 * 260, seed=58, M=2)  # ... K ragged against the slices, M = 2
+    run_case(oracle, dev, 3, 11, B=1, nh=3, nkv=3, K=65, N=11 * 128, seed=59)       # ... one tile exactly, a one-row last slice
+    run_case(oracle, dev, 3, 11, B=1, nh=1, nkv=1, K=4096, N=11 * 250, seed=60)     # ... the most rows the sliced form takes
+    run_case(oracle, dev, 3, 11, B=32, nh=32, nkv=32, K=32, N=11 * 1024, seed=61)   # too few rows to slice: widest tiles, one wave each
 
 
 @pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
