@@ -31,12 +31,20 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
-# device kernel behind each tag at this workload (the names the rocprofv3 summaries list)
-DEVICE_KERNEL = {
-    "gemv_cols[ref3]": "kvmix::gemv_cols3<2, 2, 8>", "gemv_cols[b4]": "kvmix::gemv_cols_mfma2<4>",
-    "gemv_cols[b2]": "kvmix::gemv_cols_mfma2<2>", "gemv_rows[b4]": "kvmix::gemv_rows_mfma<4, 1, 1>",
-    "gemv_rows[b2]": "kvmix::gemv_rows_mfma<2, 1, 1>", "gemv_rows[dense3]": "kvmix::gemv_rows_mfma<30, 1, 1>",
-}
+def device_kernel(_lib, tag, B, H, D, Tq):
+    """the device kernel behind a tag of the step (the name the rocprofv3 summaries list), from the
+    library's own dispatch query"""
+    fmts = {"b4": (4, _lib.FMT_REF, 32), "b2": (2, _lib.FMT_REF, 32), "b1": (1, _lib.FMT_REF, 32),
+            "ref3": (3, _lib.FMT_REF, 11), "dense3": (3, _lib.FMT_DENSE3, 32)}
+    try:
+        side, f = tag.rstrip("]").split("[")
+        bits, fmt, group = fmts[f]
+        n = Tq // group * group
+        plan = _lib.gemv_plan(group, bits, fmt, B * H, 1, 1, D, n) if side == "gemv_cols" else \
+            _lib.gemv_plan(group, bits, fmt, B * H, 1, 1, n, D)
+        return "kvmix::" + plan["kernel"]
+    except (KeyError, ValueError):
+        return ""
 
 
 def layer_bits(num_layers: int = 32, seed: int = 1):
@@ -815,7 +823,7 @@ def main():
                            "GBps": round(quant_bytes / quant_us / 1e3, 1)},
         "kernels": {k: {"launches_per_step": v["launches_per_step"], "avg_us": round(v["avg_us"], 2),
                         "GBps": round(v["bytes_per_launch"] / v["avg_us"] / 1e3, 1)} for k, v in per_kernel.items()},
-        "roofline": {"kernel": dname, "device_kernel": DEVICE_KERNEL.get(dname, ""),
+        "roofline": {"kernel": dname, "device_kernel": device_kernel(_lib, dname, B, H, D, T - R),
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "traffic_source": traffic_source,
