@@ -2466,6 +2466,7 @@ using namespace kvmix;
 extern "C" size_t kvmix_gemv_workspace_bytes(int64_t samples, int64_t M, int64_t K, int64_t N)
 {
     if (samples <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
+    if (samples > 65535 || M > 65535) return 0;  // (goes out in parts of more than 30000 rows each: never split)
     // the split count depends on the kernel and on how many query heads share a block (which
     // this query does not know): size for the largest of the possible plans
     const RowsPlan p1 = plan_rows(samples * M, K, N, kRowsMaxWaves);
@@ -2574,7 +2575,31 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
     const int64_t words = N / unit_vals * unit_words, groups = N / group;
     if (code_row_stride < words || sz_row_stride < groups || x_row_stride < K || out_row_stride < N)
         return KVMIX_ERR_SHAPE;
-    if (samples > 65535 || M > 65535) return KVMIX_ERR_SHAPE;  // grid.y / grid.z limits
+    // grid.y / grid.z hold at most 65535 blocks: a larger batch goes out as several launches of nearly equal
+    // size over whole kv heads (and whole groups of M rows), one after the other on the stream.  (Each part
+    // then still has more than 30000 output rows, which no kernel splits over blocks: no workspace.)
+    if (heads_per_kv > 65535) return KVMIX_ERR_SHAPE;
+    if (samples > 65535 || M > 65535) {
+        const int64_t kvs = samples / heads_per_kv, kv_max = 65535 / heads_per_kv;
+        const int64_t sparts = (kvs + kv_max - 1) / kv_max, mparts = (M + 65534) / 65535;
+        const int64_t kv_step = (kvs + sparts - 1) / sparts, mstep = (M + mparts - 1) / mparts;
+        for (int64_t m0 = 0; m0 < M; m0 += mstep) {
+            for (int64_t kv0 = 0; kv0 < kvs; kv0 += kv_step) {
+                const int64_t s0 = kv0 * heads_per_kv, nkv = kvs - kv0 < kv_step ? kvs - kv0 : kv_step;
+                const int64_t nm = M - m0 < mstep ? M - m0 : mstep;
+                const int rc = quantized_gemv(
+                    group, x ? (const __half *)x + s0 * x_batch_stride + m0 * x_row_stride : nullptr, x_batch_stride,
+                    x_row_stride, code ? code + kv0 * code_batch_stride : nullptr, code_batch_stride, code_row_stride,
+                    scale ? (const __half *)scale + kv0 * sz_batch_stride : nullptr,
+                    zero ? (const __half *)zero + kv0 * sz_batch_stride : nullptr, sz_batch_stride, sz_row_stride, bits,
+                    fmt, nkv * heads_per_kv, heads_per_kv, nm, K, N,
+                    out ? (__half *)out + s0 * out_batch_stride + m0 * out_row_stride : nullptr, out_batch_stride,
+                    out_row_stride, workspace, workspace_bytes, workspace_is_static, stream);
+                if (rc != KVMIX_OK) return rc;
+            }
+        }
+        return KVMIX_OK;
+    }
 
     GemvArgs a;
     a.x = (const __half *)x;

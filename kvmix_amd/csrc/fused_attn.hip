@@ -41,6 +41,7 @@ struct FusedArgs {
     int k_mode, v_mode;       // 1, 2, 4 = bits; 3 = the reference's 3-bit words (keys) / dense 3-bit (values); 30 = dense 3-bit keys
     int slab;                 // positions per block
     int slabs;
+    int head_groups;          // blocks per kv head and slab (query heads of a kv head / heads per block)
     int heads_per_kv, heads;
     float inv_sqrt_d;
 };
@@ -337,13 +338,13 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
     // index is mapped to a logical one such that consecutive logical indices share an XCD, and the
     // logical order is slab-fastest, then query head, then kv head: the slabs of one row of scales
     // (neighbours share 128-byte lines) and the query heads of one kv head meet in one L2.
-    const int64_t n_blocks = (int64_t)gridDim.x * gridDim.y * gridDim.z;
-    const int64_t launch = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    // (the grid is one-dimensional: slabs x head groups x kv heads blocks)
+    const int64_t n_blocks = gridDim.x, launch = blockIdx.x;
     const int64_t per = n_blocks / 8, rem = n_blocks % 8, xcd = launch % 8;
     const int64_t logical = xcd * per + (xcd < rem ? xcd : rem) + launch / 8;
-    const int slab = (int)(logical % gridDim.x);
-    const int head_group = (int)((logical / gridDim.x) % gridDim.z);
-    const int64_t kv = logical / ((int64_t)gridDim.x * gridDim.z);
+    const int slab = (int)(logical % a.slabs);
+    const int head_group = (int)((logical / a.slabs) % a.head_groups);
+    const int64_t kv = logical / ((int64_t)a.slabs * a.head_groups);
     const int64_t sample0 = kv * a.heads_per_kv + (int64_t)head_group * NREP;
     const int S = a.slab;
     const int64_t t0 = (int64_t)slab * S, t1 = t0 + S;
@@ -627,7 +628,7 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     }
     const int64_t slabs = fused_slabs(p);
     const int64_t kv_samples = p->samples / p->heads_per_kv;
-    if (slabs > 0x7fffffff || kv_samples > 65535) return KVMIX_ERR_SHAPE;
+    if (slabs > 0x7fffffff || slabs * p->samples > 0x7fffffff) return KVMIX_ERR_SHAPE;  // (blocks of one launch)
     if (!workspace || workspace_bytes < kvmix_decode_attention_fused_workspace_bytes(p)) return KVMIX_ERR_WORKSPACE;
 
     FusedArgs a;
@@ -678,7 +679,8 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     hipStream_t st = (hipStream_t)stream;
     // one query head per block: the heads that share a kv head re-read its slab through L2 (two heads
     // per block need more registers than a 512-thread block has)
-    const dim3 grid((unsigned)slabs, (unsigned)kv_samples, (unsigned)p->heads_per_kv);
+    a.head_groups = p->heads_per_kv;
+    const dim3 grid((unsigned)(slabs * kv_samples * p->heads_per_kv));
     hipLaunchKernelGGL(attn_fused_slab<1>, grid, dim3(kFusedThreads), 0, st, a);
     int rc = launch_status();
     if (rc != KVMIX_OK || slabs == 1) return rc;  // a single slab is normalised and stored by the slab kernel

@@ -721,7 +721,7 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
     const int64_t words = vpw ? n / vpw : n * 3 / 32;
     groups = n / group;
     if (k_token_stride < D || code_inner_stride < words || sz_inner_stride < groups) return KVMIX_ERR_SHAPE;
-    if (outer > 65535 || groups > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    if (groups > 0x7fffffff) return KVMIX_ERR_SHAPE;
     a.k = (const __half *)k;
     a.code = code;
     a.scale = (__half *)scale;
@@ -743,13 +743,23 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
 static int launch_key_tokens(const KeyTokArgs &a, int mode, int64_t groups, int64_t outer, hipStream_t st)
 {
     const int block = a.D >= 128 ? 128 : 64;
-    const dim3 grid((unsigned)groups, (unsigned)outer, (unsigned)((a.D + block - 1) / block));
-    switch (mode) {
-    case 3: hipLaunchKernelGGL((quant_key_tokens<11, 3>), grid, dim3(block), 0, st, a); break;
-    case 30: hipLaunchKernelGGL((quant_key_tokens<32, 30>), grid, dim3(block), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((quant_key_tokens<32, 4>), grid, dim3(block), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((quant_key_tokens<32, 2>), grid, dim3(block), 0, st, a); break;
-    default: hipLaunchKernelGGL((quant_key_tokens<32, 1>), grid, dim3(block), 0, st, a); break;
+    if ((a.D + block - 1) / block > 65535) return KVMIX_ERR_SHAPE;
+    // (grid.y holds at most 65535 blocks: more (batch, head) slices than that go out in several launches)
+    for (int64_t o0 = 0; o0 < outer; o0 += 65535) {
+        KeyTokArgs p = a;
+        p.k += o0 * a.k_os;
+        p.code += o0 * a.c_os;
+        p.scale += o0 * a.s_os;
+        p.zero += o0 * a.s_os;
+        const int64_t no = outer - o0 < 65535 ? outer - o0 : 65535;
+        const dim3 grid((unsigned)groups, (unsigned)no, (unsigned)((a.D + block - 1) / block));
+        switch (mode) {
+        case 3: hipLaunchKernelGGL((quant_key_tokens<11, 3>), grid, dim3(block), 0, st, p); break;
+        case 30: hipLaunchKernelGGL((quant_key_tokens<32, 30>), grid, dim3(block), 0, st, p); break;
+        case 4: hipLaunchKernelGGL((quant_key_tokens<32, 4>), grid, dim3(block), 0, st, p); break;
+        case 2: hipLaunchKernelGGL((quant_key_tokens<32, 2>), grid, dim3(block), 0, st, p); break;
+        default: hipLaunchKernelGGL((quant_key_tokens<32, 1>), grid, dim3(block), 0, st, p); break;
+        }
     }
     return launch_status();
 }

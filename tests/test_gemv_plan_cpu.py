@@ -82,6 +82,14 @@ def test_only_odd_shapes_reach_the_generic_kernel():
     assert empty["launches"] <= 1
 
 
+def test_batches_beyond_a_grid_dimension_go_out_in_parts():
+    p = _lib.gemv_plan(32, 4, REF, 70000, 1, 1, 16, 64)
+    assert p["launches"] == 2 and p["grid"][1] == 35000
+    p = _lib.gemv_plan(32, 4, REF, 3 * 65536, 4, 1, 256, 128)        # whole kv heads (four query heads) per part
+    assert p["launches"] == 4 and p["grid"][1] * 4 * 4 == 3 * 65536
+    assert _lib.load().kvmix_gemv_workspace_bytes(70000, 1, 4096, 128) == 0
+
+
 def test_plan_reports_the_call_s_own_errors():
     p = _lib.GemvPlan()
     L = _lib.load()

@@ -434,3 +434,10 @@ def test_full_size_properties_batch128_t4096(dev, bits):
         out = KVmix.quantized_gemm(g, torch.ones_like(p)[..., :2016], vcode[:, :, :2016], one[:, :, :2016],
                                    torch.zeros_like(one)[:, :, :2016], bits)
         assert torch.equal(out[:, :, 0].to(torch.int32), _unpack_torch(vcode[:, :, :2016], bits).sum(2))
+
+
+def test_more_slices_than_one_grid_dimension_holds(oracle, dev):
+    """B x heads beyond 65535 (the limit of grid.y): the call goes out in parts over whole kv heads."""
+    run_case(oracle, dev, 4, 32, B=16385, nh=4, nkv=4, K=16, N=64, seed=71)      # 65540 slices, two parts
+    run_case(oracle, dev, 2, 32, B=8193, nh=8, nkv=2, K=16, N=64, seed=72)       # 65544 query heads on 16386 kv heads
+    run_case(oracle, dev, 1, 32, B=1, nh=2, nkv=2, K=8, N=32, seed=73, M=65537)  # rows of the left operand beyond grid.z

@@ -189,6 +189,29 @@ def test_key_tokens_kernel_equals_transpose_then_quantize(oracle, dev, bits, g, 
     assert (to_np(scale[..., : off // g]) == -1).all() and (to_np(scale[..., (off + n) // g:]) == -1).all()
 
 
+def test_key_tokens_kernel_with_more_slices_than_one_grid_dimension_holds(oracle, dev):
+    """kvmix_quant_pack_key_tokens with more than 65535 (batch, head) slices: several launches."""
+    from kvmix_amd import _lib
+
+    L = _lib.load()
+    rng = np.random.default_rng(77)
+    outer, n, D, g, bits = 65539, 32, 16, 32, 4
+    tail = rng.standard_normal((outer, n, D)).astype(np.float16)
+    t = torch.from_numpy(tail).to(dev)
+    code = torch.zeros((outer, D, n // 8), dtype=torch.int32, device=dev)
+    scale = torch.zeros((outer, D, 1), dtype=torch.float16, device=dev)
+    zero = torch.zeros_like(scale)
+    rc = L.kvmix_quant_pack_key_tokens(t.data_ptr(), outer, n, D, t.stride(0), t.stride(1), g, bits, 0,
+                                       _lib.SCALE_RECIPROCAL, code.data_ptr(), code.stride(0), code.stride(1),
+                                       scale.data_ptr(), zero.data_ptr(), scale.stride(0), scale.stride(1),
+                                       torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    want = oracle.quantize_pack_last_dim(np.ascontiguousarray(tail.transpose(0, 2, 1))[None], g, bits)
+    assert same_bits(to_np(code)[None], want[0]) and same_bits(to_np(scale)[None], want[1])
+    assert same_bits(to_np(zero)[None], want[2])
+
+
 def test_scale_matches_torch_division_by_scalar_on_gpu(oracle, dev):
     """The returned scale is what `(max - min) / qmax` gives when torch evaluates that line
     (quantization_cuda.cu:711) on the GPU."""

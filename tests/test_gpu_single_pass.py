@@ -178,3 +178,26 @@ def test_single_pass_with_dense_three_bit_keys(dev):
         out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, 32, 3, 32, v_bits, **fmt)
         out_s, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, 32, 3, 32, v_bits, single_pass=True, **fmt)
         check(out_s, out_f, v_magnitude(vq, v_tail, v_bits))
+
+
+def test_more_rows_than_one_grid_dimension_holds(dev):
+    """Batch x kv heads beyond 65535: the single pass launches a one-dimensional grid, the four-launch step
+    sends its GEMVs out in parts; both must still agree."""
+    from kvmix_amd import ops
+
+    gen = torch.Generator(device=dev).manual_seed(11)
+    B, nkv, rep, k_bits, v_bits, n, tk, tv = 32770, 2, 1, 4, 2, 40, 32, 32
+    q, kq, vq, k_tail, v_tail, kg, mask, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tv, n)
+    out_f, probs = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, **fmt)
+    out_s, none = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, single_pass=True, **fmt)
+    check(out_s, out_f, v_magnitude(vq, v_tail, v_bits))
+    # the last rows against plain attention over the dequantized cache of those rows
+    from helpers import dequantize_torch
+    sl = slice(B - 2, B)
+    kd = dequantize_torch(kq[0][sl], kq[1][sl], kq[2][sl], k_bits, 32).double()          # [2, nkv, D, tk]
+    vd = dequantize_torch(vq[0][sl], vq[1][sl], vq[2][sl], v_bits, 32).double()          # [2, nkv, tv, D]
+    keys = torch.cat([kd.transpose(2, 3), k_tail[sl].double()], 2)
+    vals = torch.cat([vd, v_tail[sl].double()], 2)
+    logits = (q[sl].double() @ keys.transpose(2, 3)) / np.sqrt(128.0)
+    want = torch.softmax(logits, -1) @ vals
+    check(out_s[sl], want, v_magnitude(vq, v_tail, v_bits))
