@@ -42,59 +42,7 @@
 #include <cstdio>
 #include <mutex>
 
-#ifndef KVMIX_COLS3_HEADS_U
-#define KVMIX_COLS3_HEADS_U 4
-#endif
-#ifndef KVMIX_COLS3_HEADS_OCC
-#define KVMIX_COLS3_HEADS_OCC 2
-#endif
-#ifndef KVMIX_MFMA2_OCC4
-#define KVMIX_MFMA2_OCC4 2
-#endif
-#ifndef KVMIX_COLS_MFMA2
-#define KVMIX_COLS_MFMA2 1  // 2/4-bit MHA q.K^T: two elements per lane
-#endif
-#ifndef KVMIX_COLS_MFMA
-#define KVMIX_COLS_MFMA 1  // 1/2/4-bit q.K^T on the matrix cores
-#endif
-#ifndef KVMIX_ROWS_MFMA
-#define KVMIX_ROWS_MFMA 1  // 1/2/4-bit and dense 3-bit p.V on the matrix cores
-#endif
-
-#ifndef KVMIX_HEADS_WAVE_DIV
-#define KVMIX_HEADS_WAVE_DIV 2
-#endif
-#ifndef KVMIX_MFMA_HEADS_OCC
-#define KVMIX_MFMA_HEADS_OCC 2
-#endif
-
-#ifndef KVMIX_MFMA2_MAX_WAVES
-#define KVMIX_MFMA2_MAX_WAVES KVMIX_TARGET_WAVES  // two-element matrix-core q.K^T kernel up to this many tiles
-#endif
-#ifndef KVMIX_MFMA1_MAX_WAVES
-#define KVMIX_MFMA1_MAX_WAVES KVMIX_TARGET_WAVES  // one-element matrix-core q.K^T kernel (one head) below this many tiles
-#endif
-#ifndef KVMIX_COLS_MFMA2_1BIT
-#define KVMIX_COLS_MFMA2_1BIT 1  // 1-bit q.K^T through the two-element kernel too
-#endif
-#ifndef KVMIX_MFMA2_RESIDENT_WAVES
-#define KVMIX_MFMA2_RESIDENT_WAVES 3072  // gemv_cols_mfma2: 3 waves on each of 1024 SIMDs
-#endif
-#ifndef KVMIX_MFMA2_MAX_TPW
-#define KVMIX_MFMA2_MAX_TPW 1  // gemv_cols_mfma2: tiles a wave walks at most (measured: one tile per wave and more waves beats several tiles per wave at every size tried)
-#endif
-#ifndef KVMIX_MFMA2_KSPLIT_WAVES
-#define KVMIX_MFMA2_KSPLIT_WAVES 1536  // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
-#endif
-#ifndef KVMIX_ROWS_CHUNKS_PER_WAVE
-#define KVMIX_ROWS_CHUNKS_PER_WAVE 8  // p.V: chunks a wave should get before more waves per row are used
-#endif
-#ifndef KVMIX_ROWS_SINGLE_BLOCK_CHUNKS
-#define KVMIX_ROWS_SINGLE_BLOCK_CHUNKS 2  // p.V: keep one block per output row up to this many chunks per wave
-#endif
-#ifndef KVMIX_MFMA2_SPLIT4
-#define KVMIX_MFMA2_SPLIT4 1  // gemv_cols_mfma2, 4 bits: two dword loads per row instead of one dwordx2 + lane exchange
-#endif
+// The three switches that profiles/ quotes (the hint compiled out shows the bytes a kernel reads without it):
 #ifndef KVMIX_STREAM_NT
 #define KVMIX_STREAM_NT 1  // non-temporal loads for the packed operands
 #endif
@@ -104,16 +52,28 @@
 #ifndef KVMIX_COLS3_NT_SZ
 #define KVMIX_COLS3_NT_SZ 1  // q.K^T, reference 3-bit words, one head per pass: scales and zeros (as large as the codes) non-temporal
 #endif
-#ifndef KVMIX_COLS_NT_SZ
-#define KVMIX_COLS_NT_SZ 0  // q.K^T kernels: scales and zeros non-temporal
-#endif
-#ifndef KVMIX_TARGET_WAVES
-#define KVMIX_TARGET_WAVES 4096  // 16 waves on each of 256 CUs
-#endif
 
 namespace kvmix {
 
 constexpr int kMaxDevices = 64;  // per-device set-up state is kept for device ordinals below this
+
+// Measured constants of the dispatch (MI355X: 256 CUs x 4 SIMDs).  tests/test_gemv_plan_cpu.py pins the kernel
+// each benchmark shape ends up with.
+constexpr int kTargetWaves = 4096;          // 16 waves on each of 256 CUs
+constexpr int kCols3HeadsU = 4;             // gemv_cols3, four heads per pass: rows in flight per lane
+constexpr int kCols3U = 8;                  // gemv_cols3, one head per pass: rows in flight per lane
+constexpr int kCols3HeadsOcc = 2;           // waves per SIMD the compiler may plan for: gemv_cols3, four heads
+constexpr int kMfmaHeadsOcc = 2;            // ... gemv_rows_mfma / gemv_cols_mfma, four heads
+constexpr int kMfma2Occ = 2;                // ... gemv_cols_mfma2 (at least; it comes out at three)
+constexpr int kHeadsWaveDiv = 2;            // p.V, four heads per pass: half as many waves wanted
+constexpr int kMfma2MaxWaves = kTargetWaves;    // two-element matrix-core q.K^T kernel up to this many tiles
+constexpr int kMfma1MaxWaves = kTargetWaves;    // one-element matrix-core q.K^T kernel (one head) below this many tiles
+constexpr int kMfma2ResidentWaves = 3072;   // gemv_cols_mfma2: 3 waves on each of 1024 SIMDs
+constexpr int kMfma2KsplitWaves = 1536;     // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
+constexpr int kRowsChunksPerWave = 8;       // p.V: chunks a wave should get before more waves per row are used
+constexpr int kRowsSingleBlockChunks = 2;   // p.V: keep one block per output row up to this many chunks per wave
+constexpr int kCols3WideWaves = 4096;       // gemv_cols3: widest tiles (one wave each) from this many of them on
+constexpr int kCols3MinWaves = 2048;        // gemv_cols3: 128-word one-wave tiles from this many of them on
 
 struct GemvArgs {
     const __half *x;
@@ -564,8 +524,8 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
             const int row = idx / SEGS, seg = idx % SEGS;
             const int rowc = kc + (row < rows ? row : rows - 1);
             const uint32_t off = (uint32_t)rowc * s_rs + (uint32_t)(t0 + seg * 8);
-            s8[it] = ld_stream<Half8, KVMIX_COLS_NT_SZ>(sp + off);
-            z8[it] = ld_stream<Half8, KVMIX_COLS_NT_SZ>(zp + off);
+            s8[it] = ld_stream<Half8, false>(sp + off);
+            z8[it] = ld_stream<Half8, false>(zp + off);
         }
         uint16_t xh[(KC + kWave - 1) / kWave];
 #pragma unroll
@@ -662,7 +622,7 @@ __device__ __forceinline__ constexpr float cols3_out_scale(int i)
 }
 
 template <int RQ, int UPL, int U, int NREP>
-__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_COLS3_HEADS_OCC : 3)))
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(NREP > 1 ? kCols3HeadsOcc : 3)))
 gemv_cols3(GemvArgs a)
 {
     constexpr int VALS = 11;
@@ -1177,7 +1137,7 @@ constexpr int kRowsMfmaWaves = 16;  // waves per block at most (register budget 
 
 template <int BITS, int NREP, int DEPTH>
 __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWaves))
-    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_MFMA_HEADS_OCC : 4))) gemv_rows_mfma(GemvArgs a)
+    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? kMfmaHeadsOcc : 4))) gemv_rows_mfma(GemvArgs a)
 {
     // BITS = 30: dense 3-bit stream, a lane's 8 codes are 3 bytes
     using Elem = typename CodeElem<BITS>::type;
@@ -1470,7 +1430,7 @@ constexpr int kColsMfmaTile = 16 * 33 * 4;  // bf16 elements: 16 rows of 33 four
 
 template <int BITS, int NREP>
 __global__ void __launch_bounds__(64 * kColsWaves)
-    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? KVMIX_MFMA_HEADS_OCC : 4))) gemv_cols_mfma(GemvArgs a)
+    __attribute__((amdgpu_waves_per_eu(NREP > 1 ? kMfmaHeadsOcc : 4))) gemv_cols_mfma(GemvArgs a)
 {
     using Elem = typename CodeElem<BITS>::type;
     constexpr int CH = 32;             // rows per chunk
@@ -1547,8 +1507,8 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     auto load_small = [&](int it) {
         const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
         const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
-        s8 = ld_stream<Half8, KVMIX_COLS_NT_SZ>(sbase + off);
-        z8 = ld_stream<Half8, KVMIX_COLS_NT_SZ>(zbase + off);
+        s8 = ld_stream<Half8, false>(sbase + off);
+        z8 = ld_stream<Half8, false>(zbase + off);
 #pragma unroll
         for (int h = 0; h < NREP; h++) xh[h] = xp[h * a.x_bs + d];
     };
@@ -1666,21 +1626,24 @@ __global__ void __launch_bounds__(64 * kColsWaves)
 }
 
 // ---------------------------------------------------------------------------------------
-// gemv_cols_mfma2<BITS>   q.K^T, 4- or 2-bit codes, one query head per kv head: gemv_cols_mfma with
-// TWO 8-code elements per lane, so that a wave reads twice as many contiguous bytes of a row per
-// load instruction (512 for 4 bits: measured, the length of the contiguous pieces is what bounds
-// the streaming rate of this shape).  Tile = 128 elements = 1024 codes = 32 groups.
-//   A lane loads elements 2l and 2l+1 of every row (one dwordx2 / dword).  A quad of lanes then
-//   holds two quantization groups: lanes 0,1 the four elements of the first, lanes 2,3 those of
-//   the second.  Two MFMA sets per quad: set 0 works on the first group (lanes 2,3 fetch the
-//   second elements of lanes 0,1 with a DPP quad permute), set 1 on the second.  Per set the
-//   scheme is gemv_cols_mfma's: k = 4 channel rows, three exact bf16 parts of x*scale*2^90 as A.
-//   Rows are walked in chunks of 16 (4 k-steps); the chunk's [16][32] scales and zeros are one
+// gemv_cols_mfma2<BITS, NTC>   q.K^T, 4-, 2- or 1-bit codes, one query head per kv head: gemv_cols_mfma
+// with TWO 8-code elements per lane, so that a wave reads twice as many contiguous bytes of a row
+// (512 for 4 bits: measured, the length of the contiguous pieces is what bounds the streaming rate of
+// this shape).  Tile = 128 elements = 1024 codes = 32 groups, one tile per wave.
+//   2 bits, 1 bit: a lane loads elements 2l and 2l+1 of every row (one dword / ushort).  A quad of lanes
+//   then holds two quantization groups: lanes 0,1 the four elements of the first, lanes 2,3 those of
+//   the second.  Two MFMA sets per quad: set 0 works on the first group (lanes 2,3 fetch the second
+//   elements of lanes 0,1 with a DPP quad permute), set 1 on the second.
+//   4 bits: a lane's two dwords are element `lane` of each 256-byte half of the row piece; a quad then
+//   holds all four elements of ONE group in either half, set s works on half s with every lane's own
+//   register and nothing moves between lanes.
+//   Per set the scheme is gemv_cols_mfma's: k = 4 channel rows, three exact bf16 parts of x*scale*2^90
+//   as A.  Rows are walked in chunks of 16 (4 k-steps); the chunk's [16][32] scales and zeros are one
 //   128-bit load per lane each (64-byte pieces per row).  LDS tile: per (k-step, set) a row of
-//   64 eight-byte cells in four sub-rows at a pitch of 17 cells, rows at a pitch of 74: staging
-//   stores and operand reads are bank-conflict free.
-//   block = (64, 2..4) waves on neighbouring tiles, a wave walks `splits` tiles;
-//   grid = (tiles/(waves*splits), samples, M), XCD-swizzled.
+//   64 eight-byte cells in four sub-rows at a pitch of 17 cells, rows at a pitch of 74.
+//   Loads go through buffer descriptors (row offsets in SGPRs); NTC: codes with the non-temporal hint.
+//   block = (64, 2..4) waves on neighbouring tiles, or `ksplit` waves on ONE tile, each with a share
+//   of the K rows (small launches); grid = (tiles/waves, samples, M), XCD-swizzled.
 // ---------------------------------------------------------------------------------------
 constexpr int kColsMfma2Row = 74 * 4;                   // bf16 elements per (k-step, set) row
 constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets
@@ -1688,7 +1651,7 @@ constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets
 // NTC: the codes are loaded non-temporally (the host asks for it while the launch is no more than a few rounds of
 // resident waves: measured faster up to 8k waves, slower at 16k, where rows of neighbouring tiles meet in the L2)
 template <int BITS, bool NTC>
-__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(KVMIX_MFMA2_OCC4)))
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
 gemv_cols_mfma2(GemvArgs a)
 {
     static_assert(BITS == 4 || BITS == 2 || BITS == 1, "two elements per lane: a dwordx2, a dword or a ushort");
@@ -1703,7 +1666,7 @@ gemv_cols_mfma2(GemvArgs a)
     // loads), so that a quad of lanes holds the four elements of ONE group in either half: set s works on
     // half s with every lane's own register, no exchange between lanes.  Group g of the tile is then set
     // g / 16, quad g % 16.  (2 bits, 1 bit: neighbouring elements, sets 0 / 1 = the quad's first / second group.)
-    constexpr bool SPLIT = BITS == 4 && KVMIX_MFMA2_SPLIT4;
+    constexpr bool SPLIT = BITS == 4;
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
@@ -1717,13 +1680,12 @@ gemv_cols_mfma2(GemvArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int K = (int)a.K;
     const int ngroups = (int)(a.N / 32);
-    const int tpw = a.splits;
-    // ks > 1 (small problems, tpw == 1): ks neighbouring waves share a tile and slice its K rows
+    // ks > 1 (small problems): ks neighbouring waves share a tile and slice its K rows
     // chunk-wise, which shortens each wave's chain of dependent loads; their sums meet in LDS
     const int ks = a.ksplit;
     const int slice = wy % ks;
     const int ntw = nw / ks;            // tiles a block works on at a time
-    const int tile0 = (int)bx * tpw * ntw + wy / ks;
+    const int tile0 = (int)bx * ntw + wy / ks;   // one tile per wave
     if (tile0 * TG >= ngroups) {
         if (ks > 1) __syncthreads();    // (the one block barrier of finish_tile)
         return;
@@ -1732,7 +1694,7 @@ gemv_cols_mfma2(GemvArgs a)
     const int nch_slice = (nch_all + ks - 1) / ks;
     const int ch0 = slice * nch_slice;  // this wave's chunks: [ch0, ch0 + nch)
     const int nch = ch0 >= nch_all ? 0 : (ch0 + nch_slice <= nch_all ? nch_slice : nch_all - ch0);
-    const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
+    const int items = nch;
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
     // buffer descriptors of this (batch, kv-head) slice; a lane's two elements are 2 * BITS bytes
@@ -1769,24 +1731,16 @@ gemv_cols_mfma2(GemvArgs a)
     uint16_t xh;
     uint32_t w[KB][4][WL];
 
-    // (with one tile per wave -- the only setting in use -- an item is a chunk: no division per load)
-    constexpr bool kOneTile = KVMIX_MFMA2_MAX_TPW == 1;
+    // the last tile of a row is moved back to end at N
     const int g_first = tile0 * TG + TG <= ngroups ? tile0 * TG : ngroups - TG;
-    auto tile_g0 = [&](int it) {
-        if constexpr (kOneTile) return g_first;
-        const int g = (tile0 + (nch > 0 ? it / nch : 0) * ntw) * TG;
-        return g + TG <= ngroups ? g : ngroups - TG;
-    };
-    auto chunk_k0 = [&](int it) {
-        if constexpr (kOneTile) return (ch0 + it) * CH;
-        return (ch0 + (nch > 0 ? it % nch : 0)) * CH;
-    };
+    auto tile_g0 = [&](int) { return g_first; };
+    auto chunk_k0 = [&](int it) { return (ch0 + it) * CH; };
     auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
     auto load_small = [&](int it) {
         const uint32_t d0 = (uint32_t)chunk_base(chunk_k0(it));
         const uint32_t off = 2u * (d0 * s_rs + (uint32_t)tile_g0(it));  // bytes, the same for every lane
-        s8 = ld_buffer<Half8, KVMIX_COLS_NT_SZ>(srsrc, s_lane, off);
-        z8 = ld_buffer<Half8, KVMIX_COLS_NT_SZ>(zrsrc, s_lane, off);
+        s8 = ld_buffer<Half8, false>(srsrc, s_lane, off);
+        z8 = ld_buffer<Half8, false>(zrsrc, s_lane, off);
         xh = xp[d0 + (uint32_t)srow];
     };
     auto load_codes = [&](int it, int t) {
@@ -1844,11 +1798,6 @@ gemv_cols_mfma2(GemvArgs a)
             for (int k = 0; k < 4; k++) {
                 if constexpr (SPLIT) {
                     src[k] = w[t][k][s];
-                } else if constexpr (BITS == 4) {
-                    const uint32_t other = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][1], 0x44, 0xf, 0xf, false)
-                                                  : __builtin_amdgcn_mov_dpp(w[t][k][1], 0xEE, 0xf, 0xf, false);
-                    const bool own = s == 0 ? j4 < 2 : j4 >= 2;
-                    src[k] = own ? w[t][k][0] : other;
                 } else {
                     src[k] = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][0], 0x44, 0xf, 0xf, false)
                                     : __builtin_amdgcn_mov_dpp(w[t][k][0], 0xEE, 0xf, 0xf, false);
@@ -1963,8 +1912,8 @@ gemv_cols_mfma2(GemvArgs a)
             __builtin_amdgcn_sched_barrier(0);
         }
         wave_lds_fence();  // the next chunk overwrites the tile
-        if (kOneTile ? it == items - 1 : it % nch == nch - 1) finish_tile(it);
     }
+    finish_tile(items - 1);
 }
 
 __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
@@ -2069,8 +2018,6 @@ __global__ void __launch_bounds__(GenericCfg<MODE>::THREADS) gemv_generic(GemvAr
 
 // --------------------------- host side ---------------------------
 
-constexpr int64_t kTargetWaves = KVMIX_TARGET_WAVES;
-
 // kvmix_quantized_gemv_plan: the dispatch below runs as usual, but every launch is recorded instead of made
 static thread_local kvmix_gemv_plan_t *t_plan = nullptr;
 
@@ -2110,7 +2057,7 @@ struct RowsPlan {
 // they get half as many waves, again one resident round)
 static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_waves)
 {
-    const int64_t target = max_waves <= kRowsHeadsWaves ? kTargetWaves / KVMIX_HEADS_WAVE_DIV : kTargetWaves;
+    const int64_t target = max_waves <= kRowsHeadsWaves ? kTargetWaves / kHeadsWaveDiv : kTargetWaves;
     RowsPlan p{4, 1, K > 0 ? K : 1};
     if (!rows_shape_ok(N) || batch_rows <= 0 || K <= 0) return p;
     const int64_t chunk = 512 / (N / 32);            // rows one wave takes per step
@@ -2121,7 +2068,7 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
     // chunks per wave, fewer and longer-lived waves are faster (measured at B = 8, T = 8k: 16 -> 8
     // waves per row, 2-bit p.V 22.2 -> 20.3 us), as long as two waves per SIMD remain
     {
-        const int64_t by_chunks = (chunks + KVMIX_ROWS_CHUNKS_PER_WAVE - 1) / KVMIX_ROWS_CHUNKS_PER_WAVE;
+        const int64_t by_chunks = (chunks + kRowsChunksPerWave - 1) / kRowsChunksPerWave;
         const int64_t by_waves = (target / 2 + batch_rows - 1) / batch_rows;
         const int64_t lean = by_chunks > by_waves ? by_chunks : by_waves;
         if (lean < want) want = lean;
@@ -2131,8 +2078,8 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
     if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
     int64_t splits = (want + waves - 1) / waves;
     // a second block per output row brings the reduce_splits launch with it: not worth it while
-    // one block's waves get at most KVMIX_ROWS_SINGLE_BLOCK_CHUNKS chunks each
-    if (splits > 1 && chunks <= waves * KVMIX_ROWS_SINGLE_BLOCK_CHUNKS) splits = 1;
+    // one block's waves get at most kRowsSingleBlockChunks chunks each
+    if (splits > 1 && chunks <= waves * kRowsSingleBlockChunks) splits = 1;
     if (splits > 64) splits = 64;
     int64_t rps = (K + splits - 1) / splits;
     rps = (rps + chunk - 1) / chunk * chunk;
@@ -2150,7 +2097,7 @@ static int heads_per_block(int heads_per_kv) { return heads_per_kv % 4 == 0 ? 4 
 // (gemv_rows_mfma: N = 128, dense code rows, at least one whole 128-row chunk)
 static bool rows_use_mfma(int mode, int64_t N, int64_t K, int64_t c_rs)
 {
-    return KVMIX_ROWS_MFMA && (mode == 1 || mode == 2 || mode == 4 || mode == 30) && N == 128 && K >= 128 &&
+    return (mode == 1 || mode == 2 || mode == 4 || mode == 30) && N == 128 && K >= 128 &&
            c_rs == N * (mode == 30 ? 3 : mode) / 32;
 }
 static int rows_max_waves(bool mfma, int nrep)
@@ -2211,10 +2158,6 @@ static void launch_rows(GemvArgs &a, int64_t samples, hipStream_t st)
         launch_rows_n<MODE, 1>(a, samples, st);
 }
 
-#ifndef KVMIX_COLS_RQ
-#define KVMIX_COLS_RQ 0  // 0 = choose by problem size
-#endif
-
 // waves per block for a kernel whose waves each take one of `slots` tiles of an output row:
 // the count (2..4) that leaves the fewest launched waves without a tile
 static int pick_waves_per_block(int64_t slots)
@@ -2258,18 +2201,6 @@ static int64_t cols_min_units()
     return MODE == 3 ? 64 : 16 * ColsUpl<MODE>::value;
 }
 
-#ifndef KVMIX_COLS3_KSLICE4
-#define KVMIX_COLS3_KSLICE4 1
-#endif
-#ifndef KVMIX_COLS3_WIDE_WAVES
-#define KVMIX_COLS3_WIDE_WAVES 4096
-#endif
-#ifndef KVMIX_COLS3_MIN_WAVES
-#define KVMIX_COLS3_MIN_WAVES 2048
-#endif
-#ifndef KVMIX_COLS3_U
-#define KVMIX_COLS3_U 8
-#endif
 
 template <int RQ, int UPL, int NREP>
 static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int ks = 1)
@@ -2277,7 +2208,7 @@ static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int k
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / 11;
     const int64_t tiles = (units + TU - 1) / TU;
-    constexpr int U = NREP > 1 ? KVMIX_COLS3_HEADS_U : KVMIX_COLS3_U;  // rows in flight per lane
+    constexpr int U = NREP > 1 ? kCols3HeadsU : kCols3U;  // rows in flight per lane
     a.ksplit = ks;
     if (ks > 1) {
         // one tile per block: its ks waves slice K and leave their sums behind the x vector in LDS
@@ -2295,7 +2226,7 @@ static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int k
 // (gemv_cols_mfma: whole 512-code tiles, at least one whole 32-row chunk)
 static bool cols_use_mfma(int mode, int64_t N, int64_t K)
 {
-    return KVMIX_COLS_MFMA && (mode == 1 || mode == 2 || mode == 4) && N >= 512 && K >= 32;
+    return (mode == 1 || mode == 2 || mode == 4) && N >= 512 && K >= 32;
 }
 
 template <int BITS, int NREP>
@@ -2321,14 +2252,11 @@ static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
 {
     const int64_t tiles = (a.N / 32 + 31) / 32;
     const int64_t batch = samples * a.M;
-    // tiles per wave: as many as it takes for ONE round of resident waves (three per SIMD with this kernel's
-    // registers) to cover the problem -- a partial second round runs with most of the chip idle
-    int64_t tpw = (batch * tiles + KVMIX_MFMA2_RESIDENT_WAVES - 1) / KVMIX_MFMA2_RESIDENT_WAVES;
-    tpw = tpw < 1 ? 1 : (tpw > KVMIX_MFMA2_MAX_TPW ? KVMIX_MFMA2_MAX_TPW : tpw);
-    // few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
+    // one tile per wave (several tiles per wave, so that one round of resident waves covers the problem, were
+    // measured slower at every size).  Few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
     const int64_t chunks = (a.K + 15) / 16;
     int ks = 1;
-    while (ks < kColsWaves && batch * tiles * ks * 2 <= KVMIX_MFMA2_KSPLIT_WAVES && chunks >= ks * 4) ks *= 2;
+    while (ks < kColsWaves && batch * tiles * ks * 2 <= kMfma2KsplitWaves && chunks >= ks * 4) ks *= 2;
     a.ksplit = ks;
     if (ks > 1) {
         a.splits = 1;
@@ -2337,10 +2265,9 @@ static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
         KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, ks), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
         return;
     }
-    const int64_t slots = (tiles + tpw - 1) / tpw;
-    const int wpb = pick_waves_per_block(slots);
-    a.splits = (int)tpw;
-    const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
+    const int wpb = pick_waves_per_block(tiles);
+    a.splits = 1;
+    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
     const size_t lds = (size_t)wpb * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
     KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
 }
@@ -2351,7 +2278,7 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     // non-temporal code loads: 2 and 4 bits (a wave's 1-bit row piece is 128 bytes and shares its cache lines
     // with the neighbours'), and only while the launch is at most three rounds of resident waves
     const int64_t tiles = (a.N / 32 + 31) / 32;
-    if (BITS >= 2 && samples * a.M * tiles <= 3 * (int64_t)KVMIX_MFMA2_RESIDENT_WAVES)
+    if (BITS >= 2 && samples * a.M * tiles <= 3 * (int64_t)kMfma2ResidentWaves)
         launch_cols_mfma2_nt<BITS, true>(a, samples, st);
     else
         launch_cols_mfma2_nt<BITS, false>(a, samples, st);
@@ -2370,10 +2297,10 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // wave, is ahead up to one resident round of waves: B = 16, T = 4k: 19.6 against 22.7 us);
         // there, and for rows of up to two of gemv_cols' tiles, it replaces gemv_cols (B = 64, T = 4k:
         // 110 -> 87 us; at T = 8k gemv_cols stays ahead)
-        const bool one_bit_ok = MODE != 1 || (KVMIX_COLS_MFMA2_1BIT && a.N <= 2 * 2048 &&
-                                              samples * a.M * ((a.N / 32 + 31) / 32) >= (int64_t)KVMIX_MFMA1_MAX_WAVES);
-        if (KVMIX_COLS_MFMA2 && one_bit_ok && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
-            (MODE == 1 || samples * a.M * tiles2 <= (int64_t)KVMIX_MFMA2_MAX_WAVES || a.N <= 2 * 2048)) {
+        const bool one_bit_ok = MODE != 1 || (a.N <= 2 * 2048 &&
+                                              samples * a.M * ((a.N / 32 + 31) / 32) >= (int64_t)kMfma1MaxWaves);
+        if (one_bit_ok && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
+            (MODE == 1 || samples * a.M * tiles2 <= (int64_t)kMfma2MaxWaves || a.N <= 2 * 2048)) {
             launch_cols_mfma2<MODE>(a, samples, st);
             return;
         }
@@ -2389,7 +2316,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
                 launch_cols_mfma<MODE, 4>(a, samples, st);
                 return;
             }
-            if (batch * ((units + 31) / 32) < (int64_t)KVMIX_MFMA1_MAX_WAVES) {
+            if (batch * ((units + 31) / 32) < (int64_t)kMfma1MaxWaves) {
                 launch_cols_mfma<MODE, 1>(a, samples, st);
                 return;
             }
@@ -2402,7 +2329,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
         if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
-        else if (KVMIX_COLS3_KSLICE4 && units >= 128 && 2 * ((units + 127) / 128) * 128 <= 3 * units && a.K >= 64 &&
+        else if (units >= 128 && 2 * ((units + 127) / 128) * 128 <= 3 * units && a.K >= 64 &&
                  a.K <= 4096 && (waves(128) * 4 <= 1024 || waves(128) * 4 >= 2304))
             // tiles of 128 words (512 bytes of codes per row), each shared by four waves that slice K: measured
             // ahead of the one-wave-per-tile configurations below (T = 2.3k..32k, B = 1..128: by 2..35 %) with
@@ -2410,9 +2337,9 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
             // between one and two waves per SIMD (measured behind there), nor where the last tile, moved back
             // to end at N, would mostly repeat its neighbour.
             launch_cols3_cfg<2, 4, 1>(a, samples, st, 4);
-        else if (units >= 256 && waves(256) >= KVMIX_COLS3_WIDE_WAVES)
+        else if (units >= 256 && waves(256) >= kCols3WideWaves)
             launch_cols3_cfg<1, 4, 1>(a, samples, st);
-        else if (units >= 128 && waves(128) >= KVMIX_COLS3_MIN_WAVES)
+        else if (units >= 128 && waves(128) >= kCols3MinWaves)
             launch_cols3_cfg<2, 4, 1>(a, samples, st);
         else
             launch_cols3_cfg<2, 2, 1>(a, samples, st);
@@ -2423,15 +2350,11 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
     constexpr int UPL = ColsUpl<MODE>::value;
     const int64_t units = a.N / VALS;
     const int64_t batch = samples * a.M;
-    int rq = KVMIX_COLS_RQ;
-    if (rq == 0) {
-        if (batch * ((units + 64 * UPL - 1) / (64 * UPL)) >= kTargetWaves)
-            rq = 1;
-        else if (batch * ((units + 32 * UPL - 1) / (32 * UPL)) >= kTargetWaves)
-            rq = 2;
-        else
-            rq = 4;
-    }
+    int rq = 4;
+    if (batch * ((units + 64 * UPL - 1) / (64 * UPL)) >= kTargetWaves)
+        rq = 1;
+    else if (batch * ((units + 32 * UPL - 1) / (32 * UPL)) >= kTargetWaves)
+        rq = 2;
     while (rq < 4 && units < (64 / rq) * UPL) rq *= 2;  // the tile must fit into N
     if (rq == 4)
         launch_cols_cfg<MODE, 4, UPL>(a, samples, st);
