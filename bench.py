@@ -866,6 +866,11 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
             result["hf_generate_config4"] = hf_generate_extra(torch, dev)
         except Exception as ex:
             result["hf_generate_config4"] = {"error": f"{type(ex).__name__}: {ex}"}
+        torch.cuda.empty_cache()
+        try:  # the same at batch 16, where the transformers host loop no longer hides the cache
+            result["hf_generate_config4_batch16"] = hf_generate_extra(torch, dev, batch=16)
+        except Exception as ex:
+            result["hf_generate_config4_batch16"] = {"error": f"{type(ex).__name__}: {ex}"}
     print(json.dumps(result))
 
 
