@@ -1173,6 +1173,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
     // dense 3-bit: a group is three aligned words; lane j of the group's four loads word
     // min(j, 2), and its 24 bits [24j, 24j+24) are cut out of two neighbours' words in compute()
+    // (a dword load at byte 3j instead -- no exchange between lanes -- was measured slower: 33 against 28 us)
     const uint8_t *cp = reinterpret_cast<const uint8_t *>(a.code + kv * a.c_bs) +
                         (BITS == 30 ? (wi / 4) * 12 + (wi % 4 < 2 ? wi % 4 : 2) * 4 : wi * EB);
     [[maybe_unused]] const uint32_t sh3 = (uint32_t)(24 * (wi % 4)) % 32u;
@@ -1269,22 +1270,32 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         for (int q = 0; q < NM; q++)
             av[q] = *reinterpret_cast<const bf16x4_t *>(atile + q * AT + cell(t, lane));
         if constexpr (BITS == 30) {
-            // 24-bit stream per row: codes (2m, 2m+1) lie in the 8-bit window at bit 6m
-            uint32_t v[4];
+            // the lane's 24 bits hold code i at bit 3i.  Codes 0,1 are bits 0..5 of byte 0 and codes 6,7 bits
+            // 2..7 of byte 2; codes 2,3 and 4,5 are bits 2..7 of byte 0 and bits 0..5 of byte 1 of the stream
+            // shifted right by 4: one shift per row, and a field at bit offset o simply counts 2^o-fold
+            // (offsets by code: 0 3 2 5 0 3 2 5).
+            uint32_t v[4], u[4];
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 // words (0,0,1,2) and (0,1,2,2) of the group for lanes 0..3, funnel-shifted
                 const uint32_t lo = __builtin_amdgcn_mov_dpp(w[d][t][k], 0x90, 0xf, 0xf, false);
                 const uint32_t hi = __builtin_amdgcn_mov_dpp(w[d][t][k], 0xA4, 0xf, 0xf, false);
                 v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
+                u[k] = v[k] >> 4;
             }
 #pragma unroll
             for (int mm = 0; mm < 4; mm++) {
-                const uint32_t t01 = __builtin_amdgcn_perm(v[1] >> (6 * mm), v[0] >> (6 * mm), 0x0c040c00u);
-                const uint32_t t23 = __builtin_amdgcn_perm(v[3] >> (6 * mm), v[2] >> (6 * mm), 0x0c040c00u);
+                // byte of the source register that holds the pair: v bytes 0 / 2, u bytes 0 / 1
+                const bool from_u = mm == 1 || mm == 2;
+                const uint32_t b = from_u ? (uint32_t)(mm - 1) : (mm == 0 ? 0u : 2u);
+                const uint32_t sel = 0x0c000c00u | b | ((4u + b) << 16);
+                const uint32_t *src = from_u ? u : v;
+                const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
+                const int o0 = mm % 2 == 0 ? 0 : 2;  // bit offset of the pair's first field in its byte
 #pragma unroll
                 for (int f = 0; f < 2; f++) {
-                    const uint32_t mask = 0x00070007u << (3 * f);
+                    const uint32_t mask = 0x00070007u << (o0 + 3 * f);
                     const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
 #pragma unroll
                     for (int q = 0; q < NM; q++)
@@ -1378,7 +1389,9 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         for (int p = 0; p < NPOS; p++) {
             const float sum = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
                               acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
-            flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - FB * (p % FPB)) << 23);
+            // (bit offset of code p's field in its byte: dense 3-bit 0 3 2 5 0 3 2 5, else FB * (p % FPB))
+            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
+            flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
         }
     }
     __syncthreads();  // every wave is done with its A tile: the space becomes `red`
