@@ -42,7 +42,7 @@
 #include <cstdio>
 #include <mutex>
 
-// The three switches that profiles/ quotes (the hint compiled out shows the bytes a kernel reads without it):
+// Switches kept for measurement: with the hint compiled out the HBM counters show the bytes a kernel reads without it.
 #ifndef KVMIX_STREAM_NT
 #define KVMIX_STREAM_NT 1  // non-temporal loads for the packed operands
 #endif
