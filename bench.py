@@ -420,7 +420,8 @@ def stream_ceiling_extra(torch, _lib, lib, dev):
       rows       512-byte row pieces down 128 rows of a [512][128][4032 B] array (the q.K^T 4-bit pattern)
       rows_side  the same plus the two side arrays read as the scales and zeros are (what a 4-bit q.K^T
                  launch at B=16, T=8192 reads), blocks in XCD-aware order
-    each with plain and with non-temporal loads."""
+    each with plain and with non-temporal loads; rows_side also in the kernels' order of issue for three row
+    lengths."""
     GiB = 1 << 30
     buf = torch.empty(4 * GiB, dtype=torch.uint8, device=dev)
     buf.view(torch.int64).random_()
@@ -454,6 +455,13 @@ def stream_ceiling_extra(torch, _lib, lib, dev):
         res[f"slab_{name}"] = run(0, slab, 0, 1024, 8, 16, 8, flags, slab * 1024)
         res[f"rows_{name}"] = run(1, 128, 4032, 512, 4, 8, 16, flags, 512 * 128 * 4032)
         res[f"rows_side_{name}"] = run(2, 128, 4032, 512, 4, 8, 16, flags | XCD, 512 * 128 * (4032 + 2 * 504))
+    # the same bytes with the loads issued in the kernels' rotating order (four rows consumed, four refilled)
+    # instead of in bursts, for three row lengths: 4032 bytes is a 4-bit key row at T = 8192, 2016 a 2-bit one,
+    # 8064 a 4-bit one at T = 16384 -- the shorter the rows, the lower the ceiling of this pattern
+    ROT = 8
+    for row, count in ((2016, 1024), (4032, 512), (8064, 256)):
+        res[f"rows_side_nontemporal_kernel_order_row{row}"] = run(2, 128, row, count, 4, 8, 16, NT | XCD | ROT,
+                                                                 count * 128 * (row + 2 * (row // 8)))
     del buf
     torch.cuda.empty_cache()
     return res
