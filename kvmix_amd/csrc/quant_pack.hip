@@ -203,8 +203,10 @@ __device__ __forceinline__ void rows_g32_f16_body(const QuantArgs &a, int64_t gr
         const float scale = range / (float)qmax;
         const float rcp = quantize_rcp(scale);
         uint32_t piece = 0;  // this lane's 8 codes, 8*BITS bits
+        uint32_t q8[8];
+        quantize_codes<8>(v, mn, scale, rcp, [](int) { return qmax; }, q8);
 #pragma unroll
-        for (int t = 0; t < 8; t++) piece |= quantize_code(v[t], mn, scale, rcp, qmax) << (t * BITS);
+        for (int t = 0; t < 8; t++) piece |= q8[t] << (t * BITS);
 
         const bool act = active[p];
         uint32_t *cw = a.code + o[p] * a.c_os + i[p] * a.c_is + gr[p] * BITS;  // BITS words per group of 32
@@ -301,11 +303,16 @@ __device__ __forceinline__ void rows_g32_f16_stream_body(const QuantArgs &a, uin
 #pragma unroll
         for (int t = 0; t < BITS; t++) w[t] = 0;
 #pragma unroll
-        for (int t = 0; t < 32; t++) {
-            const uint32_t q = quantize_code(v[t], mn, scale, rcp, qmax);
-            const int bit = t * BITS;
-            w[bit >> 5] |= q << (bit & 31);
-            if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+        for (int t0 = 0; t0 < 32; t0 += 8) {
+            uint32_t q8[8];
+            quantize_codes<8>(v + t0, mn, scale, rcp, [](int) { return qmax; }, q8);
+#pragma unroll
+            for (int t = t0; t < t0 + 8; t++) {
+                const uint32_t q = q8[t - t0];
+                const int bit = t * BITS;
+                w[bit >> 5] |= q << (bit & 31);
+                if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+            }
         }
         if (active[p]) {
             uint32_t *cw = a.code + o[p] * a.c_os + i[p] * a.c_is + (int64_t)gr[p] * BITS;
@@ -369,9 +376,11 @@ __global__ void __launch_bounds__(256) quant_rows_ref3_f16(QuantArgs a, uint32_t
         const float scale = range / 7.0f;
         const float rcp = quantize_rcp(scale);
         uint32_t word = 0;
+        uint32_t q11[11];
+        quantize_codes<11>(v, mn, scale, rcp, [](int t) { return t < 10 || WRAP ? 7 : 3; }, q11);
 #pragma unroll
-        for (int t = 0; t < 10; t++) word |= quantize_code(v[t], mn, scale, rcp, 7) << (3 * t);
-        word |= (quantize_code(v[10], mn, scale, rcp, WRAP ? 7 : 3) & 3u) << 30;
+        for (int t = 0; t < 10; t++) word |= q11[t] << (3 * t);
+        word |= (q11[10] & 3u) << 30;
         if (active[p]) {
             a.code[o[p] * a.c_os + i[p] * a.c_is + wr[p]] = word;
             ((__half *)a.scale)[o[p] * a.s_os + i[p] * a.s_is + wr[p]] =
@@ -419,16 +428,23 @@ __device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float
     uint32_t w[WORDS];
 #pragma unroll
     for (int t = 0; t < WORDS; t++) w[t] = 0;
+    if constexpr (MODE == 3) {
+        uint32_t q11[11];
+        quantize_codes<11>(v, mn, scale, rcp, [](int t) { return t < 10 ? 7 : 3; }, q11);
 #pragma unroll
-    for (int t = 0; t < G; t++) {
-        if (MODE == 3) {
-            uint32_t q = quantize_code(v[t], mn, scale, rcp, t < 10 ? 7 : 3);
-            w[0] |= q << (t < 10 ? 3 * t : 30);
-        } else {
-            uint32_t q = quantize_code(v[t], mn, scale, rcp, qmax);
-            const int bit = t * BITS;
-            w[bit >> 5] |= q << (bit & 31);
-            if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+        for (int t = 0; t < 11; t++) w[0] |= q11[t] << (t < 10 ? 3 * t : 30);
+    } else {
+#pragma unroll
+        for (int t0 = 0; t0 < G; t0 += 8) {
+            uint32_t q8[8];
+            quantize_codes<8>(v + t0, mn, scale, rcp, [](int) { return qmax; }, q8);
+#pragma unroll
+            for (int t = t0; t < t0 + 8; t++) {
+                const uint32_t q = q8[t - t0];
+                const int bit = t * BITS;
+                w[bit >> 5] |= q << (bit & 31);
+                if ((bit & 31) + BITS > 32) w[(bit >> 5) + 1] |= q >> (32 - (bit & 31));
+            }
         }
     }
     uint32_t *cw = a.code + o * a.c_os + d * a.c_is + gi * WORDS;
