@@ -240,54 +240,81 @@ def cpu_baseline(layers, kbits, vbits, B, H, D, T, R, sample_layers=None, budget
                       f"C oracle with OpenMP on {int(O.num_threads())} threads"}
 
 
+def mha_pair_times(torch, lib, dev, stream, B, Tq, bits, nsets=3, warm=30, iters=100, H=32, D=128):
+    """q.K^T and p.V of one MHA shape (B x H slices, Tq quantized tokens, `bits`-bit codes in groups of 32):
+    event-timed eager launches over `nsets` buffer sets taken in turn, so that the Infinity Cache cannot
+    serve them."""
+    sets = []
+    for _ in range(nsets):
+        kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+        ks = torch.rand(B, H, D, Tq // 32, device=dev).half()
+        kz = torch.randn(B, H, D, Tq // 32, device=dev).half()
+        vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
+        vs = torch.rand(B, H, Tq, D // 32, device=dev).half()
+        vz = torch.randn(B, H, Tq, D // 32, device=dev).half()
+        sets.append((kc, ks, kz, vc, vs, vz))
+    q = torch.randn(B, H, 1, D, device=dev).half()
+    p = torch.softmax(torch.randn(B, H, 1, Tq, device=dev), -1).half()
+    lo = torch.empty(B, H, 1, Tq, device=dev, dtype=torch.float16)
+    o = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+    wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, Tq, D)
+    ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+
+    def qk(i):
+        kc, ks, kz = sets[i % nsets][:3]
+        return lib.kvmix_quantized_gemv(32, q.data_ptr(), D, D, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(),
+                                        kz.data_ptr(), ks.stride(1), ks.stride(2), bits, 0, B * H, 1, 1, D, Tq,
+                                        lo.data_ptr(), Tq, Tq, None, 0, stream)
+
+    def pv(i):
+        vc, vs, vz = sets[i % nsets][3:]
+        return lib.kvmix_quantized_gemv(32, p.data_ptr(), Tq, Tq, vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(),
+                                        vz.data_ptr(), vs.stride(1), vs.stride(2), bits, 0, B * H, 1, 1, Tq, D,
+                                        o.data_ptr(), D, D, ws.data_ptr(), wsb, stream)
+
+    nbytes = B * H * Tq * bytes_per_token(bits, "")
+    res = {}
+    for name, fn in (("qk", qk), ("pv", pv)):
+        for i in range(warm):
+            assert fn(i) == 0
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(iters):
+            fn(i)
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) * 1e3 / iters
+        res[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del sets
+    return res
+
+
 def target_shape_extra(torch, _lib, lib, dev, stream):
     """The shape the target is quoted on: B=16, 32 heads, T=8192 (8064 quantized), 4- and 2-bit."""
-    B, H, D, Tq = 16, 32, 128, 8064
     res = {}
     for bits in (4, 2):
-        sets = []
-        for _ in range(3):  # three buffer sets (~1 GB at 4 bits) so the Infinity Cache cannot serve them
-            kc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, D, Tq * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
-            ks = torch.rand(B, H, D, Tq // 32, device=dev).half()
-            kz = torch.randn(B, H, D, Tq // 32, device=dev).half()
-            vc = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, H, Tq, D * bits // 32), dtype=torch.int64, device=dev).to(torch.int32)
-            vs = torch.rand(B, H, Tq, D // 32, device=dev).half()
-            vz = torch.randn(B, H, Tq, D // 32, device=dev).half()
-            sets.append((kc, ks, kz, vc, vs, vz))
-        q = torch.randn(B, H, 1, D, device=dev).half()
-        p = torch.softmax(torch.randn(B, H, 1, Tq, device=dev), -1).half()
-        lo = torch.empty(B, H, 1, Tq, device=dev, dtype=torch.float16)
-        o = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
-        wsb = lib.kvmix_gemv_workspace_bytes(B * H, 1, Tq, D)
-        ws = torch.empty(max(wsb, 16), device=dev, dtype=torch.uint8)
+        r = mha_pair_times(torch, lib, dev, stream, 16, 8064, bits)  # three buffer sets: ~1 GB at 4 bits
+        res[f"qk_{bits}bit"], res[f"pv_{bits}bit"] = r["qk"], r["pv"]
+    return res
 
-        def qk(i):
-            kc, ks, kz = sets[i % 3][:3]
-            return lib.kvmix_quantized_gemv(32, q.data_ptr(), D, D, kc.data_ptr(), kc.stride(1), kc.stride(2), ks.data_ptr(),
-                                            kz.data_ptr(), ks.stride(1), ks.stride(2), bits, 0, B * H, 1, 1, D, Tq,
-                                            lo.data_ptr(), Tq, Tq, None, 0, stream)
 
-        def pv(i):
-            vc, vs, vz = sets[i % 3][3:]
-            return lib.kvmix_quantized_gemv(32, p.data_ptr(), Tq, Tq, vc.data_ptr(), vc.stride(1), vc.stride(2), vs.data_ptr(),
-                                            vz.data_ptr(), vs.stride(1), vs.stride(2), bits, 0, B * H, 1, 1, Tq, D,
-                                            o.data_ptr(), D, D, ws.data_ptr(), wsb, stream)
-
-        nbytes = B * H * Tq * bytes_per_token(bits, "")
-        for name, fn in (("qk", qk), ("pv", pv)):
-            for i in range(30):  # warm-up: 30 launches, then 100 timed ones
-                assert fn(i) == 0
-            torch.cuda.synchronize()
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            for i in range(100):
-                fn(i)
-            e.record()
-            torch.cuda.synchronize()
-            us = s.elapsed_time(e) * 1e3 / 100
-            res[f"{name}_{bits}bit"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
-                                        "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
-        del sets
+def length_scan_extra(torch, _lib, lib, dev, stream):
+    """The same pair against the number of quantized tokens at B = 8 and 16 (--length-scan): the time that does
+    not scale with the bytes (the intercept) and the rate the kernels approach for long rows; with the kernel
+    each launch was dispatched to."""
+    res = {}
+    for B in (8, 16):
+        for bits in (4, 2):
+            for Tq in (1024, 2048, 4096, 8064, 16128, 32256):
+                nbytes = B * 32 * Tq * bytes_per_token(bits, "")
+                nsets = int(min(12, max(3, 600e6 // nbytes + 1)))
+                r = mha_pair_times(torch, lib, dev, stream, B, Tq, bits, nsets=nsets, warm=2 * nsets, iters=5 * nsets)
+                r["qk"]["kernel"] = _lib.gemv_plan(32, bits, 0, B * 32, 1, 1, 128, Tq)["kernel"]
+                r["pv"]["kernel"] = _lib.gemv_plan(32, bits, 0, B * 32, 1, 1, Tq, 128)["kernel"]
+                res[f"B{B}_{bits}bit_T{Tq}"] = r
+                torch.cuda.empty_cache()
     return res
 
 
@@ -671,6 +698,8 @@ def main():
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="run only the streaming-read probe (what a kernel without arithmetic reaches)")
     ap.add_argument("--no-stream-ceiling", action="store_true", help="skip the streaming-read probe")
+    ap.add_argument("--length-scan", action="store_true",
+                    help="only q.K^T / p.V at B = 8 and 16 against the number of quantized tokens (1k .. 32k)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 1 GiB device copies (a known-size kernel to scale HBM counters by)")
     args = ap.parse_args()
@@ -688,6 +717,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, D, T, R = args.batch, 32, 128, args.context, 128
+    if args.length_scan:
+        print(json.dumps({"length_scan": length_scan_extra(torch, _lib, lib, dev, torch.cuda.current_stream().cuda_stream)}))
+        return
     if args.stream_ceiling:
         res = stream_ceiling_extra(torch, _lib, lib, dev)
         print(json.dumps({"hbm_read_ceiling_GBps": max(v["GBps"] for v in res.values()), "stream_ceiling": res}))
