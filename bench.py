@@ -494,7 +494,7 @@ def stream_ceiling_extra(torch, _lib, lib, dev):
     return res
 
 
-def attention_step_extra(torch, dev):
+def attention_step_extra(torch, dev, shapes=None):
     """The whole attention step of one layer (logits over packed keys + fp16 tail, softmax, output
     over packed values + fp16 tail) in its two forms: four launches with the reference's roundings,
     and one pass over the positions (two launches).  MHA 32 x 128, 128-token fp16 tails; buffer sets
@@ -504,7 +504,8 @@ def attention_step_extra(torch, dev):
     H, D, R = 32, 128, 128
     res = {}
     side = torch.cuda.Stream()
-    for (B, T, kb, vb) in [(1, 4096, 4, 4), (4, 2304, 4, 4), (4, 2304, 3, 2), (4, 2304, 2, 2), (8, 8192, 4, 4), (16, 8192, 4, 4)]:
+    for (B, T, kb, vb) in shapes or [(1, 4096, 4, 4), (4, 2304, 4, 4), (4, 2304, 3, 2), (4, 2304, 2, 2), (8, 8192, 4, 4),
+                                     (16, 8192, 4, 4)]:
         kg = 11 if kb == 3 else 32
         tk, tv = ((T - R) // kg) * kg, ((T - R) // 32) * 32
         kbytes = (1024 / 11 if kb == 3 else 16 * kb + 16) * tk
@@ -543,7 +544,8 @@ def attention_step_extra(torch, dev):
             us = s.elapsed_time(e) * 1e3 / iters
             del graph
             entry[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
-        entry["chosen"] = "single_pass" if ops.prefer_single_pass(B, H, H, D, T, kb, 0, kg, vb, 0, 32) else "four_launch"
+        entry["chosen"] = "single_pass" if ops.prefer_single_pass(B, H, H, D, T, kb, 0, kg, vb, 0, 32, k_tokens=tk,
+                                                                   v_tokens=tv) else "four_launch"
         res[f"B{B}_T{T}_k{kb}v{vb}"] = entry
         del sets
         torch.cuda.empty_cache()

@@ -184,7 +184,7 @@ class KVmixAttention:
                                      f"{(B, nh, 1, kv_seq_len)}")
                 single = (not need_weights) and ops.prefer_single_pass(
                     B, nh, key_states.shape[1], D, kv_seq_len, self.k_bits, k_fmt, k_group, self.v_bits, v_fmt,
-                    self.Vgroup_size)
+                    self.Vgroup_size, k_tokens=kv_seq_len - k_tail.shape[2], v_tokens=kv_seq_len - v_tail.shape[2])
                 attn_output, attn_weights = ops.decode_attention(
                     query_states, (kc, ks, km), (vc, vs, vm), k_tail, v_tail, k_group, self.k_bits, self.Vgroup_size,
                     self.v_bits, k_fmt, v_fmt, attention_mask, single_pass=single)

@@ -1958,6 +1958,396 @@ gemv_cols_mfma2(GemvArgs a)
     finish_tile(items - 1);
 }
 
+// ---------------------------------------------------------------------------------------
+// attn_slab_mfma<KBITS, VMODE>   the single-pass decode step over the quantized positions, on the matrix
+// cores: one wave = one slab of 1024 positions of one query head (D = 128).
+//   1. logits of the slab: the q.K^T tile of gemv_cols_mfma2 (one tile per wave), the sums kept in registers;
+//      each is rounded to fp16, scaled by 1/sqrt(D) and masked as the reference does it.
+//   2. slab maximum m, p = exp(logit - m) (fp32), their sum l; p goes to the wave's LDS row in position order.
+//   3. p.V over the same 1024 positions, as gemv_rows_mfma does it (eight 128-row chunks), with p taken from
+//      LDS instead of an fp16 vector in memory.
+//   (m, l) and the 128 unnormalised outputs go to the workspace as slab `tile` of the row; the fp16 tails are
+//   further slabs (attn_fused_slab) and attn_fused_merge combines them all.
+//   The last tile of a row is moved back to end at `tokens`; the positions it shares with its neighbour get
+//   p = 0 there.  No block barrier anywhere: a wave without a tile simply leaves.
+//   block = (64, 2..4) waves on neighbouring tiles; grid = (tiles / waves, samples), XCD-swizzled;
+//   dynamic LDS = waves * kSlabLds bytes.
+// ---------------------------------------------------------------------------------------
+constexpr int kSlabKeyBytes = (kColsMfma2Tile * 2 + 32 * 4 + 15) / 16 * 16;  // A tile of the key phase + 32 zero terms
+constexpr int kSlabLds = kSlabKeyBytes + 1024 * 4;                            // ... + the slab's probabilities
+static_assert(kRowsMfmaTile * 2 <= kSlabKeyBytes, "the value phase's A tile reuses the key phase's space");
+
+template <int KBITS, int VMODE>
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
+attn_slab_mfma(AttnSlabArgs a)
+{
+    static_assert(KBITS == 4 || KBITS == 2 || KBITS == 1, "key codes of 1, 2 or 4 bits");
+    constexpr bool NTC = KBITS >= 2;  // (as gemv_cols_mfma2: a 1-bit row piece shares its lines with the neighbours')
+    constexpr int NPOS = 8;
+    constexpr int TG = 32;            // groups per tile
+
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x;
+    const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int nw = (int)blockDim.y;
+    uint8_t *mine = reinterpret_cast<uint8_t *>(lds) + wy * kSlabLds;
+    uint16_t *atile = reinterpret_cast<uint16_t *>(mine);
+    float *pbuf = reinterpret_cast<float *>(mine + kSlabKeyBytes);  // [1024] probabilities of the slab
+    int64_t bx, sample;
+    xcd_swizzled_block(bx, sample, true);
+    const int64_t kv = sample / a.heads_per_kv;
+    const int ngroups = (int)(a.tokens / 32);
+    const int tile = (int)bx * nw + wy;
+    if (tile * TG >= ngroups) return;
+    const int g_first = tile * TG + TG <= ngroups ? tile * TG : ngroups - TG;  // (the last tile ends at `tokens`)
+    const int shift = tile * TG - g_first;                                     // its first groups are the neighbour's
+    float slab_m, slab_l;
+
+    // ---- 1. logits: gemv_cols_mfma2's tile ---------------------------------------------------------------
+    {
+        constexpr int BITS = KBITS;
+        constexpr int CH = 16, KB = CH / 4, AT = kColsMfma2Tile, FPB = 8 / BITS, K = 128;
+        constexpr int WL = BITS == 4 ? 2 : 1;
+        constexpr bool SPLIT = BITS == 4;
+        float *zl = reinterpret_cast<float *>(atile + AT);
+        const uint16_t *xp = a.q + sample * a.q_bs;
+        const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.k_code + kv * a.kc_bs);
+        const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.k_scale + kv * a.ksz_bs);
+        const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.k_zero + kv * a.ksz_bs);
+        const uint32_t c_rs = (uint32_t)a.kc_rs, s_rs = (uint32_t)a.ksz_rs;
+        const int sub = lane % 4, srow = lane / 4, j4 = lane % 4;
+        const uint32_t c_lane = SPLIT ? (uint32_t)lane * 4u : (uint32_t)lane * (2 * BITS);
+        const uint32_t s_lane = 2u * ((uint32_t)srow * s_rs + 8u * (uint32_t)sub);
+
+        f32x4_t acc[2][NPOS];
+        float zacc[8];
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) acc[q][p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) zacc[j] = 0.f;
+        auto cell = [](int t, int s, int l) { return (2 * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
+        const int aoff = SPLIT ? cell(srow / 4, sub / 2, 32 * (sub % 2)) + srow % 4 : cell(srow / 4, 0, 16 * sub) + srow % 4;
+
+        Half8 s8, z8;
+        uint16_t xh;
+        uint32_t w[KB][4][WL];
+        auto load_small = [&](int it) {
+            const uint32_t d0 = (uint32_t)(it * CH);
+            const uint32_t off = 2u * (d0 * s_rs + (uint32_t)g_first);
+            s8 = ld_buffer<Half8, false>(srsrc, s_lane, off);
+            z8 = ld_buffer<Half8, false>(zrsrc, s_lane, off);
+            xh = xp[d0 + (uint32_t)srow];
+        };
+        auto load_codes = [&](int it, int t) {
+            const uint32_t base = 4u * ((uint32_t)(it * CH + 4 * t) * c_rs + (uint32_t)g_first * BITS);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if constexpr (BITS == 1) {
+                    w[t][k][0] = ld_buffer<uint16_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                } else if constexpr (SPLIT) {
+                    w[t][k][0] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                    w[t][k][1] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane + 256u, base + 4u * (uint32_t)k * c_rs);
+                } else {
+                    w[t][k][0] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
+                }
+            }
+        };
+        auto stage = [&]() {
+            const float xv = h16_to_f32(xh);
+            const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) {
+                zacc[jj] = fmaf(xv, h16_to_f32(z8.v[jj]), zacc[jj]);
+                const float v0 = x2 * h16_to_f32(s8.v[jj]);  // split into three bf16 by truncation (exact)
+                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+                const float v1 = v0 - __uint_as_float(b0);
+                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+                const float v2 = v1 - __uint_as_float(b1);
+                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+                for (int pt = 0; pt < 3; pt++) {
+                    if constexpr (SPLIT)
+                        atile[aoff + (((4 * jj + pt) / 16) * 17 + (4 * jj + pt) % 16) * 4] = (uint16_t)(part[pt] >> 16);
+                    else
+                        atile[aoff + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+                }
+            }
+        };
+        auto compute = [&](int t) {
+            const bf16x4_t av0 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 0, lane));
+            const bf16x4_t av1 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 1, lane));
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                uint32_t src[4];
+                uint32_t hi = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    if constexpr (SPLIT) {
+                        src[k] = w[t][k][s];
+                    } else {
+                        src[k] = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][0], 0x44, 0xf, 0xf, false)
+                                        : __builtin_amdgcn_mov_dpp(w[t][k][0], 0xEE, 0xf, 0xf, false);
+                    }
+                }
+                if constexpr (BITS != 4) hi = (s == 0 ? j4 >= 2 : j4 < 2) ? (uint32_t)BITS : 0u;
+#pragma unroll
+                for (int b = 0; b < BITS; b++) {
+                    const uint32_t sel = (0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16)) + hi * 0x00010001u;
+                    const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
+                    const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
+#pragma unroll
+                    for (int f = 0; f < FPB; f++) {
+                        const bf16x4_t bv =
+                            __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<BITS>(t01, f), field_operand<BITS>(t23, f)));
+                        acc[s][b * FPB + f] =
+                            __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(s == 0 ? av0 : av1, bv, acc[s][b * FPB + f], 0, 0, 0);
+                    }
+                }
+            }
+        };
+
+        constexpr int items = K / CH;
+        load_small(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < KB; t++) {
+            load_codes(0, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int i = lane; i < AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+        wave_lds_fence();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+        for (int it = 0; it < items; it++) {
+            const int nx = it + 1 < items ? it + 1 : it;
+            stage();
+            wave_lds_fence();
+            load_small(nx);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < KB; t++) {
+                compute(t);
+                load_codes(nx, t);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wave_lds_fence();
+        }
+
+        // zero terms of the 32 groups, then the logits of this lane's 16 positions
+        {
+            float z[8];
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) z[jj] = zacc[jj];
+            const int first = scatter_reduce<8, 4, 1>(z, lane);
+            z[0] += __shfl_xor(z[0], 32);
+            zl[8 * sub + first] = z[0];
+        }
+        wave_lds_fence();
+        const int q = lane / 4;
+        const float *mrow = a.mask ? a.mask + (sample / a.heads) * a.mask_bs : nullptr;
+        float x[2][NPOS];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int grp = SPLIT ? 16 * s + q : 2 * q + s;  // group of the tile these eight positions are in
+            const int elem = SPLIT ? 64 * s + lane
+                                   : 8 * q + (s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1))));
+            const float zt = zl[grp];
+            float sums[NPOS];
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) sums[p] = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) {
+                const float v = field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+                const float dot = fmaf(v, __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt);
+                float lg = h16_to_f32(f32_to_h16(dot)) * a.inv_sqrt_d;  // fp16 logit -> scaled, masked fp32 value
+                if (mrow) lg = fmaxf(lg + mrow[(int64_t)g_first * 32 + elem * 8 + p], -3.4028234663852886e38f);
+                x[s][p] = grp >= shift ? lg : -INFINITY;
+                mx = fmaxf(mx, x[s][p]);
+            }
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        float sum = 0.f;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int elem = SPLIT ? 64 * s + lane
+                                   : 8 * q + (s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1))));
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) {
+                const float e = x[s][p] == -INFINITY ? 0.f : expf(x[s][p] - mx);
+                sum += e;
+                pbuf[elem * 8 + p] = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+        slab_m = mx;
+        slab_l = sum;
+        wave_lds_fence();
+    }
+
+    // ---- 2. p.V over the slab's 1024 positions: gemv_rows_mfma's chunks ---------------------------------
+    {
+        constexpr int BITS = VMODE;
+        using Elem = typename CodeElem<BITS>::type;
+        constexpr int EB = BITS == 30 ? 3 : BITS, FB = BITS == 30 ? 3 : BITS;
+        constexpr int LPR = 4, EPR = 16, RL = kWave / EPR, RKB = 4 * RL, CH = 128, KB = CH / RKB, FPB = 8 / FB;
+        const int rs = lane / EPR, wi = lane % EPR;
+        const int t_first = g_first * 32, t_end = t_first + 1024;
+        const uint8_t *cp = reinterpret_cast<const uint8_t *>(a.v_code + kv * a.vc_bs) +
+                            (BITS == 30 ? (wi / 4) * 12 + (wi % 4 < 2 ? wi % 4 : 2) * 4 : wi * EB);
+        [[maybe_unused]] const uint32_t sh3 = (uint32_t)(24 * (wi % 4)) % 32u;
+        const uint16_t *sp = a.v_scale + kv * a.vsz_bs;
+        const uint16_t *zp = a.v_zero + kv * a.vsz_bs;
+
+        f32x4_t acc[NPOS];
+        float zacc[LPR];
+#pragma unroll
+        for (int p = 0; p < NPOS; p++) acc[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g = 0; g < LPR; g++) zacc[g] = 0.f;
+        auto cell = [](int t, int l) { return ((4 * t + l / EPR) * 17 + (l % EPR)) * 4 + (t >> 2) * 4; };
+        const int row0 = 2 * lane;
+        int aoff[2];
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int r = row0 + e;
+            aoff[e] = cell(r / RKB, (r % RL) * EPR) + (r % RKB) / RL;
+        }
+        Half8 s8, z8;
+        Elem w[KB][4];
+        // (a chunk past the slab's end -- the prefetch of the last step -- is the last chunk again)
+        auto chunk_base = [&](int k0) { return k0 + CH <= t_end ? k0 : t_end - CH; };
+        auto load_small = [&](int k0) {
+            const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
+            s8 = ld_stream<Half8>(sp + kr * LPR);
+            z8 = ld_stream<Half8>(zp + kr * LPR);
+        };
+        auto load_codes = [&](int k0, int t) {
+            const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
+#pragma unroll
+            for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
+        };
+        auto stage = [&](int k0) {
+            const float2 pv = *reinterpret_cast<const float2 *>(pbuf + (k0 - t_first) + row0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int q = e / LPR, g = e % LPR;
+                const float xv = q == 0 ? pv.x : pv.y;
+                zacc[g] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[g]);
+                // p * scale * 2^90 in three bf16 parts by truncation (24 of the product's bits)
+                const float v0 = (xv * 1237940039285380274899124224.0f) * h16_to_f32(s8.v[e]);
+                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+                const float v1 = v0 - __uint_as_float(b0);
+                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+                const float v2 = v1 - __uint_as_float(b1);
+                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+                for (int pt = 0; pt < 3; pt++) atile[aoff[q] + g * 16 + pt * 4] = (uint16_t)(part[pt] >> 16);
+            }
+        };
+        auto compute = [&](int t) {
+            const bf16x4_t av = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, lane));
+            if constexpr (BITS == 30) {
+                uint32_t v[4], u[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t lo = __builtin_amdgcn_mov_dpp(w[t][k], 0x90, 0xf, 0xf, false);
+                    const uint32_t hi = __builtin_amdgcn_mov_dpp(w[t][k], 0xA4, 0xf, 0xf, false);
+                    v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
+                    u[k] = v[k] >> 4;
+                }
+#pragma unroll
+                for (int mm = 0; mm < 4; mm++) {
+                    const bool from_u = mm == 1 || mm == 2;
+                    const uint32_t b = from_u ? (uint32_t)(mm - 1) : (mm == 0 ? 0u : 2u);
+                    const uint32_t sel = 0x0c000c00u | b | ((4u + b) << 16);
+                    const uint32_t *src = from_u ? u : v;
+                    const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
+                    const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
+                    const int o0 = mm % 2 == 0 ? 0 : 2;
+#pragma unroll
+                    for (int f = 0; f < 2; f++) {
+                        const uint32_t mask = 0x00070007u << (o0 + 3 * f);
+                        const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+                        acc[mm * 2 + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[mm * 2 + f], 0, 0, 0);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < EB; b++) {
+                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+                    const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[t][1], (uint32_t)w[t][0], sel);
+                    const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[t][3], (uint32_t)w[t][2], sel);
+#pragma unroll
+                    for (int f = 0; f < FPB; f++) {
+                        const bf16x4_t bv =
+                            __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
+                        acc[b * FPB + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[b * FPB + f], 0, 0, 0);
+                    }
+                }
+            }
+        };
+
+        load_small(t_first);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < KB; t++) {
+            load_codes(t_first, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int i = lane; i < kRowsMfmaTile / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+        wave_lds_fence();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+        for (int k0 = t_first; k0 < t_end; k0 += CH) {
+            stage(k0);
+            wave_lds_fence();
+            load_small(k0 + CH);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < KB; t++) {
+                compute(t);
+                load_codes(k0 + CH, t);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wave_lds_fence();
+        }
+
+        // zero term of the lane's group; code sums; the four row slots (lane bits 4, 5) meet
+        float z[LPR];
+#pragma unroll
+        for (int g = 0; g < LPR; g++) z[g] = zacc[g];
+        scatter_reduce<LPR, 8, 0>(z, lane);
+        z[0] += __shfl_xor(z[0], 1);
+        z[0] += __shfl_xor(z[0], 2);
+        z[0] += __shfl_xor(z[0], 16);
+        z[0] += __shfl_xor(z[0], 32);
+        float sums[NPOS], flat[NPOS];
+#pragma unroll
+        for (int p = 0; p < NPOS; p++) sums[p] = (acc[p][0] + acc[p][1]) + acc[p][2];
+#pragma unroll
+        for (int p = 0; p < NPOS; p++) {
+            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
+            const float sum = BITS == 30 ? sums[p] : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+            flat[p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
+        }
+        const int first = scatter_reduce<NPOS, 16, 1>(flat, lane);  // two of the lane's eight columns are left
+        float *wo = a.ws_o + ((int64_t)sample * a.slabs + tile) * 128 + wi * NPOS + first;
+        wo[0] = flat[0] + z[0];
+        wo[1] = flat[1] + z[0];
+        if (lane == 0) {
+            float *ml = a.ws_ml + ((int64_t)sample * a.slabs + tile) * 2;
+            ml[0] = slab_m;
+            ml[1] = slab_l;
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256) reduce_splits(GemvArgs a)
 {
     const int64_t sample = blockIdx.y;
@@ -2324,6 +2714,33 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
         launch_cols_mfma2_nt<BITS, true>(a, samples, st);
     else
         launch_cols_mfma2_nt<BITS, false>(a, samples, st);
+}
+
+int launch_attn_slab_mfma(const AttnSlabArgs &a, int k_bits, int v_mode, int64_t samples, hipStream_t stream)
+{
+    const int64_t tiles = (a.tokens / 32 + 31) / 32;
+    if (a.tokens < 1024 || a.tokens % 32 != 0 || samples <= 0 || samples > 65535 || tiles > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    const int wpb = pick_waves_per_block(tiles);
+    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples), block(kWave, wpb);
+    const size_t lds = (size_t)wpb * kSlabLds;
+#define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_slab_mfma<KB_, VM_>), grid, block, lds, stream, a)
+#define KVMIX_SLAB_V(KB_)                          \
+    switch (v_mode) {                              \
+    case 1: KVMIX_SLAB(KB_, 1); break;             \
+    case 2: KVMIX_SLAB(KB_, 2); break;             \
+    case 4: KVMIX_SLAB(KB_, 4); break;             \
+    case 30: KVMIX_SLAB(KB_, 30); break;           \
+    default: return KVMIX_ERR_UNSUPPORTED;         \
+    }
+    switch (k_bits) {
+    case 1: KVMIX_SLAB_V(1) break;
+    case 2: KVMIX_SLAB_V(2) break;
+    case 4: KVMIX_SLAB_V(4) break;
+    default: return KVMIX_ERR_UNSUPPORTED;
+    }
+#undef KVMIX_SLAB_V
+#undef KVMIX_SLAB
+    return launch_status();
 }
 
 template <int MODE>

@@ -40,7 +40,10 @@ struct FusedArgs {
     int64_t k_tokens, v_tokens, k_slots, v_slots, k_len, v_len;
     int k_mode, v_mode;       // 1, 2, 4 = bits; 3 = the reference's 3-bit words (keys) / dense 3-bit (values); 30 = dense 3-bit keys
     int slab;                 // positions per block
-    int slabs;
+    int slabs;                // slabs of a row in the workspace
+    int launch_slabs;         // slabs this launch works on: workspace slabs slab0 .., positions from t_begin on
+    int slab0;
+    int64_t t_begin;
     int head_groups;          // blocks per kv head and slab (query heads of a kv head / heads per block)
     int heads_per_kv, heads;
     float inv_sqrt_d;
@@ -342,12 +345,12 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
     const int64_t n_blocks = gridDim.x, launch = blockIdx.x;
     const int64_t per = n_blocks / 8, rem = n_blocks % 8, xcd = launch % 8;
     const int64_t logical = xcd * per + (xcd < rem ? xcd : rem) + launch / 8;
-    const int slab = (int)(logical % a.slabs);
-    const int head_group = (int)((logical / a.slabs) % a.head_groups);
-    const int64_t kv = logical / ((int64_t)a.slabs * a.head_groups);
+    const int slab = (int)(logical % a.launch_slabs);
+    const int head_group = (int)((logical / a.launch_slabs) % a.head_groups);
+    const int64_t kv = logical / ((int64_t)a.launch_slabs * a.head_groups);
     const int64_t sample0 = kv * a.heads_per_kv + (int64_t)head_group * NREP;
     const int S = a.slab;
-    const int64_t t0 = (int64_t)slab * S, t1 = t0 + S;
+    const int64_t t0 = a.t_begin + (int64_t)slab * S, t1 = t0 + S;
     int64_t k_len = a.k_len_dev ? *a.k_len_dev : a.k_len;
     int64_t v_len = a.v_len_dev ? *a.v_len_dev : a.v_len;
     k_len = k_len < 0 ? 0 : (k_len > a.k_slots ? a.k_slots : k_len);  // a length from device memory never leads past the window
@@ -495,13 +498,13 @@ __global__ void __launch_bounds__(kFusedThreads) attn_fused_slab(FusedArgs a)
 #pragma unroll
         for (int w = 0; w < kFusedWaves; w++) o += red[(w * NREP + h) * kFusedD + c];
         if (a.slabs == 1) a.out[(sample0 + h) * a.o_bs + c] = f32_to_h16(l_h[h] > 0.f ? o / l_h[h] : 0.f);
-        else a.ws_o[((sample0 + h) * a.slabs + slab) * kFusedD + c] = o;
+        else a.ws_o[((sample0 + h) * a.slabs + a.slab0 + slab) * kFusedD + c] = o;
     }
     if (tid == 0 && a.slabs > 1) {
 #pragma unroll
         for (int h = 0; h < NREP; h++) {
-            a.ws_ml[((sample0 + h) * a.slabs + slab) * 2 + 0] = m_h[h];
-            a.ws_ml[((sample0 + h) * a.slabs + slab) * 2 + 1] = l_h[h];
+            a.ws_ml[((sample0 + h) * a.slabs + a.slab0 + slab) * 2 + 0] = m_h[h];
+            a.ws_ml[((sample0 + h) * a.slabs + a.slab0 + slab) * 2 + 1] = l_h[h];
         }
     }
 }
@@ -580,6 +583,39 @@ static int64_t fused_slabs(const kvmix_decode_attn_t *p)
     return (fused_width(p) + s - 1) / s;
 }
 
+// How a row's positions are divided into slabs.  Large steps whose keys and values are quantized to the same
+// length take the quantized positions through the matrix-core kernel (attn_slab_mfma: tiles of 1024 positions, the
+// formats of gemv_cols_mfma2 and gemv_rows_mfma) and only the fp16 tails through attn_fused_slab; everything
+// else goes through attn_fused_slab from position 0.
+#ifndef KVMIX_SLAB_MFMA_MIN_WAVES
+#define KVMIX_SLAB_MFMA_MIN_WAVES 512  // (measured: 512 waves 34 against 38 us, 256 waves 33 against 25 us)
+#endif
+struct FusedLayout {
+    bool mfma;
+    int64_t tiles;       // slabs of the matrix-core kernel (first in the workspace)
+    int64_t tail_slabs;  // slabs of attn_fused_slab, from position t_begin on
+    int64_t t_begin;
+    int64_t slabs() const { return tiles + tail_slabs; }
+};
+
+static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
+{
+    FusedLayout l{false, 0, fused_slabs(p), 0};
+    const int km = fused_key_mode(p), vm = fused_value_mode(p);
+    const int vbits = vm == 3 ? 3 : vm;
+    const int64_t tiles = (p->k_tokens / 32 + 31) / 32;
+    if (p->k_tokens >= 1024 && p->k_tokens == p->v_tokens && (km == 1 || km == 2 || km == 4) && vm != 0 &&
+        p->v_code_row_stride == kFusedD * vbits / 32 && p->v_sz_row_stride == kFusedD / 32 && p->samples <= 65535 &&
+        (kFusedD + 1) * p->k_code_row_stride < (1ll << 29) && (kFusedD + 1) * p->k_sz_row_stride < (1ll << 30) &&
+        p->samples * tiles >= KVMIX_SLAB_MFMA_MIN_WAVES) {
+        l.mfma = true;
+        l.tiles = tiles;
+        l.t_begin = p->k_tokens;
+        l.tail_slabs = (fused_width(p) - p->k_tokens + kSlabG32 - 1) / kSlabG32;
+    }
+    return l;
+}
+
 extern "C" int kvmix_decode_attention_fused_supported(const kvmix_decode_attn_t *p)
 {
     if (!p) return 0;
@@ -591,7 +627,8 @@ extern "C" int kvmix_decode_attention_fused_supported(const kvmix_decode_attn_t 
 extern "C" size_t kvmix_decode_attention_fused_workspace_bytes(const kvmix_decode_attn_t *p)
 {
     if (!p || p->samples <= 0) return 0;
-    return (size_t)p->samples * (size_t)fused_slabs(p) * (kFusedD + 2) * sizeof(float);
+    if (!kvmix_decode_attention_fused_supported(p)) return 0;
+    return (size_t)p->samples * (size_t)fused_layout(p).slabs() * (kFusedD + 2) * sizeof(float);
 }
 
 extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *workspace, size_t workspace_bytes,
@@ -626,7 +663,8 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
         if (!p->v_code || !p->v_scale || !p->v_zero) return KVMIX_ERR_NULL;
         if (p->v_code_row_stride < kFusedD * p->v_bits / 32 || p->v_sz_row_stride < kFusedD / 32) return KVMIX_ERR_SHAPE;
     }
-    const int64_t slabs = fused_slabs(p);
+    const FusedLayout lay = fused_layout(p);
+    const int64_t slabs = lay.slabs();
     const int64_t kv_samples = p->samples / p->heads_per_kv;
     if (slabs > 0x7fffffff || slabs * p->samples > 0x7fffffff) return KVMIX_ERR_SHAPE;  // (blocks of one launch)
     if (!workspace || workspace_bytes < kvmix_decode_attention_fused_workspace_bytes(p)) return KVMIX_ERR_WORKSPACE;
@@ -672,6 +710,9 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     a.v_mode = v_mode;
     a.slab = fused_slab(p);
     a.slabs = (int)slabs;
+    a.launch_slabs = (int)lay.tail_slabs;
+    a.slab0 = (int)lay.tiles;
+    a.t_begin = lay.t_begin;
     a.heads_per_kv = p->heads_per_kv;
     a.heads = p->heads;
     a.inv_sqrt_d = 1.0f / sqrtf((float)p->D);
@@ -680,10 +721,29 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     // one query head per block: the heads that share a kv head re-read its slab through L2 (two heads
     // per block need more registers than a 512-thread block has)
     a.head_groups = p->heads_per_kv;
-    const dim3 grid((unsigned)(slabs * kv_samples * p->heads_per_kv));
-    hipLaunchKernelGGL(attn_fused_slab<1>, grid, dim3(kFusedThreads), 0, st, a);
-    int rc = launch_status();
-    if (rc != KVMIX_OK || slabs == 1) return rc;  // a single slab is normalised and stored by the slab kernel
+    int rc = KVMIX_OK;
+    if (lay.mfma) {
+        AttnSlabArgs m;
+        m.q = a.q, m.q_bs = a.q_bs;
+        m.k_code = a.k_code, m.k_scale = a.k_scale, m.k_zero = a.k_zero;
+        m.kc_bs = a.kc_bs, m.kc_rs = a.kc_rs, m.ksz_bs = a.ksz_bs, m.ksz_rs = a.ksz_rs;
+        m.v_code = a.v_code, m.v_scale = a.v_scale, m.v_zero = a.v_zero;
+        m.vc_bs = a.vc_bs, m.vsz_bs = a.vsz_bs;
+        m.mask = a.mask, m.mask_bs = a.mask_bs;
+        m.ws_o = a.ws_o, m.ws_ml = a.ws_ml;
+        m.tokens = p->k_tokens;
+        m.heads_per_kv = p->heads_per_kv, m.heads = p->heads;
+        m.slabs = (int)slabs;
+        m.inv_sqrt_d = a.inv_sqrt_d;
+        rc = launch_attn_slab_mfma(m, k_mode, v_mode == 3 ? 30 : v_mode, p->samples, st);
+        if (rc != KVMIX_OK) return rc;
+    }
+    if (lay.tail_slabs > 0) {
+        const dim3 grid((unsigned)(lay.tail_slabs * kv_samples * p->heads_per_kv));
+        hipLaunchKernelGGL(attn_fused_slab<1>, grid, dim3(kFusedThreads), 0, st, a);
+        rc = launch_status();
+    }
+    if (rc != KVMIX_OK || (slabs == 1 && !lay.mfma)) return rc;  // a single slab of attn_fused_slab is normalised and stored by that kernel
     hipLaunchKernelGGL(attn_fused_merge, dim3((unsigned)p->samples), dim3(kFusedD), 0, st, a.ws_o, a.ws_ml, (int)slabs,
                        (uint16_t *)p->out, p->out_stride);
     return launch_status();

@@ -118,6 +118,28 @@ __device__ __forceinline__ int scatter_reduce(float *v, int lane)
     }
 }
 
+// One slab of the single-pass decode step on the matrix cores (attn_slab_mfma in dequant_gemv.hip, launched for
+// kvmix_decode_attention_fused in fused_attn.hip): the quantized positions [0, tokens) of keys and values alike.
+struct AttnSlabArgs {
+    const uint16_t *q;        // [samples, 128] fp16
+    int64_t q_bs;
+    const uint32_t *k_code;   // [kv samples, 128, words], groups of 32 positions
+    const uint16_t *k_scale, *k_zero;
+    int64_t kc_bs, kc_rs, ksz_bs, ksz_rs;
+    const uint32_t *v_code;   // [kv samples, tokens, 128 * bits / 32], dense rows
+    const uint16_t *v_scale, *v_zero;
+    int64_t vc_bs, vsz_bs;
+    const float *mask;        // optional [batch, width]
+    int64_t mask_bs;
+    float *ws_o, *ws_ml;      // [samples, slabs, 128] partial outputs, [samples, slabs, 2] slab maximum and sum
+    int64_t tokens;           // a multiple of 32, at least 1024
+    int heads_per_kv, heads;  // query heads per kv head; query heads per batch entry (for the mask row)
+    int slabs;                // slabs of a row in the workspace (these tiles first, the tail's slabs after them)
+    float inv_sqrt_d;
+};
+// k_bits in {1, 2, 4}; v_mode in {1, 2, 4, 30 (dense 3-bit)}
+int launch_attn_slab_mfma(const AttnSlabArgs &a, int k_bits, int v_mode, int64_t samples, hipStream_t stream);
+
 inline int launch_status()
 {
     return hipGetLastError() == hipSuccess ? KVMIX_OK : KVMIX_ERR_LAUNCH;

@@ -196,7 +196,8 @@ class GraphDecoder(Decoder):
             kc, _, ks, km, vc, _, vs, vm, _ = cache.as_tuple()
             width = max(cache.k_tokens, cache.v_tokens) + R
             single = ops.prefer_single_pass(B, cfg.num_heads, cfg.num_kv_heads, D, width, cache.k_bits, cache.k_fmt,
-                                            cache.Kgroup_size, cache.v_bits, cache.v_fmt, cache.Vgroup_size)
+                                            cache.Kgroup_size, cache.v_bits, cache.v_fmt, cache.Vgroup_size,
+                                            k_tokens=cache.k_tokens, v_tokens=cache.v_tokens)
             out, _ = ops.decode_attention(q, (kc, ks, km), (vc, vs, vm), kwin, vwin, cache.Kgroup_size, cache.k_bits,
                                           cache.Vgroup_size, cache.v_bits, cache.k_fmt, cache.v_fmt,
                                           k_tail_len=klive, v_tail_len=vlive, single_pass=single)

@@ -220,3 +220,17 @@ def test_python_ops_reject_bad_arguments_like_the_reference():
         KVmix.process_value_quantization_cuda(x, q[..., :0], s[..., :0], s[..., :0], 11, 3)
     assert sorted(KVmix.__all__) == sorted(["quantized_gemm", "quantize_pack_last_dim_cuda",
                                             "process_value_quantization_cuda", "process_key_quantization_cuda"])
+
+
+def test_single_pass_policy_knows_the_matrix_core_steps():
+    """prefer_single_pass: small steps always; large ones only where the library can run the quantized
+    positions on the matrix cores (needs the quantized lengths)."""
+    from kvmix_amd import ops
+
+    small = ops.prefer_single_pass(4, 32, 32, 128, 2304, 4, 0, 32, 4, 0, 32)
+    large_unknown = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32)
+    large = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32, k_tokens=8064, v_tokens=8064)
+    uneven = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32, k_tokens=8064, v_tokens=8032)
+    ref3 = ops.prefer_single_pass(16, 32, 32, 128, 8192, 3, 0, 11, 4, 0, 32, k_tokens=8063, v_tokens=8063)
+    few = ops.prefer_single_pass(2, 32, 32, 128, 16384, 4, 0, 32, 4, 0, 32, k_tokens=2048, v_tokens=2048)
+    assert (small, large_unknown, large, uneven, ref3, few) == (True, False, True, False, False, False)

@@ -201,3 +201,57 @@ def test_more_rows_than_one_grid_dimension_holds(dev):
     logits = (q[sl].double() @ keys.transpose(2, 3)) / np.sqrt(128.0)
     want = torch.softmax(logits, -1) @ vals
     check(out_s[sl], want, v_magnitude(vq, v_tail, v_bits))
+
+
+@pytest.mark.parametrize("k_bits", [1, 2, 4])
+@pytest.mark.parametrize("v_bits", [1, 2, 3, 4])
+def test_large_steps_on_the_matrix_cores(dev, k_bits, v_bits):
+    """Steps with at least 1024 (query head, 1024-position tile) pairs whose keys and values are quantized to
+    the same length run their quantized positions through the matrix-core slab kernel: against the four-launch
+    step, with a padding mask, query heads sharing kv heads, a last tile that is moved back (8064 = 7.875 tiles)
+    and, for one pair, fp64 attention over the dequantized cache of two rows."""
+    from kvmix_amd import ops
+    from helpers import dequantize_torch
+
+    gen = torch.Generator(device=dev).manual_seed(100 + 10 * k_bits + v_bits)
+    rng = np.random.default_rng(k_bits * 7 + v_bits)
+    B, nkv, rep, tk, n = 2, 32, 2, 8064, 8064 + 97
+    q, kq, vq, k_tail, v_tail, kg, mask, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tk, n, mask_rng=rng)
+    out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, **fmt)
+    out_s, none = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask,
+                                       single_pass=True, **fmt)
+    assert none is None
+    vm = v_magnitude(vq, v_tail, v_bits)
+    check(out_s, out_f, vm)
+    if (k_bits, v_bits) in ((4, 2), (2, 3), (1, 4)):
+        sl = slice(B - 1, B)
+        kd = dequantize_torch(kq[0][sl, :2], kq[1][sl, :2], kq[2][sl, :2], k_bits, 32).double()      # [1, 2, D, tk]
+        vd = dequantize_torch(vq[0][sl, :2], vq[1][sl, :2], vq[2][sl, :2], v_bits, 32, dense3=v_bits == 3).double()
+        keys = torch.cat([kd.transpose(2, 3), k_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+        vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+        qq = q[sl, :2 * rep].double()
+        logits = (qq @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
+        want = torch.softmax(logits, -1) @ vals
+        check(out_s[sl, :2 * rep], want, vm)
+
+
+def test_matrix_core_slabs_with_short_rows_and_device_side_lengths(dev):
+    """Two tiles of which the second is moved back almost wholly (1056 positions), tails in longer windows
+    with their lengths on the device."""
+    from kvmix_amd import ops
+
+    gen = torch.Generator(device=dev).manual_seed(77)
+    B, nkv, rep, k_bits, v_bits, tk = 16, 32, 1, 4, 4, 1056
+    lk = 41
+    q, kq, vq, k_tail, v_tail, kg, _, fmt, _, _ = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tk, tk + lk)
+    want, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, **fmt)
+    got, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, single_pass=True, **fmt)
+    check(got, want, v_magnitude(vq, v_tail, v_bits))
+    R = lk + 23
+    kwin = torch.full((B, nkv, R, 128), 77.0, dtype=torch.float16, device=dev)
+    vwin = torch.full((B, nkv, R, 128), float("nan"), dtype=torch.float16, device=dev)
+    kwin[:, :, :lk], vwin[:, :, :lk] = k_tail, v_tail
+    klen = torch.tensor([lk], dtype=torch.int64, device=dev)
+    got2, _ = ops.decode_attention(q, kq, vq, kwin, vwin, kg, k_bits, 32, v_bits, k_tail_len=klen, v_tail_len=klen.clone(),
+                                   single_pass=True, **fmt)
+    assert torch.equal(got2, got)
