@@ -295,6 +295,10 @@ int kvmix_decode_attention(const kvmix_decode_attn_t *step, void *workspace, siz
  * logits, 1/sqrt(D), mask, clamp) but not the reference's roundings after it: probabilities are not
  * rounded to fp16 and the quantized and tail halves of the output are not rounded separately, so the
  * result differs from kvmix_decode_attention's by up to about 2^-10 of the largest value magnitude.
+ * Large steps (at least 512 (query head, 1024-position tile) pairs) whose keys (1, 2 or 4 bits) and values are
+ * quantized to the same length of at least 1024 positions, with dense value rows, run those positions on the
+ * matrix cores -- one wave per tile: logits, slab softmax and the product with the values of the same positions --
+ * and only the fp16 tails through the vector-ALU slab kernel (three launches); everything else as described above.
  *
  * Supported (kvmix_decode_attention_fused_supported returns 1, else the call returns
  * KVMIX_ERR_UNSUPPORTED): D = 128; keys 1/2/4-bit or dense 3-bit in groups of 32 or the reference's 3-bit words;
