@@ -408,14 +408,19 @@ struct KeyTokArgs {
     float inv_qmax;
 };
 
-// G values of one channel -> packed words, scale, zero, stored at group gi of channel d
+// words of one quantization group of a channel
 template <int G, int MODE>
-__device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float (&v)[G], int64_t gi, int64_t o,
-                                                int64_t d)
+constexpr int key_group_words() { return MODE == 3 ? 1 : (G * (MODE == 30 ? 3 : MODE)) / 32; }
+
+// G values of one channel -> packed words, scale, zero
+template <int G, int MODE>
+__device__ __forceinline__ void key_group_codes(const KeyTokArgs &a, const float (&v)[G],
+                                                uint32_t (&w)[key_group_words<G, MODE>()], __half &scale_out,
+                                                __half &zero_out)
 {
     constexpr int BITS = MODE == 30 ? 3 : MODE;
     constexpr int qmax = (1 << BITS) - 1;
-    constexpr int WORDS = MODE == 3 ? 1 : (G * BITS) / 32;  // words per group
+    constexpr int WORDS = key_group_words<G, MODE>();
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
 #pragma unroll
     for (int t = 0; t < G; t++) {
@@ -425,7 +430,6 @@ __device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float
     const float range = mx - mn;
     const float scale = range / (float)qmax;
     const float rcp = quantize_rcp(scale);
-    uint32_t w[WORDS];
 #pragma unroll
     for (int t = 0; t < WORDS; t++) w[t] = 0;
     if constexpr (MODE == 3) {
@@ -447,12 +451,24 @@ __device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float
             }
         }
     }
+    scale_out = __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
+    zero_out = __float2half_rn(mn);
+}
+
+// ... stored at group gi of channel d
+template <int G, int MODE>
+__device__ __forceinline__ void key_group_store(const KeyTokArgs &a, const float (&v)[G], int64_t gi, int64_t o,
+                                                int64_t d)
+{
+    constexpr int WORDS = key_group_words<G, MODE>();
+    uint32_t w[WORDS];
+    __half sc, zr;
+    key_group_codes<G, MODE>(a, v, w, sc, zr);
     uint32_t *cw = a.code + o * a.c_os + d * a.c_is + gi * WORDS;
 #pragma unroll
     for (int t = 0; t < WORDS; t++) cw[t] = w[t];
-    a.scale[o * a.s_os + d * a.s_is + gi] =
-        __float2half_rn(scale_for_output(range, scale, a.inv_qmax, a.scale_mode));
-    a.zero[o * a.s_os + d * a.s_is + gi] = __float2half_rn(mn);
+    a.scale[o * a.s_os + d * a.s_is + gi] = sc;
+    a.zero[o * a.s_os + d * a.s_is + gi] = zr;
 }
 
 template <int G, int MODE>
@@ -499,6 +515,94 @@ __device__ __forceinline__ void key_tokens_tile_body(const KeyTokArgs &a, int64_
     if (valid) key_group_store<G, MODE>(a, v, gi, o, t);
 }
 
+// Reference 3-bit keys (groups of 11 tokens, one word each), D = 128 with 16-byte-aligned token rows:
+// 256 threads take up to 11 groups (121 tokens) of 64 channels of one outer slice.  The [tokens][64] tile
+// goes through LDS as above; thread (channel t % 64, t / 64) packs groups t / 64, + 4, + 8; the words,
+// scales and zeros are then handed over through LDS so that neighbouring lanes write neighbouring
+// entries of a channel row (44 + 22 + 22 contiguous bytes per row instead of 33 separate stores
+// from different blocks).  Units: (outer, chunk of 11 groups, channel half), channel half fastest.
+// Every thread of the block must call it (block barriers).
+constexpr int kRef3SlabGroups = 11;
+constexpr int kRef3SlabChannels = 64;
+static inline int64_t ref3_slab_units(int64_t outer, int64_t k_groups)
+{
+    return outer * ((k_groups + kRef3SlabGroups - 1) / kRef3SlabGroups) * (128 / kRef3SlabChannels);
+}
+// what both tiled key paths ask of the operand: D = 128, token rows that 128-bit loads can fetch
+static inline bool key_rows_tileable(const KeyTokArgs &a)
+{
+    return a.D == 128 && (uintptr_t)a.k % 16 == 0 && a.k_ts % 8 == 0 && a.k_os % 8 == 0;
+}
+__device__ __forceinline__ void key_tokens_ref3_slab_body(const KeyTokArgs &a, int64_t k_groups, int64_t unit,
+                                                          uint16_t *tile)
+{
+    constexpr int GC = kRef3SlabGroups, CH = kRef3SlabChannels, PPR = CH / 8;  // 16-byte pieces per tile row
+    const int tid = threadIdx.x;
+    const uint32_t chunks = (uint32_t)((k_groups + GC - 1) / GC);
+    const uint32_t u = (uint32_t)unit;  // (the host keeps the units below 2^31)
+    const uint32_t half = u % 2u, rest = u / 2u, chunk = rest % chunks;
+    const int64_t o = rest / chunks;
+    const int g0 = (int)chunk * GC;
+    const int ng = (int)(k_groups - g0 < GC ? k_groups - g0 : GC);
+    const int pieces = ng * 11 * PPR;
+    const __half *src = a.k + o * a.k_os + (int64_t)g0 * 11 * a.k_ts + half * CH;
+    constexpr int ROUNDS = (GC * 11 * PPR + 255) / 256;
+    uint4 raw[ROUNDS];
+#pragma unroll
+    for (int i = 0; i < ROUNDS; i++) {
+        int pc = i * 256 + tid;
+        pc = pc < pieces ? pc : pieces - 1;
+        raw[i] = *reinterpret_cast<const uint4 *>(src + (int64_t)(pc / PPR) * a.k_ts + (pc % PPR) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < ROUNDS; i++) {
+        const int pc = i * 256 + tid;
+        if (pc < pieces) *reinterpret_cast<uint4 *>(tile + (pc / PPR) * CH + (pc % PPR) * 8) = raw[i];
+    }
+    __syncthreads();
+    const int dl = tid % CH, gq = tid / CH;
+    uint32_t w[3];
+    __half sc[3], zr[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int g = gq + 4 * j;
+        if (g < ng) {
+            float v[11];
+#pragma unroll
+            for (int r = 0; r < 11; r++) v[r] = h16_to_f32(tile[(g * 11 + r) * CH + dl]);
+            uint32_t w1[1];
+            key_group_codes<11, 3>(a, v, w1, sc[j], zr[j]);
+            w[j] = w1[0];
+        }
+    }
+    __syncthreads();  // the tile is read: its memory now carries the results, [channel][group]
+    uint32_t *ow = reinterpret_cast<uint32_t *>(tile);
+    __half *os = reinterpret_cast<__half *>(tile + 2 * CH * GC), *oz = os + CH * GC;
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int g = gq + 4 * j;
+        if (g < ng) {
+            ow[dl * ng + g] = w[j];
+            os[dl * ng + g] = sc[j];
+            oz[dl * ng + g] = zr[j];
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < CH * ng; idx += 256) {
+        const int d = idx / ng, g = idx - d * ng;
+        const int64_t row = (int64_t)half * CH + d;
+        a.code[o * a.c_os + row * a.c_is + g0 + g] = ow[idx];
+        a.scale[o * a.s_os + row * a.s_is + g0 + g] = os[idx];
+        a.zero[o * a.s_os + row * a.s_is + g0 + g] = oz[idx];
+    }
+}
+
+__global__ void __launch_bounds__(256) quant_key_tokens_ref3_slab(KeyTokArgs a, int64_t k_groups, int64_t unit0)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t tile[kRef3SlabGroups * 11 * kRef3SlabChannels];
+    key_tokens_ref3_slab_body(a, k_groups, unit0 + blockIdx.x, tile);
+}
+
 template <int G, int MODE>
 __global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
 {
@@ -519,13 +623,14 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
                                                       int64_t v_total_groups)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[2][32][128];
-    if (blockIdx.x < k_blocks && k_tiled) {
+    if (blockIdx.x < k_blocks && k_tiled == 2) {
+        key_tokens_ref3_slab_body(ka, k_groups, blockIdx.x, &tile[0][0][0]);
+    } else if (blockIdx.x < k_blocks && k_tiled) {
         // (k_threads = pairs * 128: one block = two (group, outer) pairs)
         const int64_t pairs = k_threads / 128, first = (int64_t)blockIdx.x * 2;
         switch (kmode) {
         case 1: key_tokens_tile_body<32, 1>(ka, k_groups, pairs, first, tile); break;
         case 2: key_tokens_tile_body<32, 2>(ka, k_groups, pairs, first, tile); break;
-        case 3: key_tokens_tile_body<11, 3>(ka, k_groups, pairs, first, tile); break;
         case 4: key_tokens_tile_body<32, 4>(ka, k_groups, pairs, first, tile); break;
         default: key_tokens_tile_body<32, 30>(ka, k_groups, pairs, first, tile); break;
         }
@@ -758,6 +863,12 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
 
 static int launch_key_tokens(const KeyTokArgs &a, int mode, int64_t groups, int64_t outer, hipStream_t st)
 {
+    if (mode == 3 && key_rows_tileable(a)) {
+        const int64_t units = ref3_slab_units(outer, groups);
+        if (units > 0x7fffffff) return KVMIX_ERR_SHAPE;
+        hipLaunchKernelGGL(quant_key_tokens_ref3_slab, dim3((unsigned)units), dim3(256), 0, st, a, groups, (int64_t)0);
+        return launch_status();
+    }
     const int block = a.D >= 128 ? 128 : 64;
     if ((a.D + block - 1) / block > 65535) return KVMIX_ERR_SHAPE;
     // (grid.y holds at most 65535 blocks: more (batch, head) slices than that go out in several launches)
@@ -847,14 +958,13 @@ extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmi
         }
         return vempty ? KVMIX_OK : launch_last_dim(va, KVMIX_F16, vpw, vfast, st);
     }
+    // key tile paths: D = 128, token rows 16-byte aligned (2: the reference 3-bit slabs)
+    const int k_tiled = !(KVMIX_FLUSH_K_TILED && key_rows_tileable(ka)) ? 0 : (kmode == 3 ? 2 : 1);
     const int64_t k_threads = kgroups * kf->outer * kf->D;
-    const int64_t k_blocks = (k_threads + 255) / 256;
+    const int64_t k_blocks = k_tiled == 2 ? ref3_slab_units(kf->outer, kgroups) : (k_threads + 255) / 256;
     const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
     const int64_t v_blocks = (v_total * 4 + 256 * KVMIX_FLUSH_V_PIECES - 1) / (256 * KVMIX_FLUSH_V_PIECES);
     if (k_blocks + v_blocks > 0x7fffffff || k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    // key tile path: D = 128, token rows 16-byte aligned
-    const int k_tiled = KVMIX_FLUSH_K_TILED && kf->D == 128 && (uintptr_t)kf->k % 16 == 0 && kf->k_token_stride % 8 == 0 &&
-                        kf->k_outer_stride % 8 == 0;
     hipLaunchKernelGGL(quant_kv_flush, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, ka, kmode, kgroups,
                        k_threads, (unsigned)k_blocks, k_tiled, va, v_groups, v_total);
     return launch_status();

@@ -154,17 +154,19 @@ def test_value_append_3bit_placeholder(oracle, dev):
     check_triplet(got, want)
 
 
-@pytest.mark.parametrize("bits,g,fmt", [(4, 32, 0), (2, 32, 0), (1, 32, 0), (3, 11, 0)])
-def test_key_tokens_kernel_equals_transpose_then_quantize(oracle, dev, bits, g, fmt):
+@pytest.mark.parametrize("bits,g,fmt,groups", [(4, 32, 0, 4), (2, 32, 0, 4), (1, 32, 0, 4), (3, 11, 0, 4),
+                                               (3, 11, 0, 11), (3, 11, 0, 25)])
+def test_key_tokens_kernel_equals_transpose_then_quantize(oracle, dev, bits, g, fmt, groups):
     """C ABI kvmix_quant_pack_key_tokens == quantize_pack_last_dim(tail[:, :, :n].transpose(2,3))
-    written at an offset into a larger channel-major cache."""
+    written at an offset into a larger channel-major cache.  (The reference 3-bit kernel takes the groups of a
+    slice eleven at a time: fewer than, exactly and more than eleven, the last chunk ragged.)"""
     from kvmix_amd import _lib
 
     L = _lib.load()
     rng = np.random.default_rng(bits + 70)
     B, H, D = 2, 3, 128
-    n = g * 4
-    cap_tokens = g * 10
+    n = g * groups
+    cap_tokens = g * (groups + 6)
     vpw = oracle.values_per_word(bits)
     tail = kv_like(rng, (B, H, n + 5, D), outlier_axis=3)     # longer tail, only n flushed
     t = torch.from_numpy(tail).to(dev)
