@@ -481,62 +481,38 @@ __device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi,
     key_group_store<G, MODE>(a, v, gi, o, d);
 }
 
-// The same for D = 128 with 16-byte-aligned token rows, 256 threads = two (group, outer) pairs:
-// the pair's [G tokens][128 channels] tile is fetched with 128-bit loads (a thread: 8 channels of
-// one token) into LDS and each thread then reads its channel's column -- 4 wide loads per
-// thread instead of 32 two-byte ones.  Every thread of the block must call it (block barrier).
-template <int G, int MODE>
-__device__ __forceinline__ void key_tokens_tile_body(const KeyTokArgs &a, int64_t k_groups, int64_t pairs,
-                                                     int64_t first_pair, uint16_t (*tile)[32][128])
+// The same for D = 128 with 16-byte-aligned token rows: 256 threads take a chunk of groups (four of 32
+// tokens, or eleven of the reference 3-bit format's 11) of 64 channels of one outer slice.  The
+// [tokens][64] tile is fetched with 128-bit loads (a thread: 8 channels of one token) into LDS; thread
+// (channel t % 64, t / 64) reads its channel's column and packs groups t / 64, + 4, + 8 of the chunk; the
+// words, scales and zeros are then handed over through LDS so that neighbouring lanes write neighbouring
+// entries of a channel row: one contiguous piece of codes, one of scales and one of zeros per row (for
+// the reference 3-bit format 44 + 22 + 22 bytes instead of 33 separate stores from different blocks).
+// Units: (outer, chunk, channel half), channel half fastest.  Every thread of the block must call it
+// (block barriers).
+constexpr int kKeySlabChannels = 64;
+template <int MODE>
+constexpr int key_slab_groups() { return MODE == 3 ? 11 : 4; }   // 121 or 128 tokens: a 16 KB tile
+static inline int64_t key_slab_units(int mode, int64_t outer, int64_t k_groups)
 {
-    const int half = threadIdx.x / 128, t = threadIdx.x % 128;
-    const int64_t pair = first_pair + half;
-    const bool valid = pair < pairs;
-    const uint32_t pc = (uint32_t)(valid ? pair : pairs - 1);  // (the host keeps pairs below 2^31)
-    const int64_t o = pc / (uint32_t)k_groups, gi = pc - (uint32_t)o * (uint32_t)k_groups;
-    const __half *src = a.k + o * a.k_os + gi * G * a.k_ts;
-    constexpr int PIECES = G * 16;  // 16-byte pieces of the tile
-    uint4 raw[(PIECES + 127) / 128];
-#pragma unroll
-    for (int i = 0; i < (PIECES + 127) / 128; i++) {
-        int pc8 = i * 128 + t;
-        pc8 = pc8 < PIECES ? pc8 : PIECES - 1;
-        raw[i] = *reinterpret_cast<const uint4 *>(src + (int64_t)(pc8 / 16) * a.k_ts + (pc8 % 16) * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < (PIECES + 127) / 128; i++) {
-        const int pc8 = i * 128 + t;
-        if (pc8 < PIECES) *reinterpret_cast<uint4 *>(&tile[half][pc8 / 16][(pc8 % 16) * 8]) = raw[i];
-    }
-    __syncthreads();
-    float v[G];
-#pragma unroll
-    for (int r = 0; r < G; r++) v[r] = h16_to_f32(tile[half][r][t]);
-    if (valid) key_group_store<G, MODE>(a, v, gi, o, t);
+    const int gc = mode == 3 ? key_slab_groups<3>() : key_slab_groups<4>();
+    return outer * ((k_groups + gc - 1) / gc) * (128 / kKeySlabChannels);
 }
-
-// Reference 3-bit keys (groups of 11 tokens, one word each), D = 128 with 16-byte-aligned token rows:
-// 256 threads take up to 11 groups (121 tokens) of 64 channels of one outer slice.  The [tokens][64] tile
-// goes through LDS as above; thread (channel t % 64, t / 64) packs groups t / 64, + 4, + 8; the words,
-// scales and zeros are then handed over through LDS so that neighbouring lanes write neighbouring
-// entries of a channel row (44 + 22 + 22 contiguous bytes per row instead of 33 separate stores
-// from different blocks).  Units: (outer, chunk of 11 groups, channel half), channel half fastest.
-// Every thread of the block must call it (block barriers).
-constexpr int kRef3SlabGroups = 11;
-constexpr int kRef3SlabChannels = 64;
-static inline int64_t ref3_slab_units(int64_t outer, int64_t k_groups)
-{
-    return outer * ((k_groups + kRef3SlabGroups - 1) / kRef3SlabGroups) * (128 / kRef3SlabChannels);
-}
-// what both tiled key paths ask of the operand: D = 128, token rows that 128-bit loads can fetch
+// what the slab path asks of the operand: D = 128, token rows that 128-bit loads can fetch
 static inline bool key_rows_tileable(const KeyTokArgs &a)
 {
     return a.D == 128 && (uintptr_t)a.k % 16 == 0 && a.k_ts % 8 == 0 && a.k_os % 8 == 0;
 }
-__device__ __forceinline__ void key_tokens_ref3_slab_body(const KeyTokArgs &a, int64_t k_groups, int64_t unit,
-                                                          uint16_t *tile)
+constexpr int kKeySlabTile = 8192;  // fp16 elements of LDS a block needs (128 tokens x 64 channels)
+
+template <int G, int MODE>
+__device__ __forceinline__ void key_tokens_slab_body(const KeyTokArgs &a, int64_t k_groups, int64_t unit,
+                                                     uint16_t *tile)
 {
-    constexpr int GC = kRef3SlabGroups, CH = kRef3SlabChannels, PPR = CH / 8;  // 16-byte pieces per tile row
+    constexpr int GC = key_slab_groups<MODE>(), CH = kKeySlabChannels, PPR = CH / 8;  // 16-byte pieces per tile row
+    constexpr int WORDS = key_group_words<G, MODE>();
+    constexpr int JMAX = (GC + 3) / 4;  // groups per thread
+    static_assert(GC * G * CH <= kKeySlabTile, "the tile of a chunk");
     const int tid = threadIdx.x;
     const uint32_t chunks = (uint32_t)((k_groups + GC - 1) / GC);
     const uint32_t u = (uint32_t)unit;  // (the host keeps the units below 2^31)
@@ -544,9 +520,9 @@ __device__ __forceinline__ void key_tokens_ref3_slab_body(const KeyTokArgs &a, i
     const int64_t o = rest / chunks;
     const int g0 = (int)chunk * GC;
     const int ng = (int)(k_groups - g0 < GC ? k_groups - g0 : GC);
-    const int pieces = ng * 11 * PPR;
-    const __half *src = a.k + o * a.k_os + (int64_t)g0 * 11 * a.k_ts + half * CH;
-    constexpr int ROUNDS = (GC * 11 * PPR + 255) / 256;
+    const int pieces = ng * G * PPR;
+    const __half *src = a.k + o * a.k_os + (int64_t)g0 * G * a.k_ts + half * CH;
+    constexpr int ROUNDS = (GC * G * PPR + 255) / 256;
     uint4 raw[ROUNDS];
 #pragma unroll
     for (int i = 0; i < ROUNDS; i++) {
@@ -561,46 +537,50 @@ __device__ __forceinline__ void key_tokens_ref3_slab_body(const KeyTokArgs &a, i
     }
     __syncthreads();
     const int dl = tid % CH, gq = tid / CH;
-    uint32_t w[3];
-    __half sc[3], zr[3];
+    uint32_t w[JMAX][WORDS];
+    __half sc[JMAX], zr[JMAX];
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
+    for (int j = 0; j < JMAX; j++) {
         const int g = gq + 4 * j;
         if (g < ng) {
-            float v[11];
+            float v[G];
 #pragma unroll
-            for (int r = 0; r < 11; r++) v[r] = h16_to_f32(tile[(g * 11 + r) * CH + dl]);
-            uint32_t w1[1];
-            key_group_codes<11, 3>(a, v, w1, sc[j], zr[j]);
-            w[j] = w1[0];
+            for (int r = 0; r < G; r++) v[r] = h16_to_f32(tile[(g * G + r) * CH + dl]);
+            key_group_codes<G, MODE>(a, v, w[j], sc[j], zr[j]);
         }
     }
-    __syncthreads();  // the tile is read: its memory now carries the results, [channel][group]
+    __syncthreads();  // the tile is read: its memory now carries the results, [channel][group] at odd pitches
+    const int nw = ng * WORDS, wp = nw | 1, sp = ng | 1;
     uint32_t *ow = reinterpret_cast<uint32_t *>(tile);
-    __half *os = reinterpret_cast<__half *>(tile + 2 * CH * GC), *oz = os + CH * GC;
+    __half *os = reinterpret_cast<__half *>(tile + 2 * CH * ((GC * WORDS) | 1)), *oz = os + CH * (GC | 1);
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
+    for (int j = 0; j < JMAX; j++) {
         const int g = gq + 4 * j;
         if (g < ng) {
-            ow[dl * ng + g] = w[j];
-            os[dl * ng + g] = sc[j];
-            oz[dl * ng + g] = zr[j];
+#pragma unroll
+            for (int t = 0; t < WORDS; t++) ow[dl * wp + g * WORDS + t] = w[j][t];
+            os[dl * sp + g] = sc[j];
+            oz[dl * sp + g] = zr[j];
         }
     }
     __syncthreads();
+    const int64_t row0 = (int64_t)half * CH;
+    for (int idx = tid; idx < CH * nw; idx += 256) {
+        const int d = idx / nw, t = idx - d * nw;
+        a.code[o * a.c_os + (row0 + d) * a.c_is + (int64_t)g0 * WORDS + t] = ow[d * wp + t];
+    }
     for (int idx = tid; idx < CH * ng; idx += 256) {
         const int d = idx / ng, g = idx - d * ng;
-        const int64_t row = (int64_t)half * CH + d;
-        a.code[o * a.c_os + row * a.c_is + g0 + g] = ow[idx];
-        a.scale[o * a.s_os + row * a.s_is + g0 + g] = os[idx];
-        a.zero[o * a.s_os + row * a.s_is + g0 + g] = oz[idx];
+        a.scale[o * a.s_os + (row0 + d) * a.s_is + g0 + g] = os[d * sp + g];
+        a.zero[o * a.s_os + (row0 + d) * a.s_is + g0 + g] = oz[d * sp + g];
     }
 }
 
-__global__ void __launch_bounds__(256) quant_key_tokens_ref3_slab(KeyTokArgs a, int64_t k_groups, int64_t unit0)
+template <int G, int MODE>
+__global__ void __launch_bounds__(256) quant_key_tokens_slab(KeyTokArgs a, int64_t k_groups)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[kRef3SlabGroups * 11 * kRef3SlabChannels];
-    key_tokens_ref3_slab_body(a, k_groups, unit0 + blockIdx.x, tile);
+    __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
+    key_tokens_slab_body<G, MODE>(a, k_groups, blockIdx.x, tile);
 }
 
 template <int G, int MODE>
@@ -622,17 +602,14 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
                                                       QuantArgs va, int64_t v_groups_per_row,
                                                       int64_t v_total_groups)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[2][32][128];
-    if (blockIdx.x < k_blocks && k_tiled == 2) {
-        key_tokens_ref3_slab_body(ka, k_groups, blockIdx.x, &tile[0][0][0]);
-    } else if (blockIdx.x < k_blocks && k_tiled) {
-        // (k_threads = pairs * 128: one block = two (group, outer) pairs)
-        const int64_t pairs = k_threads / 128, first = (int64_t)blockIdx.x * 2;
+    __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
+    if (blockIdx.x < k_blocks && k_tiled) {
         switch (kmode) {
-        case 1: key_tokens_tile_body<32, 1>(ka, k_groups, pairs, first, tile); break;
-        case 2: key_tokens_tile_body<32, 2>(ka, k_groups, pairs, first, tile); break;
-        case 4: key_tokens_tile_body<32, 4>(ka, k_groups, pairs, first, tile); break;
-        default: key_tokens_tile_body<32, 30>(ka, k_groups, pairs, first, tile); break;
+        case 1: key_tokens_slab_body<32, 1>(ka, k_groups, blockIdx.x, tile); break;
+        case 2: key_tokens_slab_body<32, 2>(ka, k_groups, blockIdx.x, tile); break;
+        case 3: key_tokens_slab_body<11, 3>(ka, k_groups, blockIdx.x, tile); break;
+        case 4: key_tokens_slab_body<32, 4>(ka, k_groups, blockIdx.x, tile); break;
+        default: key_tokens_slab_body<32, 30>(ka, k_groups, blockIdx.x, tile); break;
         }
     } else if (blockIdx.x < k_blocks) {
         const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -863,10 +840,17 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
 
 static int launch_key_tokens(const KeyTokArgs &a, int mode, int64_t groups, int64_t outer, hipStream_t st)
 {
-    if (mode == 3 && key_rows_tileable(a)) {
-        const int64_t units = ref3_slab_units(outer, groups);
+    if (KVMIX_FLUSH_K_TILED && key_rows_tileable(a)) {
+        const int64_t units = key_slab_units(mode, outer, groups);
         if (units > 0x7fffffff) return KVMIX_ERR_SHAPE;
-        hipLaunchKernelGGL(quant_key_tokens_ref3_slab, dim3((unsigned)units), dim3(256), 0, st, a, groups, (int64_t)0);
+        const dim3 grid((unsigned)units);
+        switch (mode) {
+        case 3: hipLaunchKernelGGL((quant_key_tokens_slab<11, 3>), grid, dim3(256), 0, st, a, groups); break;
+        case 30: hipLaunchKernelGGL((quant_key_tokens_slab<32, 30>), grid, dim3(256), 0, st, a, groups); break;
+        case 4: hipLaunchKernelGGL((quant_key_tokens_slab<32, 4>), grid, dim3(256), 0, st, a, groups); break;
+        case 2: hipLaunchKernelGGL((quant_key_tokens_slab<32, 2>), grid, dim3(256), 0, st, a, groups); break;
+        default: hipLaunchKernelGGL((quant_key_tokens_slab<32, 1>), grid, dim3(256), 0, st, a, groups); break;
+        }
         return launch_status();
     }
     const int block = a.D >= 128 ? 128 : 64;
@@ -958,10 +942,10 @@ extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmi
         }
         return vempty ? KVMIX_OK : launch_last_dim(va, KVMIX_F16, vpw, vfast, st);
     }
-    // key tile paths: D = 128, token rows 16-byte aligned (2: the reference 3-bit slabs)
-    const int k_tiled = !(KVMIX_FLUSH_K_TILED && key_rows_tileable(ka)) ? 0 : (kmode == 3 ? 2 : 1);
+    // key slab path: D = 128, token rows 16-byte aligned
+    const int k_tiled = KVMIX_FLUSH_K_TILED && key_rows_tileable(ka);
     const int64_t k_threads = kgroups * kf->outer * kf->D;
-    const int64_t k_blocks = k_tiled == 2 ? ref3_slab_units(kf->outer, kgroups) : (k_threads + 255) / 256;
+    const int64_t k_blocks = k_tiled ? key_slab_units(kmode, kf->outer, kgroups) : (k_threads + 255) / 256;
     const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
     const int64_t v_blocks = (v_total * 4 + 256 * KVMIX_FLUSH_V_PIECES - 1) / (256 * KVMIX_FLUSH_V_PIECES);
     if (k_blocks + v_blocks > 0x7fffffff || k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
