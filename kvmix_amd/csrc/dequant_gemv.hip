@@ -2481,6 +2481,18 @@ static void plan_record(const dim3 &grid, const dim3 &block, size_t lds, const c
             hipLaunchKernelGGL(kernel, grid, block, lds, st, args);       \
     } while (0)
 
+// Every tiled kernel moves the last tile of a row back so that it ends at N: a tile wider than the row would
+// start before the row.  The dispatch never picks such a kernel; each launcher checks it all the same, launches
+// nothing when the tile does not fit, and the entry point then reports the shape -- so that a change of the
+// dispatch rules cannot turn into an access outside the operands.
+static thread_local int t_refused = KVMIX_OK;
+static bool tile_fits(int64_t units, int64_t tile_units)
+{
+    if (units >= tile_units) return true;
+    t_refused = KVMIX_ERR_SHAPE;
+    return false;
+}
+
 static bool rows_shape_ok(int64_t N) { return N == 64 || N == 128 || N == 256; }
 
 struct RowsPlan {
@@ -2552,6 +2564,7 @@ static void launch_rows_n(GemvArgs &a, int64_t samples, hipStream_t st)
     a.rows_per_split = p.rows_per_split;
     const dim3 grid((unsigned)a.splits, (unsigned)(samples / NREP), (unsigned)a.M), block(kWave, p.waves);
     if (mfma) {
+        if (!tile_fits(a.K, 128)) return;  // (a chunk past the end is moved back to end at K)
         // one A tile per wave and MFMA set; the block reduction (waves*NREP*128 floats) reuses it
         const size_t lds = (size_t)p.waves * rows_mfma_sets(NREP) * kRowsMfmaTile * sizeof(uint16_t);
         constexpr int DEPTH = 1;  // chunks in flight per wave (deeper costs occupancy and was slower)
@@ -2624,6 +2637,7 @@ static void launch_cols_cfg(const GemvArgs &a, int64_t samples, hipStream_t st)
     constexpr int VALS = Fmt<MODE>::VALS;
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / VALS;
+    if (!tile_fits(units, TU)) return;
     const int64_t tiles = (units + TU - 1) / TU;
     const int wpb = pick_waves_per_block(tiles);
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
@@ -2644,6 +2658,7 @@ static void launch_cols3_cfg(GemvArgs &a, int64_t samples, hipStream_t st, int k
 {
     constexpr int TU = (kWave / RQ) * UPL;
     const int64_t units = a.N / 11;
+    if (!tile_fits(units, TU)) return;
     const int64_t tiles = (units + TU - 1) / TU;
     constexpr int U = NREP > 1 ? kCols3HeadsU : kCols3U;  // rows in flight per lane
     a.ksplit = ks;
@@ -2669,6 +2684,7 @@ static bool cols_use_mfma(int mode, int64_t N, int64_t K)
 template <int BITS, int NREP>
 static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
 {
+    if (!tile_fits(a.N / 32, 16) || !tile_fits(a.K, 32)) return;  // a 512-code tile, a 32-row chunk
     const int64_t tiles = (a.N / 32 + 15) / 16;
     const int64_t batch = samples / NREP * a.M;
     // tiles per wave: as many as still leave one resident round of waves (4 per SIMD, 2 for
@@ -2687,6 +2703,7 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
 template <int BITS, bool NTC>
 static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
 {
+    if (!tile_fits(a.N / 32, 32) || !tile_fits(a.K, 16)) return;  // a 1024-code tile, a 16-row chunk
     const int64_t tiles = (a.N / 32 + 31) / 32;
     const int64_t batch = samples * a.M;
     // one tile per wave (several tiles per wave, so that one round of resident waves covers the problem, were
@@ -3035,6 +3052,7 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
     default: fn<30>(a, samples, st); break;                  \
     }
 
+    t_refused = KVMIX_OK;
     if (use_rows) {
         const int nrep = heads_per_block(heads_per_kv);
         const RowsPlan p = plan_rows(samples / nrep * M, K, N,
@@ -3056,6 +3074,7 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
         KVMIX_DISPATCH(launch_generic)
     }
 #undef KVMIX_DISPATCH
+    if (t_refused != KVMIX_OK) return t_refused;  // (a launcher found its kernel's tile wider than the problem)
     if (t_plan) {
         t_plan->splits = a.splits;
         t_plan->ksplit = a.ksplit;

@@ -97,3 +97,47 @@ def test_plan_reports_the_call_s_own_errors():
     assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 100, 16, 4, ctypes.byref(p)) == -3   # ..._STEPS_GROUP
     assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 128, 8, 4, ctypes.byref(p)) == -8    # ..._SHAPE
     assert L.kvmix_quantized_gemv_plan(32, 4, 0, 1, 1, 1, 128, 128, 16, 4, None) == -7              # ..._NULL
+
+
+# tile widths (in group units along N) of the tiled q.K^T kernels, from their names: a tile must fit into the row
+def _tile_units(kernel):
+    import re
+
+    m = re.match(r"gemv_cols3<(\d+),(\d+),", kernel)
+    if m:
+        return (64 // int(m.group(1))) * int(m.group(2))
+    m = re.match(r"gemv_cols<(\d+),(\d+),(\d+)>", kernel)
+    if m:
+        return (64 // int(m.group(2))) * int(m.group(3))
+    if kernel.startswith("gemv_cols_mfma2<"):
+        return 32
+    if kernel.startswith("gemv_cols_mfma<"):
+        return 16
+    return 0
+
+
+def test_no_shape_is_given_a_kernel_whose_tile_is_wider_than_the_row():
+    """A sweep of q.K^T and p.V problems through the dispatch (no launch): every one is accepted -- a launcher
+    that found its kernel's tile wider than the row, or its chunk longer than K, would make the query fail --
+    and the kernel named covers the row with whole tiles that fit into it."""
+    checked = 0
+    for bits, fmt, group, unit in ((1, REF, 32, 32), (2, REF, 32, 32), (4, REF, 32, 32), (3, REF, 11, 11), (3, DENSE3, 32, 32)):
+        for rep in (1, 4, 8):
+            for batch in (1, 2, 8, 64, 700):
+                samples = batch * 2 * rep
+                for units in (1, 2, 7, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 209, 255, 256, 257, 511, 733, 1024, 2978, 9000):
+                    tokens = units * unit
+                    for head_dim in (16, 64, 128, 256):
+                        p = _lib.gemv_plan(group, bits, fmt, samples, rep, 1, head_dim, tokens)      # q.K^T
+                        tu = _tile_units(p["kernel"])
+                        assert tu <= units, (p["kernel"], bits, fmt, samples, rep, head_dim, tokens)
+                        if p["kernel"].startswith("gemv_cols_mfma"):
+                            assert head_dim >= (16 if "mfma2" in p["kernel"] else 32)
+                        if fmt == REF and bits == 3:
+                            continue  # (values are never in the reference's 3-bit key format here)
+                        if head_dim % 32 == 0 and tokens % 8 == 0:
+                            q = _lib.gemv_plan(32, bits, fmt, samples, rep, 1, tokens, head_dim)     # p.V
+                            if q["kernel"].startswith("gemv_rows_mfma"):
+                                assert tokens >= 128, (q["kernel"], tokens)
+                        checked += 1
+    assert checked > 5000
