@@ -17,6 +17,8 @@
 //                        unaligned rows).
 //   quant_key_tokens     keys straight from the token-major fp16 tail: one thread per channel
 //                        holds one group of tokens in registers (fuses the caller's transpose).
+//   quant_key_tokens_slab  the same for D = 128 with aligned rows: a block takes a chunk of groups of 64
+//                        channels through LDS and writes each channel row's results as contiguous pieces.
 
 #include "kvmix_common.h"
 
@@ -392,7 +394,7 @@ __global__ void __launch_bounds__(256) quant_rows_ref3_f16(QuantArgs a, uint32_t
 
 // ---------------------------------------------------------------------------------------
 // keys from the token-major tail: k [outer, n, D] -> code [outer, D, n/vpw], groups of G
-// tokens per channel.  One thread per channel, one block row per (group, outer).
+// tokens per channel.  One thread per (group, channel) holds the group in registers.
 // MODE: 1, 2, 4 = reference layout bits; 3 = reference 3-bit (G must be 11); 30 = dense 3-bit.
 // ---------------------------------------------------------------------------------------
 struct KeyTokArgs {
