@@ -587,9 +587,7 @@ static int64_t fused_slabs(const kvmix_decode_attn_t *p)
 // length take the quantized positions through the matrix-core kernel (attn_slab_mfma: tiles of 1024 positions, the
 // formats of gemv_cols_mfma2 and gemv_rows_mfma) and only the fp16 tails through attn_fused_slab; everything
 // else goes through attn_fused_slab from position 0.
-#ifndef KVMIX_SLAB_MFMA_MIN_WAVES
-#define KVMIX_SLAB_MFMA_MIN_WAVES 512  // (measured: 512 waves 34 against 38 us, 256 waves 33 against 25 us)
-#endif
+constexpr int64_t kSlabMfmaMinWaves = 512;  // (measured: 512 waves 34 against 38 us, 256 waves 33 against 25 us)
 struct FusedLayout {
     bool mfma;
     int64_t tiles;       // slabs of the matrix-core kernel (first in the workspace)
@@ -607,7 +605,7 @@ static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
     if (p->k_tokens >= 1024 && p->k_tokens == p->v_tokens && (km == 1 || km == 2 || km == 4) && vm != 0 &&
         p->v_code_row_stride == kFusedD * vbits / 32 && p->v_sz_row_stride == kFusedD / 32 && p->samples <= 65535 &&
         (kFusedD + 1) * p->k_code_row_stride < (1ll << 29) && (kFusedD + 1) * p->k_sz_row_stride < (1ll << 30) &&
-        p->samples * tiles >= KVMIX_SLAB_MFMA_MIN_WAVES) {
+        p->samples * tiles >= kSlabMfmaMinWaves) {
         l.mfma = true;
         l.tiles = tiles;
         l.t_begin = p->k_tokens;

@@ -22,17 +22,9 @@
 
 #include "kvmix_common.h"
 
-#ifndef KVMIX_FLUSH_K_TILED
-#define KVMIX_FLUSH_K_TILED 1
-#endif
-#ifndef KVMIX_FLUSH_V_PIECES
-#define KVMIX_FLUSH_V_PIECES 1
-#endif
-#ifndef KVMIX_QUANT_STREAM
-#define KVMIX_QUANT_STREAM 1
-#endif
-
 namespace kvmix {
+
+constexpr int kFlushValuePieces = 1;  // value half of the fused flush: 128-bit pieces per thread (more measured no faster)
 
 struct QuantArgs {
     const void *x;
@@ -628,12 +620,12 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
         default: key_tokens_body<32, 30>(ka, gi, o, d); break;
         }
     } else {
-        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * (256 * KVMIX_FLUSH_V_PIECES) + threadIdx.x;
+        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
         switch (va.bits) {
-        case 1: rows_g32_f16_body<1, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        default: rows_g32_f16_body<4, KVMIX_FLUSH_V_PIECES, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 1: rows_g32_f16_body<1, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        default: rows_g32_f16_body<4, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
         }
     }
 }
@@ -729,7 +721,7 @@ static int launch_last_dim(const QuantArgs &a, int x_dtype, int vpw, bool fast, 
     const int64_t groups = a.steps / a.group;
     if (fast) {
         const int64_t total_groups = a.outer * a.inner * groups;
-        if (KVMIX_QUANT_STREAM && total_groups >= (int64_t)256 * 2 * 4096 && groups < (1ll << 31)) {
+        if (total_groups >= (int64_t)256 * 2 * 4096 && groups < (1ll << 31)) {
             const unsigned nb = (unsigned)((total_groups + 511) / 512);
             switch (a.bits) {
             case 1: hipLaunchKernelGGL((quant_rows_g32_f16_stream<1, 2>), dim3(nb), dim3(256), 0, st, a, (uint32_t)groups, total_groups); break;
@@ -842,7 +834,7 @@ static int setup_key_tokens(const void *k, int64_t outer, int64_t n, int64_t D, 
 
 static int launch_key_tokens(const KeyTokArgs &a, int mode, int64_t groups, int64_t outer, hipStream_t st)
 {
-    if (KVMIX_FLUSH_K_TILED && key_rows_tileable(a)) {
+    if (key_rows_tileable(a)) {
         const int64_t units = key_slab_units(mode, outer, groups);
         if (units > 0x7fffffff) return KVMIX_ERR_SHAPE;
         const dim3 grid((unsigned)units);
@@ -945,11 +937,11 @@ extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmi
         return vempty ? KVMIX_OK : launch_last_dim(va, KVMIX_F16, vpw, vfast, st);
     }
     // key slab path: D = 128, token rows 16-byte aligned
-    const int k_tiled = KVMIX_FLUSH_K_TILED && key_rows_tileable(ka);
+    const int k_tiled = key_rows_tileable(ka);
     const int64_t k_threads = kgroups * kf->outer * kf->D;
     const int64_t k_blocks = k_tiled ? key_slab_units(kmode, kf->outer, kgroups) : (k_threads + 255) / 256;
     const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
-    const int64_t v_blocks = (v_total * 4 + 256 * KVMIX_FLUSH_V_PIECES - 1) / (256 * KVMIX_FLUSH_V_PIECES);
+    const int64_t v_blocks = (v_total * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
     if (k_blocks + v_blocks > 0x7fffffff || k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
     hipLaunchKernelGGL(quant_kv_flush, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, ka, kmode, kgroups,
                        k_threads, (unsigned)k_blocks, k_tiled, va, v_groups, v_total);
