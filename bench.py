@@ -875,44 +875,37 @@ def main():
 
 
 def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H, D, T, R):
+    def extra(key, fn):
+        """One more object on the line; whatever goes wrong in it, the headline is still printed."""
+        try:
+            result[key] = fn()
+        except Exception as ex:
+            result[key] = {"error": f"{type(ex).__name__}: {ex}"}
+        torch.cuda.empty_cache()
+
+    st = torch.cuda.current_stream().cuda_stream
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(layers, kbits, vbits, B, H, D, T, R)
+        extra("cpu_baseline", lambda: cpu_baseline(layers, kbits, vbits, B, H, D, T, R))
     if not args.no_target_shape:
         # free the 32-layer cache first: the target-shape buffers need ~3 GB of their own
         for L in layers:
             L.__dict__.clear()
         torch.cuda.empty_cache()
         if not args.no_stream_ceiling:
-            res = stream_ceiling_extra(torch, _lib, lib, dev)
-            result["hbm_read_ceiling_GBps"] = max(v["GBps"] for v in res.values())
-            result["stream_ceiling"] = res
-        result["target_shape_B16_T8192"] = target_shape_extra(torch, _lib, lib, dev,
-                                                              torch.cuda.current_stream().cuda_stream)
-        torch.cuda.empty_cache()
-        result["gqa_config2_B16_T32768"] = gqa_shape_extra(torch, _lib, lib, dev,
-                                                           torch.cuda.current_stream().cuda_stream)
-        torch.cuda.empty_cache()
-    if not args.no_target_shape and not args.no_sweep:
-        result["sweep_config3_T4096"] = sweep_extra(torch, _lib, lib, dev, torch.cuda.current_stream().cuda_stream)
-    if not args.no_target_shape and not args.no_attention_step:
-        torch.cuda.empty_cache()
-        result["attention_step"] = attention_step_extra(torch, dev)
+            extra("stream_ceiling", lambda: stream_ceiling_extra(torch, _lib, lib, dev))
+            if "error" not in result["stream_ceiling"]:
+                result["hbm_read_ceiling_GBps"] = max(v["GBps"] for v in result["stream_ceiling"].values())
+        extra("target_shape_B16_T8192", lambda: target_shape_extra(torch, _lib, lib, dev, st))
+        extra("gqa_config2_B16_T32768", lambda: gqa_shape_extra(torch, _lib, lib, dev, st))
+        if not args.no_sweep:
+            extra("sweep_config3_T4096", lambda: sweep_extra(torch, _lib, lib, dev, st))
+        if not args.no_attention_step:
+            extra("attention_step", lambda: attention_step_extra(torch, dev))
     if not args.no_e2e:
-        torch.cuda.empty_cache()
-        try:
-            result["e2e_config4_llama2_7b"] = e2e_extra(torch, dev)
-        except Exception as ex:  # the headline line must still be printed
-            result["e2e_config4_llama2_7b"] = {"error": f"{type(ex).__name__}: {ex}"}
-        torch.cuda.empty_cache()
-        try:
-            result["hf_generate_config4"] = hf_generate_extra(torch, dev)
-        except Exception as ex:
-            result["hf_generate_config4"] = {"error": f"{type(ex).__name__}: {ex}"}
-        torch.cuda.empty_cache()
-        try:  # the same at batch 16, where the transformers host loop no longer hides the cache
-            result["hf_generate_config4_batch16"] = hf_generate_extra(torch, dev, batch=16)
-        except Exception as ex:
-            result["hf_generate_config4_batch16"] = {"error": f"{type(ex).__name__}: {ex}"}
+        extra("e2e_config4_llama2_7b", lambda: e2e_extra(torch, dev))
+        extra("hf_generate_config4", lambda: hf_generate_extra(torch, dev))
+        # the same at batch 16, where the transformers host loop no longer hides the cache
+        extra("hf_generate_config4_batch16", lambda: hf_generate_extra(torch, dev, batch=16))
     print(json.dumps(result))
 
 
