@@ -45,6 +45,7 @@ extern "C" {
 #define KVMIX_ERR_WORKSPACE (-11)  /* workspace smaller than kvmix_gemv_workspace_bytes() */
 #define KVMIX_ERR_LAUNCH (-12)     /* hipGetLastError() after a launch was not hipSuccess */
 #define KVMIX_ERR_STATIC_SCRATCH (-13) /* kvmix_quantized_gemv_static: problem beyond the built-in buffer */
+#define KVMIX_ERR_STATIC_LOOKUP (-14)  /* kvmix_quantized_gemv_static: the built-in buffer's address could not be obtained */
 
 #define KVMIX_F16 0
 #define KVMIX_F32 1
@@ -204,8 +205,10 @@ int kvmix_quantized_gemv_plan(int group, int bits, int fmt, int64_t samples, int
  * Same arguments minus the workspace, same kernels, same results bit for bit: the split-K partial
  * sums go to a buffer of KVMIX_GEMV_STATIC_SCRATCH_BYTES that is part of the library's device
  * image (every device the library runs on holds it until the process ends).  The call allocates
- * and frees nothing.  A problem whose kvmix_gemv_workspace_bytes() exceeds the buffer is refused
- * with KVMIX_ERR_STATIC_SCRATCH before anything is launched.  The buffer covers every q.K^T product
+ * and frees nothing.  The arguments are checked as in kvmix_quantized_gemv (same codes); then a problem whose
+ * kvmix_gemv_workspace_bytes() exceeds the buffer is refused with KVMIX_ERR_STATIC_SCRATCH before anything is
+ * launched.  Only a call whose plan splits K looks the buffer up (KVMIX_ERR_STATIC_LOOKUP if the device does not
+ * give its address).  The buffer covers every q.K^T product
  * and every p.V product with N <= 128 (at most 1.06 MiB of partial sums, reached near 120 output
  * rows of 128k tokens; launches of 1024 and more output rows need none); with N = 256 a few shapes
  * around 120 output rows of 64k and more tokens need up to 2.11 MiB and are refused.
@@ -311,6 +314,26 @@ int kvmix_decode_attention_fused(const kvmix_decode_attn_t *step, void *workspac
                                  kvmix_stream_t stream);
 
 /*
+ * How kvmix_decode_attention_fused would run a step of these sizes: which positions go through the matrix-core
+ * kernel, how the rest is cut into slabs, and the launches' geometry.  No counterpart in the reference; it needs no
+ * GPU and launches nothing (for the dispatch tests, for callers that choose between the two step forms, and for
+ * reading profiles).  Only the sizes, strides, formats and the mask / device-length pointers' being NULL or not are
+ * read from `step`; the operand pointers may be NULL.  Returns the code kvmix_decode_attention_fused would return
+ * for the same sizes (KVMIX_ERR_NULL and KVMIX_ERR_WORKSPACE aside).
+ */
+typedef struct kvmix_attn_plan {
+    int matrix;              /* 1: quantized positions [0, slab_begin) run on the matrix cores, one wave per tile */
+    int launches;            /* kernel launches of the step, the merge included */
+    int64_t matrix_tiles;    /* tiles of 1024 positions per query head (0 without the matrix-core kernel) */
+    int64_t slab_positions;  /* positions per slab of the vector-ALU slab kernel */
+    int64_t slab_begin;      /* first position those slabs cover */
+    int64_t slabs;           /* their number per query head */
+    unsigned matrix_grid[3], matrix_block[3];
+    unsigned slab_grid[3];
+} kvmix_attn_plan_t;
+int kvmix_decode_attention_fused_plan(const kvmix_decode_attn_t *step, kvmix_attn_plan_t *plan);
+
+/*
  * The tail append of a decode step fused with the rotary embedding before it: what
  * LlamaAttention_KVmix.forward does at models/modeling_llama_KVmix.py:102-112 for one new token
  * (apply_rotary_pos_emb on q and k, then torch.cat of k and v onto the fp16 tails), in one launch
@@ -365,10 +388,12 @@ int kvmix_rope_append(const kvmix_rope_append_t *step, kvmix_stream_t stream);
  *       16-byte load per lane from each of two side arrays [count][a0][a1 / 8] that follow the code
  *       array in buf (64-byte pieces per row and wave, as the scales and zeros are read).
  *       Reads count * a0 * a1 * 1.25 bytes.
+ * count >= 1, a0 >= 1 (pattern 2: >= 16), waves >= 1, else KVMIX_ERR_SHAPE.
  * bytes_per_lane in {4, 8, 16}, in_flight in {4, 8, 16}; sink: 4 writable bytes (never written
  * for a buffer that does not xor to one particular pattern).
  * flags: KVMIX_PROBE_NT non-temporal loads (pattern 2: of the code array); pattern 2 only:
- * KVMIX_PROBE_NT_SIDE the side arrays too, KVMIX_PROBE_XCD_ORDER consecutive logical blocks on one XCD,
+ * KVMIX_PROBE_NT_SIDE the side arrays too (in the burst order only: the rotating order always reads them
+ * with plain loads, as the GEMV kernels do), KVMIX_PROBE_XCD_ORDER consecutive logical blocks on one XCD,
  * KVMIX_PROBE_ROTATING the kernels' order of issue (four rows consumed, four refilled) instead of
  * 18 loads in a burst, KVMIX_PROBE_ALU(n) n = 0..15 rounds of synthetic arithmetic per four rows (a
  * round: 16 integer vector operations, four of them 32-bit multiplies, and one 4x4x4 matrix-core

@@ -8,7 +8,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libkvmix_hip.so")
+# KVMIX_HIP_LIB names another build of the same library (a build under test: its dispatch can be checked on the
+# CPU with tests/test_gemv_plan_cpu.py before it is run on a GPU)
+LIB_PATH = os.environ.get("KVMIX_HIP_LIB") or os.path.join(_HERE, "libkvmix_hip.so")
 
 OK = 0
 F16, F32 = 0, 1
@@ -31,6 +33,7 @@ EXPORTS = (
     "kvmix_decode_attention_fused_supported",
     "kvmix_decode_attention_fused_workspace_bytes",
     "kvmix_decode_attention_fused",
+    "kvmix_decode_attention_fused_plan",
     "kvmix_rope_append",
     "kvmix_probe_stream_read",
 )
@@ -96,6 +99,13 @@ class GemvPlan(ctypes.Structure):
                 ("launches", ctypes.c_int)]
 
 
+class AttnPlan(ctypes.Structure):
+    """kvmix_attn_plan_t"""
+    _fields_ = [("matrix", ctypes.c_int), ("launches", ctypes.c_int), ("matrix_tiles", ctypes.c_int64),
+                ("slab_positions", ctypes.c_int64), ("slab_begin", ctypes.c_int64), ("slabs", ctypes.c_int64),
+                ("matrix_grid", ctypes.c_uint * 3), ("matrix_block", ctypes.c_uint * 3), ("slab_grid", ctypes.c_uint * 3)]
+
+
 class KVmixLibraryMissing(ImportError):
     pass
 
@@ -142,6 +152,8 @@ def load() -> ctypes.CDLL:
     L.kvmix_decode_attention_fused_workspace_bytes.argtypes = [ctypes.POINTER(DecodeAttn)]
     L.kvmix_decode_attention_fused.restype = i32
     L.kvmix_decode_attention_fused.argtypes = [ctypes.POINTER(DecodeAttn), vp, sz, vp]
+    L.kvmix_decode_attention_fused_plan.restype = i32
+    L.kvmix_decode_attention_fused_plan.argtypes = [ctypes.POINTER(DecodeAttn), ctypes.POINTER(AttnPlan)]
     L.kvmix_rope_append.restype = i32
     L.kvmix_rope_append.argtypes = [ctypes.POINTER(RopeAppend), vp]
     L.kvmix_probe_stream_read.restype = i32
@@ -163,6 +175,45 @@ def gemv_plan(group: int, bits: int, fmt: int, samples: int, heads_per_kv: int, 
                                            sz_row_stride, ctypes.byref(plan)))
     return {"kernel": plan.kernel.decode(), "grid": tuple(plan.grid), "block": tuple(plan.block),
             "lds_bytes": plan.lds_bytes, "splits": plan.splits, "ksplit": plan.ksplit, "launches": plan.launches}
+
+
+def attn_step_descriptor(batch: int, heads: int, kv_heads: int, head_dim: int, k_bits: int, k_fmt: int, k_group: int,
+                         k_tokens: int, v_bits: int, v_fmt: int, v_group: int, v_tokens: int, k_tail_slots: int,
+                         v_tail_slots: int, k_code_row_stride: int = None, v_code_row_stride: int = None) -> DecodeAttn:
+    """A kvmix_decode_attn_t that carries the sizes of a step over dense operands and no pointers: what the
+    plan and support queries read."""
+    st = DecodeAttn()
+    D = head_dim
+    st.samples, st.heads, st.heads_per_kv, st.D = batch * heads, heads, heads // kv_heads, D
+    st.q_stride = st.out_stride = D
+    st.k_bits, st.k_fmt, st.k_group, st.k_tokens = k_bits, k_fmt, k_group, k_tokens
+    ref3 = k_bits == 3 and k_fmt == FMT_REF
+    words = k_tokens // 11 if ref3 else k_tokens * k_bits // 32
+    st.k_code_row_stride = words if k_code_row_stride is None else k_code_row_stride
+    st.k_code_batch_stride = D * st.k_code_row_stride
+    st.k_sz_row_stride = k_tokens // (11 if ref3 else max(k_group, 1))
+    st.k_sz_batch_stride = D * st.k_sz_row_stride
+    st.v_bits, st.v_fmt, st.v_group, st.v_tokens = v_bits, v_fmt, v_group, v_tokens
+    st.v_code_row_stride = D * v_bits // 32 if v_code_row_stride is None else v_code_row_stride
+    st.v_code_batch_stride = v_tokens * st.v_code_row_stride
+    st.v_sz_row_stride = D // max(v_group, 1)
+    st.v_sz_batch_stride = v_tokens * st.v_sz_row_stride
+    for prefix, slots in (("k", k_tail_slots), ("v", v_tail_slots)):
+        setattr(st, prefix + "_tail_slots", slots)
+        setattr(st, prefix + "_tail_len", slots)
+        setattr(st, prefix + "_tail_token_stride", D)
+        setattr(st, prefix + "_tail_batch_stride", slots * D)
+    return st
+
+
+def attn_plan(step: DecodeAttn) -> dict:
+    """kvmix_decode_attention_fused_plan as a dict (raises on the codes the step itself would return).  Needs no GPU."""
+    plan = AttnPlan()
+    check(load().kvmix_decode_attention_fused_plan(ctypes.byref(step), ctypes.byref(plan)))
+    return {"matrix": bool(plan.matrix), "launches": plan.launches, "matrix_tiles": plan.matrix_tiles,
+            "slab_positions": plan.slab_positions, "slab_begin": plan.slab_begin, "slabs": plan.slabs,
+            "matrix_grid": tuple(plan.matrix_grid), "matrix_block": tuple(plan.matrix_block),
+            "slab_grid": tuple(plan.slab_grid)}
 
 
 def strerror(code: int) -> str:

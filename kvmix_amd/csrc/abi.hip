@@ -24,8 +24,10 @@ extern "C" const char *kvmix_strerror(int code)
     case KVMIX_ERR_LAUNCH: return "kernel launch failed";
     case KVMIX_ERR_STATIC_SCRATCH:
         return "problem needs more split-K scratch than kvmix_quantized_gemv_static's built-in buffer holds "
-               "(KVMIX_GEMV_STATIC_SCRATCH_BYTES), or that buffer's address could not be obtained on this device: "
-               "use kvmix_quantized_gemv with a caller-owned workspace";
+               "(KVMIX_GEMV_STATIC_SCRATCH_BYTES): use kvmix_quantized_gemv with a caller-owned workspace";
+    case KVMIX_ERR_STATIC_LOOKUP:
+        return "the address of kvmix_quantized_gemv_static's built-in buffer could not be obtained on this device "
+               "(hipGetSymbolAddress failed): use kvmix_quantized_gemv with a caller-owned workspace";
     default: return "unknown kvmix error";
     }
 }

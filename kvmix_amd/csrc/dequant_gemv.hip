@@ -101,10 +101,20 @@ struct GemvArgs {
 // registers per load, formed by vector-ALU adds; here the row arithmetic runs on the scalar unit and costs
 // the vector ALU nothing.  Offsets are 32-bit: the host only sends problems whose (batch, kv-head)
 // slice stays below 2^32 bytes to the kernels that use this.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const void *base)
+// `bytes` is the extent of the slice (from its first byte to the end of its last row): the descriptor's
+// num_records.  The hardware compares every dword's byte offset with it and returns zero for a dword at or past
+// it, so a wave that were handed a tile outside its operand would compute with zeros instead of touching memory
+// that is not the caller's -- the kernels' own index arithmetic never goes there, this is the second fence.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const void *base, uint32_t bytes)
 {
-    // raw buffer, no stride, no bounds (num_records = 2^32 - 1 bytes), 32-bit data format
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)0xffffffffu, 0x00020000);
+    // raw buffer, no stride, 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+// extent in bytes of one (batch, kv-head) slice of `rows` rows at a pitch of `row_stride` elements of `elem_bytes`
+// bytes, the last row holding `row_elems` of them
+__device__ __forceinline__ uint32_t slice_bytes(int64_t rows, int64_t row_stride, int64_t row_elems, int elem_bytes)
+{
+    return rows > 0 ? (uint32_t)(((rows - 1) * row_stride + row_elems) * elem_bytes) : 0u;
 }
 template <typename T, bool NT>
 __device__ __forceinline__ T ld_buffer(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_bytes, uint32_t wave_bytes)
@@ -458,9 +468,10 @@ __global__ void __launch_bounds__(64 * kColsWaves) gemv_cols(GemvArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int K = (int)a.K;
     const int nunits = (int)(a.N / VALS);
+    if (nunits < TU) return;                    // (never launched so: a tile wider than the row would leave the operand)
     int t0 = (int)(bx * blockDim.y + wy) * TU;  // first unit of this wave's tile
     if (t0 >= nunits) return;                   // whole wave outside (no block barrier below)
-    t0 = t0 + TU <= nunits ? t0 : nunits - TU;  // last tile: shifted left, still whole
+    t0 = t0 + TU <= nunits ? t0 : max(nunits - TU, 0);  // last tile: shifted left, still whole
     const int unit0 = t0 + gl * UPL;            // this lane's first unit
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
 
@@ -642,6 +653,7 @@ gemv_cols3(GemvArgs a)
     const int64_t kv = sample0 / a.heads_per_kv;
     const int K = (int)a.K;
     const int nunits = (int)(a.N / VALS);
+    if (nunits < TU) return;  // (never launched so: a tile wider than the row would leave the operand; the same for every thread)
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample0 * a.x_bs + m * a.x_rs;
     for (int i = wy * kWave + lane; i < NREP * (K + 1); i += blockDim.y * kWave) {
@@ -660,7 +672,7 @@ gemv_cols3(GemvArgs a)
         if (ks > 1) __syncthreads();  // (the barrier of the combine step)
         return;
     }
-    t0 = t0 + TU <= nunits ? t0 : nunits - TU;
+    t0 = t0 + TU <= nunits ? t0 : max(nunits - TU, 0);
     const int unit0 = t0 + gl * UPL;
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
     const uint32_t *cp = a.code + kv * a.c_bs + unit0;
@@ -1235,6 +1247,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     // chunk repeats meet x == 0.  A chunk wholly past the end is all zeros.
     // The wave index is made scalar so that the loop is uniform control flow.
     const int ke32 = (int)kend;
+    if (a.K < CH) return;  // (never launched so: a chunk longer than K would leave the operand; the same for every thread)
     const int stride = KW * CH;
     const int kfirst = (int)kbeg + __builtin_amdgcn_readfirstlane(wy) * CH;
     struct __attribute__((packed, aligned(2))) Half2x {
@@ -1245,7 +1258,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     Half2x xh[DEPTH][NREP];
     Elem w[DEPTH][KB][4];
 
-    auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : ke32 - CH; };
+    auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : max(ke32 - CH, 0); };
     auto load_small = [&](int d, int k0) {
         const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
         s8[d] = ld_stream<Half8>(sp + kr * LPR);
@@ -1495,6 +1508,7 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     // one (recomputed, stored twice with identical values): uniform control flow, no branches.
     const int tpw = a.splits;
     const int tile0 = (int)bx * tpw * nw + wy;
+    if (ngroups < TG || K < CH) return;  // (never launched so: a tile wider than the row, a chunk longer than K)
     if (tile0 * TG >= ngroups) return;  // (no block barrier below)
     const int nch = (K + CH - 1) / CH;
     const int items = tpw * nch;        // (tile, chunk) pairs of this wave, in order
@@ -1536,10 +1550,10 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     // item -> first group of its tile, first row of its chunk (moved back to end at K)
     auto tile_g0 = [&](int it) {
         const int g = (tile0 + (it / nch) * nw) * TG;
-        return g + TG <= ngroups ? g : ngroups - TG;
+        return g + TG <= ngroups ? g : max(ngroups - TG, 0);
     };
     auto chunk_k0 = [&](int it) { return (it % nch) * CH; };
-    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
+    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : max(K - CH, 0); };
     auto load_small = [&](int it) {
         const uint32_t d = (uint32_t)(chunk_base(chunk_k0(it)) + srow);
         const uint32_t off = d * s_rs + (uint32_t)tile_g0(it);
@@ -1726,6 +1740,7 @@ gemv_cols_mfma2(GemvArgs a)
     const int slice = wy % ks;
     const int ntw = nw / ks;            // tiles a block works on at a time
     const int tile0 = (int)bx * ntw + wy / ks;   // one tile per wave
+    if (ngroups < TG || K < CH) return;  // (never launched so: a tile wider than the row, a chunk longer than K; the same for every thread)
     if (tile0 * TG >= ngroups) {
         if (ks > 1) __syncthreads();    // (the one block barrier of finish_tile)
         return;
@@ -1738,9 +1753,10 @@ gemv_cols_mfma2(GemvArgs a)
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
     // buffer descriptors of this (batch, kv-head) slice; a lane's two elements are 2 * BITS bytes
-    const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.code + kv * a.c_bs);
-    const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.scale + kv * a.s_bs);
-    const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.zero + kv * a.s_bs);
+    const uint32_t sz_bytes = slice_bytes(K, a.s_rs, ngroups, 2);
+    const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.code + kv * a.c_bs, slice_bytes(K, a.c_rs, (int64_t)ngroups * BITS, 4));
+    const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.scale + kv * a.s_bs, sz_bytes);
+    const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.zero + kv * a.s_bs, sz_bytes);
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
     const int sub = lane % 4;   // staging: row lane/4 of the chunk, groups 8*sub .. 8*sub+7
     const int srow = lane / 4;
@@ -1772,10 +1788,10 @@ gemv_cols_mfma2(GemvArgs a)
     uint32_t w[KB][4][WL];
 
     // the last tile of a row is moved back to end at N
-    const int g_first = tile0 * TG + TG <= ngroups ? tile0 * TG : ngroups - TG;
+    const int g_first = tile0 * TG + TG <= ngroups ? tile0 * TG : max(ngroups - TG, 0);
     auto tile_g0 = [&](int) { return g_first; };
     auto chunk_k0 = [&](int it) { return (ch0 + it) * CH; };
-    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : K - CH; };
+    auto chunk_base = [&](int k0) { return k0 + CH <= K ? k0 : max(K - CH, 0); };
     auto load_small = [&](int it) {
         const uint32_t d0 = (uint32_t)chunk_base(chunk_k0(it));
         const uint32_t off = 2u * (d0 * s_rs + (uint32_t)tile_g0(it));  // bytes, the same for every lane
@@ -2003,8 +2019,9 @@ attn_slab_mfma(AttnSlabArgs a)
     const int64_t kv = sample / a.heads_per_kv;
     const int ngroups = (int)(a.tokens / 32);
     const int tile = (int)bx * nw + wy;
+    if (ngroups < TG) return;  // (never launched so: a slab longer than the row would leave the operands)
     if (tile * TG >= ngroups) return;
-    const int g_first = tile * TG + TG <= ngroups ? tile * TG : ngroups - TG;  // (the last tile ends at `tokens`)
+    const int g_first = tile * TG + TG <= ngroups ? tile * TG : max(ngroups - TG, 0);  // (the last tile ends at `tokens`)
     const int shift = tile * TG - g_first;                                     // its first groups are the neighbour's
     float slab_m, slab_l;
 
@@ -2016,9 +2033,10 @@ attn_slab_mfma(AttnSlabArgs a)
         constexpr bool SPLIT = BITS == 4;
         float *zl = reinterpret_cast<float *>(atile + AT);
         const uint16_t *xp = a.q + sample * a.q_bs;
-        const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.k_code + kv * a.kc_bs);
-        const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.k_scale + kv * a.ksz_bs);
-        const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.k_zero + kv * a.ksz_bs);
+        const uint32_t sz_bytes = slice_bytes(K, a.ksz_rs, ngroups, 2);
+        const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.k_code + kv * a.kc_bs, slice_bytes(K, a.kc_rs, (int64_t)ngroups * BITS, 4));
+        const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.k_scale + kv * a.ksz_bs, sz_bytes);
+        const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.k_zero + kv * a.ksz_bs, sz_bytes);
         const uint32_t c_rs = (uint32_t)a.kc_rs, s_rs = (uint32_t)a.ksz_rs;
         const int sub = lane % 4, srow = lane / 4, j4 = lane % 4;
         const uint32_t c_lane = SPLIT ? (uint32_t)lane * 4u : (uint32_t)lane * (2 * BITS);
@@ -2226,7 +2244,7 @@ attn_slab_mfma(AttnSlabArgs a)
         Half8 s8, z8;
         Elem w[KB][4];
         // (a chunk past the slab's end -- the prefetch of the last step -- is the last chunk again)
-        auto chunk_base = [&](int k0) { return k0 + CH <= t_end ? k0 : t_end - CH; };
+        auto chunk_base = [&](int k0) { return k0 + CH <= t_end ? k0 : max(t_end - CH, 0); };
         auto load_small = [&](int k0) {
             const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
             s8 = ld_stream<Half8>(sp + kr * LPR);
@@ -2738,12 +2756,23 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
         launch_cols_mfma2_nt<BITS, false>(a, samples, st);
 }
 
+int plan_attn_slab_mfma(int64_t tokens, int64_t samples, unsigned grid[3], unsigned block[3])
+{
+    const int64_t tiles = (tokens / 32 + 31) / 32;
+    if (tokens < 1024 || tokens % 32 != 0 || samples <= 0 || samples > 65535 || tiles > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    const int wpb = pick_waves_per_block(tiles);
+    grid[0] = (unsigned)((tiles + wpb - 1) / wpb), grid[1] = (unsigned)samples, grid[2] = 1;
+    block[0] = kWave, block[1] = (unsigned)wpb, block[2] = 1;
+    return KVMIX_OK;
+}
+
 int launch_attn_slab_mfma(const AttnSlabArgs &a, int k_bits, int v_mode, int64_t samples, hipStream_t stream)
 {
-    const int64_t tiles = (a.tokens / 32 + 31) / 32;
-    if (a.tokens < 1024 || a.tokens % 32 != 0 || samples <= 0 || samples > 65535 || tiles > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    const int wpb = pick_waves_per_block(tiles);
-    const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples), block(kWave, wpb);
+    unsigned g[3], b[3];
+    const int prc = plan_attn_slab_mfma(a.tokens, samples, g, b);
+    if (prc != KVMIX_OK) return prc;
+    const int wpb = (int)b[1];
+    const dim3 grid(g[0], g[1]), block(b[0], b[1]);
     const size_t lds = (size_t)wpb * kSlabLds;
 #define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_slab_mfma<KB_, VM_>), grid, block, lds, stream, a)
 #define KVMIX_SLAB_V(KB_)                          \
@@ -2938,13 +2967,11 @@ extern "C" int kvmix_quantized_gemv_static(int group, const void *x, int64_t x_b
                                            int64_t out_batch_stride, int64_t out_row_stride,
                                            kvmix_stream_t stream)
 {
-    // the documented bound, not the launch plan's exact need: what is refused depends on sizes only
-    if (kvmix_gemv_workspace_bytes(samples, M, K, N) > KVMIX_GEMV_STATIC_SCRATCH_BYTES) return KVMIX_ERR_STATIC_SCRATCH;
-    void *ws = static_scratch();
-    if (!ws) return KVMIX_ERR_STATIC_SCRATCH;
+    // (the arguments are checked first, as in kvmix_quantized_gemv; the buffer is looked up only by a call whose
+    // plan splits K, so q.K^T products and unsplit batches never touch the lock or the symbol)
     return quantized_gemv(group, x, x_batch_stride, x_row_stride, code, code_batch_stride, code_row_stride, scale,
                           zero, sz_batch_stride, sz_row_stride, bits, fmt, samples, heads_per_kv, M, K, N, out,
-                          out_batch_stride, out_row_stride, ws, KVMIX_GEMV_STATIC_SCRATCH_BYTES, true, stream);
+                          out_batch_stride, out_row_stride, nullptr, 0, true, stream);
 }
 
 static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
@@ -2979,6 +3006,10 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
     const int64_t words = N / unit_vals * unit_words, groups = N / group;
     if (code_row_stride < words || sz_row_stride < groups || x_row_stride < K || out_row_stride < N)
         return KVMIX_ERR_SHAPE;
+    // the built-in buffer: the documented bound, not the launch plan's exact need -- what is refused depends on
+    // the sizes only
+    if (workspace_is_static && kvmix_gemv_workspace_bytes(samples, M, K, N) > KVMIX_GEMV_STATIC_SCRATCH_BYTES)
+        return KVMIX_ERR_STATIC_SCRATCH;
     // grid.y / grid.z hold at most 65535 blocks: a larger batch goes out as several launches of nearly equal
     // size over whole kv heads (and whole groups of M rows), one after the other on the stream.  (Each part
     // then still has more than 30000 output rows, which no kernel splits over blocks: no workspace.)
@@ -3057,10 +3088,15 @@ static int quantized_gemv(int group, const void *x, int64_t x_batch_stride,
         const int nrep = heads_per_block(heads_per_kv);
         const RowsPlan p = plan_rows(samples / nrep * M, K, N,
                                      rows_max_waves(rows_use_mfma(mode, N, K, code_row_stride), nrep));
-        if (p.splits > 1) {
+        if (p.splits > 1 && !t_plan) {
             const size_t need = (size_t)(samples * M) * (size_t)p.splits * (size_t)N * sizeof(float);
-            if (!t_plan && (!workspace || workspace_bytes < need))
-                return workspace_is_static ? KVMIX_ERR_STATIC_SCRATCH : KVMIX_ERR_WORKSPACE;
+            if (workspace_is_static) {
+                if (need > KVMIX_GEMV_STATIC_SCRATCH_BYTES) return KVMIX_ERR_STATIC_SCRATCH;
+                a.partial = (float *)static_scratch();
+                if (!a.partial) return KVMIX_ERR_STATIC_LOOKUP;
+            } else if (!workspace || workspace_bytes < need) {
+                return KVMIX_ERR_WORKSPACE;
+            }
         }
         switch (mode) {
         case 1: launch_rows<1>(a, samples, st); break;

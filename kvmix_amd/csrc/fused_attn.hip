@@ -605,6 +605,8 @@ static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
     if (p->k_tokens >= 1024 && p->k_tokens == p->v_tokens && (km == 1 || km == 2 || km == 4) && vm != 0 &&
         p->v_code_row_stride == kFusedD * vbits / 32 && p->v_sz_row_stride == kFusedD / 32 && p->samples <= 65535 &&
         (kFusedD + 1) * p->k_code_row_stride < (1ll << 29) && (kFusedD + 1) * p->k_sz_row_stride < (1ll << 30) &&
+        // (the value phase forms 32-bit byte offsets of code rows and 32-bit element offsets of scale rows)
+        p->v_tokens * p->v_code_row_stride < (1ll << 30) && p->v_tokens * p->v_sz_row_stride < (1ll << 31) &&
         p->samples * tiles >= kSlabMfmaMinWaves) {
         l.mfma = true;
         l.tiles = tiles;
@@ -629,8 +631,9 @@ extern "C" size_t kvmix_decode_attention_fused_workspace_bytes(const kvmix_decod
     return (size_t)p->samples * (size_t)fused_layout(p).slabs() * (kFusedD + 2) * sizeof(float);
 }
 
-extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *workspace, size_t workspace_bytes,
-                                            kvmix_stream_t stream)
+// the argument checks of kvmix_decode_attention_fused; `pointers`: also that the operands are there (the plan query
+// passes sizes only)
+static int fused_check(const kvmix_decode_attn_t *p, bool pointers)
 {
     if (!p) return KVMIX_ERR_NULL;
     if (p->samples < 0 || p->D <= 0 || p->k_tokens < 0 || p->v_tokens < 0 || p->k_tail_slots < 0 || p->v_tail_slots < 0 ||
@@ -644,27 +647,66 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
     if (width == 0) return KVMIX_ERR_SHAPE;
     if (!p->k_tail_len_dev && !p->v_tail_len_dev && p->k_tokens + p->k_tail_len != p->v_tokens + p->v_tail_len)
         return KVMIX_ERR_SHAPE;
-    if (!p->q || !p->out) return KVMIX_ERR_NULL;
-    if ((p->k_tail_slots > 0 && !p->k_tail) || (p->v_tail_slots > 0 && !p->v_tail)) return KVMIX_ERR_NULL;
+    if (pointers) {
+        if (!p->q || !p->out) return KVMIX_ERR_NULL;
+        if ((p->k_tail_slots > 0 && !p->k_tail) || (p->v_tail_slots > 0 && !p->v_tail)) return KVMIX_ERR_NULL;
+    }
     if (p->out_stride < p->D || p->q_stride < p->D || (p->mask && p->mask_stride < width)) return KVMIX_ERR_SHAPE;
     if ((p->k_tail_slots > 0 && p->k_tail_token_stride < p->D) || (p->v_tail_slots > 0 && p->v_tail_token_stride < p->D))
         return KVMIX_ERR_SHAPE;
-    const int k_mode = fused_key_mode(p), v_mode = fused_value_mode(p);
+    const int k_mode = fused_key_mode(p);
     if (p->k_tokens > 0) {
-        if (!p->k_code || !p->k_scale || !p->k_zero) return KVMIX_ERR_NULL;
+        if (pointers && (!p->k_code || !p->k_scale || !p->k_zero)) return KVMIX_ERR_NULL;
         const int64_t unit = k_mode == 3 ? 11 : 32;
         if (p->k_tokens % unit != 0) return KVMIX_ERR_SHAPE;
         const int64_t words = k_mode == 3 ? p->k_tokens / 11 : p->k_tokens * (k_mode == 30 ? 3 : k_mode) / 32;
         if (p->k_code_row_stride < words || p->k_sz_row_stride < p->k_tokens / unit) return KVMIX_ERR_SHAPE;
     }
     if (p->v_tokens > 0) {
-        if (!p->v_code || !p->v_scale || !p->v_zero) return KVMIX_ERR_NULL;
+        if (pointers && (!p->v_code || !p->v_scale || !p->v_zero)) return KVMIX_ERR_NULL;
         if (p->v_code_row_stride < kFusedD * p->v_bits / 32 || p->v_sz_row_stride < kFusedD / 32) return KVMIX_ERR_SHAPE;
     }
     const FusedLayout lay = fused_layout(p);
     const int64_t slabs = lay.slabs();
-    const int64_t kv_samples = p->samples / p->heads_per_kv;
     if (slabs > 0x7fffffff || slabs * p->samples > 0x7fffffff) return KVMIX_ERR_SHAPE;  // (blocks of one launch)
+    return KVMIX_OK;
+}
+
+extern "C" int kvmix_decode_attention_fused_plan(const kvmix_decode_attn_t *p, kvmix_attn_plan_t *plan)
+{
+    if (!plan) return KVMIX_ERR_NULL;
+    *plan = kvmix_attn_plan_t{};
+    const int rc = fused_check(p, false);
+    if (rc != KVMIX_OK || p->samples == 0) return rc;
+    const FusedLayout lay = fused_layout(p);
+    plan->matrix = lay.mfma ? 1 : 0;
+    plan->matrix_tiles = lay.tiles;
+    plan->slab_positions = fused_slab(p);
+    plan->slab_begin = lay.t_begin;
+    plan->slabs = lay.tail_slabs;
+    if (lay.mfma) {
+        const int prc = plan_attn_slab_mfma(p->k_tokens, p->samples, plan->matrix_grid, plan->matrix_block);
+        if (prc != KVMIX_OK) return prc;
+        plan->launches++;
+    }
+    if (lay.tail_slabs > 0) {
+        plan->slab_grid[0] = (unsigned)(lay.tail_slabs * p->samples);
+        plan->slab_grid[1] = plan->slab_grid[2] = 1;
+        plan->launches++;
+    }
+    if (!(lay.slabs() == 1 && !lay.mfma)) plan->launches++;  // the merge
+    return KVMIX_OK;
+}
+
+extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *workspace, size_t workspace_bytes,
+                                            kvmix_stream_t stream)
+{
+    const int chk = fused_check(p, true);
+    if (chk != KVMIX_OK || p->samples == 0) return chk;
+    const int k_mode = fused_key_mode(p), v_mode = fused_value_mode(p);
+    const FusedLayout lay = fused_layout(p);
+    const int64_t slabs = lay.slabs();
+    const int64_t kv_samples = p->samples / p->heads_per_kv;
     if (!workspace || workspace_bytes < kvmix_decode_attention_fused_workspace_bytes(p)) return KVMIX_ERR_WORKSPACE;
 
     FusedArgs a;

@@ -227,10 +227,13 @@ extern "C" int kvmix_probe_stream_read(const void *buf, int pattern, int64_t a0,
 {
     if (!buf || !sink) return KVMIX_ERR_NULL;
     if (pattern == 2) {
+        // (count, a0 and waves are checked like those of patterns 0 and 1: the kernel redirects rows past the end
+        // to rows - 1 and rows - 16, and the grid is ceil(pieces / waves))
         // a0 = rows (multiple of 16), a1 = row bytes (multiple of 8, at least 512); side arrays of a1 / 8 bytes per
         // row follow the code array in buf; in_flight and bytes_per_lane are ignored
         const int64_t side_row = a1 / 8;
-        if (a0 % 16 != 0 || a1 % 8 != 0 || a1 < 512 || side_row < 64 || side_row % 2 != 0 || count > 65535 || waves > 4)
+        if (count <= 0 || a0 < 16 || waves < 1 || waves > 4) return KVMIX_ERR_SHAPE;
+        if (a0 % 16 != 0 || a1 % 8 != 0 || a1 < 512 || side_row < 64 || side_row % 2 != 0 || count > 65535)
             return KVMIX_ERR_SHAPE;
         const uint8_t *b = (const uint8_t *)buf;
         const uint8_t *s0 = b + (int64_t)count * a0 * a1, *s1 = s0 + (int64_t)count * a0 * side_row;

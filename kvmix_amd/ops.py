@@ -281,12 +281,10 @@ def quantized_gemm(group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: 
 # (measured on MI355X, Llama-2-7B heads: 12-20 us against 20-30 us at 1-4 sequences of 2k-4k tokens;
 # equal at about 2^19 entries, i.e. 1024 blocks).  Keys in the reference's 3-bit words break even earlier.
 # Beyond that it is the faster one again where the library runs the quantized positions on the matrix cores
-# (keys and values quantized to the same length of at least 1024, keys of 1, 2 or 4 bits; at least
-# SINGLE_PASS_MATRIX_MIN_WAVES (query head, 1024-position tile) pairs): 16 x 8k 120 against 131 us, 4 x 8k 40
-# against 51 us.
+# (16 x 8k 120 against 131 us, 4 x 8k 40 against 51 us); which steps those are is the library's decision and is
+# asked of it (kvmix_decode_attention_fused_plan), not repeated here.
 SINGLE_PASS_MAX_ENTRIES = 1 << 19
 SINGLE_PASS_MAX_ENTRIES_REF3 = 360_000
-SINGLE_PASS_MATRIX_MIN_WAVES = 512
 
 
 def prefer_single_pass(batch: int, heads: int, kv_heads: int, head_dim: int, width: int, k_bits: int, k_fmt: int,
@@ -294,17 +292,23 @@ def prefer_single_pass(batch: int, heads: int, kv_heads: int, head_dim: int, wid
                        v_tokens: int = None) -> bool:
     """Policy for callers that do not need the probabilities: whether the single-pass step is both
     available for this layout and the faster of the two at this size.  k_tokens / v_tokens: the quantized
-    lengths, where the caller knows them (they decide whether a large step can use the matrix cores)."""
+    lengths, where the caller knows them (they decide whether a large step can use the matrix cores: the
+    library is asked, kvmix_decode_attention_fused_plan)."""
     if kv_heads <= 0 or heads % kv_heads != 0:
         return False
+    if not single_pass_supported(head_dim, heads // kv_heads, k_bits, k_fmt, k_group, v_bits, v_fmt, v_group):
+        return False
     limit = SINGLE_PASS_MAX_ENTRIES_REF3 if (k_bits == 3 and k_fmt == _lib.FMT_REF) else SINGLE_PASS_MAX_ENTRIES
-    if batch * heads * width > limit:
-        matrix = (k_tokens is not None and k_tokens == v_tokens and k_tokens >= 1024 and head_dim == 128
-                  and k_bits in (1, 2, 4) and k_fmt == _lib.FMT_REF and k_group == 32 and batch * heads <= 65535
-                  and batch * heads * ((k_tokens + 1023) // 1024) >= SINGLE_PASS_MATRIX_MIN_WAVES)
-        if not matrix:
-            return False
-    return single_pass_supported(head_dim, heads // kv_heads, k_bits, k_fmt, k_group, v_bits, v_fmt, v_group)
+    if batch * heads * width <= limit:
+        return True
+    if k_tokens is None or v_tokens is None or width < max(k_tokens, v_tokens):
+        return False
+    step = _lib.attn_step_descriptor(batch, heads, kv_heads, head_dim, k_bits, k_fmt, k_group, k_tokens, v_bits, v_fmt,
+                                     v_group, v_tokens, width - k_tokens, width - v_tokens)
+    try:
+        return _lib.attn_plan(step)["matrix"]
+    except RuntimeError:
+        return False
 
 
 def rope_append(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int, kv_heads: int,

@@ -45,8 +45,9 @@ def test_version_and_error_text(lib):
     assert "divisible by group_length" in _lib.strerror(-3)
     assert "32 / quant_bits" in _lib.strerror(-4)
     assert "divisible by KV heads" in _lib.strerror(-5)
-    codes = {_lib.strerror(c) for c in range(-12, 0)}
-    assert len(codes) == 12  # distinct text per code
+    codes = {_lib.strerror(c) for c in range(-14, 0)}
+    assert len(codes) == 14  # distinct text per code
+    assert "built-in buffer" in _lib.strerror(-13) and "hipGetSymbolAddress" in _lib.strerror(-14)
     with pytest.raises(RuntimeError, match="KV heads"):
         _lib.check(-5)
 

@@ -141,3 +141,63 @@ def test_no_shape_is_given_a_kernel_whose_tile_is_wider_than_the_row():
                                 assert tokens >= 128, (q["kernel"], tokens)
                         checked += 1
     assert checked > 5000
+
+
+# ---- the single-pass attention step's plan (kvmix_decode_attention_fused_plan: no launch, no GPU) ----
+
+def _step(batch, heads, kv_heads, k_bits, k_fmt, k_tokens, v_bits, v_fmt, v_tokens, width, **kw):
+    k_group = 11 if (k_bits == 3 and k_fmt == REF) else 32
+    return _lib.attn_step_descriptor(batch, heads, kv_heads, 128, k_bits, k_fmt, k_group, k_tokens, v_bits, v_fmt, 32,
+                                     v_tokens, width - k_tokens, width - v_tokens, **kw)
+
+
+def test_attention_step_plans_of_the_measured_shapes():
+    # B = 16, T = 8192, 4-bit keys and values quantized to the same length: matrix cores over [0, 8064), the two
+    # 128-token fp16 tails as one further slab, and the merge
+    p = _lib.attn_plan(_step(16, 32, 32, 4, REF, 8064, 4, REF, 8064, 8192))
+    assert p["matrix"] and p["matrix_tiles"] == 8 and p["slab_begin"] == 8064 and p["slabs"] == 1 and p["launches"] == 3
+    assert p["matrix_grid"][:2] == (2, 512) and p["matrix_block"] == (64, 4, 1)
+    # configs[4]'s size: the vector-ALU slab kernel from position 0
+    p = _lib.attn_plan(_step(4, 32, 32, 4, REF, 2176, 4, REF, 2176, 2304))
+    assert not p["matrix"] and p["slab_begin"] == 0 and p["slabs"] == 5 and p["launches"] == 2
+    # one slab: the slab kernel stores the result itself
+    p = _lib.attn_plan(_step(8, 32, 32, 2, REF, 384, 2, REF, 384, 512))
+    assert not p["matrix"] and p["slabs"] == 1 and p["launches"] == 1
+
+
+def test_no_attention_step_is_given_a_tile_longer_than_its_quantized_part():
+    """A sweep of step sizes through the plan query: wherever the matrix-core kernel is chosen, its 1024-position
+    tiles fit into the quantized part, that part is whole groups, the grid covers every tile with no more than
+    65535 rows, and the vector-ALU slabs cover every position from where the tiles end."""
+    checked = 0
+    for k_bits, k_fmt in ((1, REF), (2, REF), (4, REF), (3, REF), (3, DENSE3)):
+        unit = 11 if (k_bits == 3 and k_fmt == REF) else 32
+        for v_bits, v_fmt in ((1, REF), (2, REF), (4, REF), (3, DENSE3)):
+            for batch, heads, kv_heads in ((1, 32, 32), (4, 32, 8), (16, 32, 32), (64, 32, 32), (2100, 32, 32)):
+                for units in (0, 1, 3, 31, 32, 33, 63, 64, 93, 252, 1000):
+                    for tail in (0, 1, 32, 128):
+                        for dv in (0, 32, -32):
+                            k_tokens = units * unit
+                            v_tokens = max(k_tokens // 32 * 32 + dv, 0) if unit == 32 else max((k_tokens + tail) // 32 * 32 + dv, 0)
+                            width = max(k_tokens, v_tokens) + tail
+                            if width == 0:
+                                continue
+                            st = _step(batch, heads, kv_heads, k_bits, k_fmt, k_tokens, v_bits, v_fmt, v_tokens, width)
+                            plan = _lib.AttnPlan()
+                            rc = _lib.load().kvmix_decode_attention_fused_plan(ctypes.byref(st), ctypes.byref(plan))
+                            if batch * heads * ((width + 511) // 512) > 0x7fffffff:
+                                assert rc == -8
+                                continue
+                            assert rc == 0, (rc, k_bits, k_fmt, v_bits, batch, k_tokens, v_tokens, width)
+                            if plan.matrix:
+                                assert k_tokens >= 1024 and k_tokens % 32 == 0 and k_tokens == v_tokens
+                                assert batch * heads <= 65535
+                                assert plan.matrix_tiles == (k_tokens + 1023) // 1024
+                                assert plan.matrix_grid[0] * plan.matrix_block[1] >= plan.matrix_tiles
+                                assert plan.matrix_grid[1] == batch * heads and 1 <= plan.matrix_block[1] <= 4
+                                assert plan.slab_begin == k_tokens
+                            else:
+                                assert plan.slab_begin == 0 and plan.matrix_tiles == 0
+                            assert plan.slab_begin + plan.slabs * plan.slab_positions >= width
+                            checked += 1
+    assert checked > 5000

@@ -91,3 +91,45 @@ def test_static_scratch_rejects_oversized_problem(dev):
         assert rc == -13
         assert "built-in buffer" in _lib.strerror(rc)
         torch.cuda.synchronize()
+
+
+def test_static_scratch_gemv_allocates_nothing_and_replays_from_a_graph(oracle, dev):
+    """What the entry point promises: after one warm call (the buffer's address is looked up then) further calls
+    leave the device's free memory and torch's allocator untouched; and a call recorded into a HIP graph -- where an
+    allocation would fail the capture -- replays to the eager result, every time."""
+    from kvmix_amd import _lib
+
+    L = _lib.load()
+    bits, g, B, nh, nkv, K, N = 4, 32, 1, 16, 16, 4096 + 32, 128    # a p.V product that is split over K
+    assert L.kvmix_gemv_workspace_bytes(B * nh, 1, K, N) > 0
+    with torch.cuda.device(dev):
+        dv, want64, abs64 = _operands(oracle, dev, bits, g, B, nh, nkv, K, N, seed=7)
+        x, code, scale, zero = dv
+        out = torch.full((B, nh, 1, N), float("nan"), dtype=torch.float16, device=dev)
+        head = (g, x.data_ptr(), K, K, code.data_ptr(), code.stride(1), code.stride(2), scale.data_ptr(), zero.data_ptr(),
+                scale.stride(1), scale.stride(2), bits, 0, B * nh, nh // nkv, 1, K, N, out.data_ptr(), N, N)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        assert L.kvmix_quantized_gemv_static(*head, stream) == 0     # warm: symbol lookup, kernel attributes
+        torch.cuda.synchronize()
+        eager = out.clone()
+        ok, worst = gemv_close(eager.cpu().numpy(), want64, abs64)
+        assert ok, worst
+        free0, alloc0, reserved0 = torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev)
+        for _ in range(3):
+            assert L.kvmix_quantized_gemv_static(*head, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(dev)[0] == free0
+        assert (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev)) == (alloc0, reserved0)
+        assert torch.equal(out, eager)
+        # under capture: the launches are recorded on the capturing stream, nothing else happens
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(dev)
+        with torch.cuda.graph(graph, stream=side):
+            rc = L.kvmix_quantized_gemv_static(*head, side.cuda_stream)
+        assert rc == 0, _lib.strerror(rc)
+        for _ in range(3):
+            out.fill_(float("nan"))        # the program's own eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
