@@ -40,6 +40,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <mutex>
 
 // Switches kept for measurement: with the hint compiled out the HBM counters show the bytes a kernel reads without it.
@@ -69,6 +70,8 @@ constexpr int kHeadsWaveDiv = 2;            // p.V, four heads per pass: half as
 constexpr int kMfma2MaxWaves = kTargetWaves;    // two-element matrix-core q.K^T kernel up to this many tiles
 constexpr int kMfma1MaxWaves = kTargetWaves;    // one-element matrix-core q.K^T kernel (one head) below this many tiles
 constexpr int kMfma2ResidentWaves = 3072;   // gemv_cols_mfma2: 3 waves on each of 1024 SIMDs
+constexpr int64_t kMfma2WideMinCodes = 6144;    // gemv_cols_mfma2: rows from this many codes on may take the wide tiles
+constexpr int64_t kMfma2WideMaxWaves = 2048;    // ... in launches of up to this many of them (one round, two waves per SIMD)
 constexpr int kMfma2KsplitWaves = 1536;     // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
 constexpr int kRowsChunksPerWave = 8;       // p.V: chunks a wave should get before more waves per row are used
 constexpr int kRowsSingleBlockChunks = 2;   // p.V: keep one block per output row up to this many chunks per wave
@@ -1680,54 +1683,65 @@ __global__ void __launch_bounds__(64 * kColsWaves)
 }
 
 // ---------------------------------------------------------------------------------------
-// gemv_cols_mfma2<BITS, NTC>   q.K^T, 4-, 2- or 1-bit codes, one query head per kv head: gemv_cols_mfma
-// with TWO 8-code elements per lane, so that a wave reads twice as many contiguous bytes of a row
-// (512 for 4 bits: measured, the length of the contiguous pieces is what bounds the streaming rate of
-// this shape).  Tile = 128 elements = 1024 codes = 32 groups, one tile per wave.
-//   2 bits, 1 bit: a lane loads elements 2l and 2l+1 of every row (one dword / ushort).  A quad of lanes
-//   then holds two quantization groups: lanes 0,1 the four elements of the first, lanes 2,3 those of
-//   the second.  Two MFMA sets per quad: set 0 works on the first group (lanes 2,3 fetch the second
-//   elements of lanes 0,1 with a DPP quad permute), set 1 on the second.
-//   4 bits: a lane's two dwords are element `lane` of each 256-byte half of the row piece; a quad then
-//   holds all four elements of ONE group in either half, set s works on half s with every lane's own
-//   register and nothing moves between lanes.
+// gemv_cols_mfma2<BITS, NTC, WIDE>   q.K^T, 4-, 2- or 1-bit codes, one query head per kv head: gemv_cols_mfma
+// with several 8-code elements per lane, so that a wave reads longer contiguous pieces of a row and the launch
+// needs fewer waves (measured: both the length of the pieces and the number of waves bound this shape).
+// A row piece is cut into `HALVES` sub-pieces of 64 lanes x one load each; a quad of lanes holds one (4 bits) or
+// two (2 bits, 1 bit) quantization groups per sub-piece, and each group of the quad is one MFMA set:
+//   4 bits: the lane's dword of a sub-piece is element `lane` of its 256 bytes; a quad then holds all four elements
+//   of ONE group, the set works on every lane's own register and nothing moves between lanes.
+//   2 bits, 1 bit: the lane's dword / ushort is elements 2l and 2l+1 of the sub-piece; lanes 0,1 of a quad hold the
+//   four elements of one group, lanes 2,3 those of the next.  The set of the first group takes the second elements
+//   of lanes 0,1 to lanes 2,3 with a DPP quad permute, the set of the second group mirrors it.
+//   Plain: 4 bits two sub-pieces (512 bytes), 2 bits one (256 bytes), 1 bit one (128 bytes): tile = 1024 codes = 32
+//   groups, two sets.  WIDE: twice the sub-pieces: tile = 2048 codes = 64 groups, four sets, half as many waves with
+//   twice the bytes in flight each (two waves per SIMD instead of three).
 //   Per set the scheme is gemv_cols_mfma's: k = 4 channel rows, three exact bf16 parts of x*scale*2^90
-//   as A.  Rows are walked in chunks of 16 (4 k-steps); the chunk's [16][32] scales and zeros are one
-//   128-bit load per lane each (64-byte pieces per row).  LDS tile: per (k-step, set) a row of
-//   64 eight-byte cells in four sub-rows at a pitch of 17 cells, rows at a pitch of 74.
+//   as A.  Rows are walked in chunks of 16 (4 k-steps); the chunk's [16][groups] scales and zeros are one
+//   128-bit load per lane and 32 groups each (plain: 64-byte pieces per row; WIDE: 128-byte pieces, 8 rows per
+//   load).  LDS tile: per (k-step, set) a row of 64 eight-byte cells in four sub-rows at a pitch of 17 cells, rows
+//   at a pitch of 74.
 //   Loads go through buffer descriptors (row offsets in SGPRs); NTC: codes with the non-temporal hint.
 //   block = (64, 2..4) waves on neighbouring tiles, or `ksplit` waves on ONE tile, each with a share
 //   of the K rows (small launches); grid = (tiles/waves, samples, M), XCD-swizzled.
 // ---------------------------------------------------------------------------------------
 constexpr int kColsMfma2Row = 74 * 4;                   // bf16 elements per (k-step, set) row
-constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets
+constexpr int kColsMfma2Tile = 8 * kColsMfma2Row;       // 4 k-steps x 2 sets (plain); WIDE: twice that
+constexpr int cols_mfma2_sets(bool wide) { return wide ? 4 : 2; }
+constexpr int cols_mfma2_groups(bool wide) { return 16 * cols_mfma2_sets(wide); }   // groups of 32 codes per tile
+constexpr size_t cols_mfma2_lds(bool wide)  // bytes per wave: the A tile + the tile's zero terms
+{
+    return (size_t)4 * cols_mfma2_sets(wide) * kColsMfma2Row * sizeof(uint16_t) + cols_mfma2_groups(wide) * sizeof(float);
+}
 
 // NTC: the codes are loaded non-temporally (the host asks for it while the launch is no more than a few rounds of
 // resident waves: measured faster up to 8k waves, slower at 16k, where rows of neighbouring tiles meet in the L2)
-template <int BITS, bool NTC>
+template <int BITS, bool NTC, bool WIDE>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
 gemv_cols_mfma2(GemvArgs a)
 {
-    static_assert(BITS == 4 || BITS == 2 || BITS == 1, "two elements per lane: a dwordx2, a dword or a ushort");
+    static_assert(BITS == 4 || BITS == 2 || BITS == 1, "per sub-piece a dword (4, 2 bits) or a ushort (1 bit) per lane");
     constexpr int CH = 16;             // rows per chunk
     constexpr int KB = CH / 4;         // MFMA k-steps per chunk
-    constexpr int AT = kColsMfma2Tile;
     constexpr int NPOS = 8;
     constexpr int FPB = 8 / BITS;
-    constexpr int TG = 32;             // groups per tile
-    constexpr int WL = BITS == 4 ? 2 : 1;  // registers per lane and row (1 bit: a ushort in one register)
-    // 4 bits: the lane's two elements are element `lane` of each 256-byte half of the tile row (two dword
-    // loads), so that a quad of lanes holds the four elements of ONE group in either half: set s works on
-    // half s with every lane's own register, no exchange between lanes.  Group g of the tile is then set
-    // g / 16, quad g % 16.  (2 bits, 1 bit: neighbouring elements, sets 0 / 1 = the quad's first / second group.)
-    constexpr bool SPLIT = BITS == 4;
+    constexpr bool SPLIT = BITS == 4;  // a quad holds ONE group per sub-piece (else two, exchanged by DPP)
+    constexpr int SPH = SPLIT ? 1 : 2;                       // sets (groups of a quad) per sub-piece
+    constexpr int HALVES = (SPLIT ? 2 : 1) * (WIDE ? 2 : 1); // sub-pieces per row piece = registers per lane and row
+    constexpr int NS = HALVES * SPH;                         // MFMA sets
+    constexpr int TG = 16 * NS;                              // groups per tile
+    constexpr int HB = BITS == 1 ? 128 : 256;                // bytes of a sub-piece
+    constexpr int AT = KB * NS * kColsMfma2Row;              // bf16 elements of the A tile
+    constexpr int NSZ = TG / 32;                             // 128-bit scale (and zero) loads per lane and chunk
+    constexpr int UPR = TG / 8;                              // staging units (8 groups) per row
+    static_assert(NS == cols_mfma2_sets(WIDE) && TG == cols_mfma2_groups(WIDE), "host-side sizes");
 
     extern __shared__ float lds[];
     const int lane = threadIdx.x;
     const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const int nw = (int)blockDim.y;
     uint16_t *atile = reinterpret_cast<uint16_t *>(lds) + wy * (AT + TG * 2);
-    float *zl = reinterpret_cast<float *>(atile + AT);  // [32] zero terms of a tile
+    float *zl = reinterpret_cast<float *>(atile + AT);  // [TG] zero terms of a tile
     int64_t bx, sample;
     xcd_swizzled_block(bx, sample, true);
     const int64_t m = blockIdx.z;
@@ -1752,23 +1766,25 @@ gemv_cols_mfma2(GemvArgs a)
     const int items = nch;
 
     const uint16_t *xp = reinterpret_cast<const uint16_t *>(a.x) + sample * a.x_bs + m * a.x_rs;
-    // buffer descriptors of this (batch, kv-head) slice; a lane's two elements are 2 * BITS bytes
+    // buffer descriptors of this (batch, kv-head) slice
     const uint32_t sz_bytes = slice_bytes(K, a.s_rs, ngroups, 2);
     const __amdgpu_buffer_rsrc_t crsrc = stream_rsrc(a.code + kv * a.c_bs, slice_bytes(K, a.c_rs, (int64_t)ngroups * BITS, 4));
     const __amdgpu_buffer_rsrc_t srsrc = stream_rsrc(a.scale + kv * a.s_bs, sz_bytes);
     const __amdgpu_buffer_rsrc_t zrsrc = stream_rsrc(a.zero + kv * a.s_bs, sz_bytes);
     const uint32_t c_rs = (uint32_t)a.c_rs, s_rs = (uint32_t)a.s_rs;
-    const int sub = lane % 4;   // staging: row lane/4 of the chunk, groups 8*sub .. 8*sub+7
-    const int srow = lane / 4;
-    const uint32_t c_lane = SPLIT ? (uint32_t)lane * 4u : (uint32_t)lane * (2 * BITS);  // bytes
-    const uint32_t s_lane = 2u * ((uint32_t)srow * s_rs + 8u * (uint32_t)sub);    // bytes
+    // staging: unit u = lane + 64 i (i < NSZ) is row u / UPR of the chunk, groups 8 * (u % UPR) .. + 7
+    // (u % UPR = lane % UPR for every i: a lane stages the same eight groups in NSZ rows)
+    const int sub = lane % UPR;
+    const uint32_t c_lane = (uint32_t)lane * (BITS == 1 ? 2u : 4u);                       // bytes, inside a sub-piece
+    const uint32_t s_lane = 2u * ((uint32_t)(lane / UPR) * s_rs + 8u * (uint32_t)sub);    // bytes, unit i = 0
+    const uint32_t s_step = 2u * (uint32_t)(kWave / UPR) * s_rs;                          // ... from unit i to i + 1
     const int j4 = lane % 4;    // position in the quad
 
-    f32x4_t acc[2][NPOS];
+    f32x4_t acc[NS][NPOS];
     float zacc[8];
     auto clear = [&]() {
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
+        for (int q = 0; q < NS; q++) {
 #pragma unroll
             for (int p = 0; p < NPOS; p++) acc[q][p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
@@ -1778,14 +1794,20 @@ gemv_cols_mfma2(GemvArgs a)
     clear();
 
     // cell (four bf16 k-slots) of (k-step t, set s, operand lane l)
-    auto cell = [](int t, int s, int l) { return (2 * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
-    // staged row srow is k-slot srow%4 of k-step srow/4; its group g = 8*sub + jj is set g%2 of quad g/2,
-    // i.e. operand lanes 4*(g/2) + i = 16*sub + 4*(jj/2) + i
-    const int aoff = SPLIT ? cell(srow / 4, sub / 2, 32 * (sub % 2)) + srow % 4 : cell(srow / 4, 0, 16 * sub) + srow % 4;
+    auto cell = [](int t, int s, int l) { return (NS * t + s) * kColsMfma2Row + ((l / 16) * 17 + l % 16) * 4; };
+    // Group g = 8 * sub + jj of the tile is sub-piece g / (16 SPH); 4 bits: quad g % 16 of set g / 16; else quad
+    // (g % 32) / 2 of set 2 (g / 32) + g % 2.  Its three parts go to operand lanes 4 quad + part.  Staged row r is
+    // k-slot r % 4 of k-step r / 4.  With `sub` folded into a per-lane base, the 24 stores of a unit are base + constant.
+    int aoff[NSZ];
+#pragma unroll
+    for (int i = 0; i < NSZ; i++) {
+        const int srow = (lane + kWave * i) / UPR;
+        aoff[i] = (SPLIT ? cell(srow / 4, sub / 2, 32 * (sub % 2)) : cell(srow / 4, 2 * (sub / 4), 16 * (sub % 4))) + srow % 4;
+    }
 
-    Half8 s8, z8;
-    uint16_t xh;
-    uint32_t w[KB][4][WL];
+    Half8 s8[NSZ], z8[NSZ];
+    uint16_t xh[NSZ];
+    uint32_t w[KB][4][HALVES];
 
     // the last tile of a row is moved back to end at N
     const int g_first = tile0 * TG + TG <= ngroups ? tile0 * TG : max(ngroups - TG, 0);
@@ -1795,71 +1817,75 @@ gemv_cols_mfma2(GemvArgs a)
     auto load_small = [&](int it) {
         const uint32_t d0 = (uint32_t)chunk_base(chunk_k0(it));
         const uint32_t off = 2u * (d0 * s_rs + (uint32_t)tile_g0(it));  // bytes, the same for every lane
-        s8 = ld_buffer<Half8, false>(srsrc, s_lane, off);
-        z8 = ld_buffer<Half8, false>(zrsrc, s_lane, off);
-        xh = xp[d0 + (uint32_t)srow];
+#pragma unroll
+        for (int i = 0; i < NSZ; i++) {
+            s8[i] = ld_buffer<Half8, false>(srsrc, s_lane + (uint32_t)i * s_step, off);
+            z8[i] = ld_buffer<Half8, false>(zrsrc, s_lane + (uint32_t)i * s_step, off);
+            xh[i] = xp[d0 + (uint32_t)((lane + kWave * i) / UPR)];
+        }
     };
     auto load_codes = [&](int it, int t) {
         // (a group of 32 codes is BITS words)
         const uint32_t base = 4u * ((uint32_t)(chunk_base(chunk_k0(it)) + 4 * t) * c_rs + (uint32_t)tile_g0(it) * BITS);
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            if constexpr (BITS == 1) {
-                w[t][k][0] = ld_buffer<uint16_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
-            } else if constexpr (SPLIT) {
-                w[t][k][0] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
-                w[t][k][1] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane + 256u, base + 4u * (uint32_t)k * c_rs);
-            } else {
-                const Words<WL> v = ld_buffer<Words<WL>, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane, base + 4u * (uint32_t)k * c_rs);
 #pragma unroll
-                for (int e = 0; e < WL; e++) w[t][k][e] = v.v[e];
+            for (int h = 0; h < HALVES; h++) {
+                if constexpr (BITS == 1)
+                    w[t][k][h] = ld_buffer<uint16_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane + (uint32_t)(h * HB), base + 4u * (uint32_t)k * c_rs);
+                else
+                    w[t][k][h] = ld_buffer<uint32_t, (KVMIX_COLS_NT_CODES && NTC)>(crsrc, c_lane + (uint32_t)(h * HB), base + 4u * (uint32_t)k * c_rs);
             }
         }
     };
     auto stage = [&](int it) {
         const int k0 = chunk_k0(it);
         const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
-        const float xv = srow >= skip ? h16_to_f32(xh) : 0.f;
-        const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90
 #pragma unroll
-        for (int jj = 0; jj < 8; jj++) {
-            zacc[jj] = fmaf(xv, h16_to_f32(z8.v[jj]), zacc[jj]);
-            const float v0 = x2 * h16_to_f32(s8.v[jj]);  // split into three bf16 by truncation (exact)
-            const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
-            const float v1 = v0 - __uint_as_float(b0);
-            const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
-            const float v2 = v1 - __uint_as_float(b1);
-            const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+        for (int i = 0; i < NSZ; i++) {
+            const int srow = (lane + kWave * i) / UPR;
+            const float xv = srow >= skip ? h16_to_f32(xh[i]) : 0.f;
+            const float x2 = xv * 1237940039285380274899124224.0f;  // 2^90
 #pragma unroll
-            for (int pt = 0; pt < 3; pt++) {
-                if constexpr (SPLIT)  // operand lane 32 * (sub % 2) + 4 * jj + pt of set sub / 2
-                    atile[aoff + (((4 * jj + pt) / 16) * 17 + (4 * jj + pt) % 16) * 4] = (uint16_t)(part[pt] >> 16);
-                else
-                    atile[aoff + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+            for (int jj = 0; jj < 8; jj++) {
+                zacc[jj] = fmaf(xv, h16_to_f32(z8[i].v[jj]), zacc[jj]);
+                const float v0 = x2 * h16_to_f32(s8[i].v[jj]);  // split into three bf16 by truncation (exact)
+                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+                const float v1 = v0 - __uint_as_float(b0);
+                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+                const float v2 = v1 - __uint_as_float(b1);
+                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+                for (int pt = 0; pt < 3; pt++) {
+                    if constexpr (SPLIT)  // operand lane 32 * (sub % 2) + 4 * jj + pt of set sub / 2
+                        atile[aoff[i] + (((4 * jj + pt) / 16) * 17 + (4 * jj + pt) % 16) * 4] = (uint16_t)(part[pt] >> 16);
+                    else                  // operand lane 16 * (sub % 4) + 4 * (jj / 2) + pt of set 2 * (sub / 4) + jj % 2
+                        atile[aoff[i] + (jj % 2) * kColsMfma2Row + (4 * (jj / 2) + pt) * 4] = (uint16_t)(part[pt] >> 16);
+                }
             }
         }
     };
-    // first element (8 codes) of the group set s works on, as this lane sees it: for 4 bits the
-    // word itself, for 2 bits the half of the word given by the byte offset in the selector
     auto compute = [&](int t) {
-        const bf16x4_t av0 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 0, lane));
-        const bf16x4_t av1 = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, 1, lane));
+        bf16x4_t av[NS];
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            // set 0: lanes 0,1 of a quad hold the group's elements 0,2 (their first) and lanes 2,3
-            // take elements 1,3 (the second of lanes 0,1); set 1 mirrors it for lanes 2,3
+        for (int s = 0; s < NS; s++) av[s] = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, s, lane));
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const int h = s / SPH, s2 = s % SPH;  // sub-piece; which of the quad's groups in it
+            // first group of the quad (s2 == 0): lanes 0,1 hold its elements 0,2 (their first) and lanes 2,3
+            // take elements 1,3 (the second of lanes 0,1); the second group mirrors it for lanes 2,3
             uint32_t src[4];
             uint32_t hi = 0;  // 2 bits / 1 bit: byte offset (0 or 2 / 0 or 1) of the element inside the register
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 if constexpr (SPLIT) {
-                    src[k] = w[t][k][s];
+                    src[k] = w[t][k][h];
                 } else {
-                    src[k] = s == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][0], 0x44, 0xf, 0xf, false)
-                                    : __builtin_amdgcn_mov_dpp(w[t][k][0], 0xEE, 0xf, 0xf, false);
+                    src[k] = s2 == 0 ? __builtin_amdgcn_mov_dpp(w[t][k][h], 0x44, 0xf, 0xf, false)
+                                     : __builtin_amdgcn_mov_dpp(w[t][k][h], 0xEE, 0xf, 0xf, false);
                 }
             }
-            if constexpr (BITS != 4) hi = (s == 0 ? j4 >= 2 : j4 < 2) ? (uint32_t)BITS : 0u;  // byte offset of the element
+            if constexpr (BITS != 4) hi = (s2 == 0 ? j4 >= 2 : j4 < 2) ? (uint32_t)BITS : 0u;  // byte offset of the element
 #pragma unroll
             for (int b = 0; b < BITS; b++) {
                 const uint32_t sel = (0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16)) + hi * 0x00010001u;
@@ -1869,8 +1895,7 @@ gemv_cols_mfma2(GemvArgs a)
                 for (int f = 0; f < FPB; f++) {
                     const bf16x4_t bv =
                         __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<BITS>(t01, f), field_operand<BITS>(t23, f)));
-                    acc[s][b * FPB + f] =
-                        __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(s == 0 ? av0 : av1, bv, acc[s][b * FPB + f], 0, 0, 0);
+                    acc[s][b * FPB + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av[s], bv, acc[s][b * FPB + f], 0, 0, 0);
                 }
             }
         }
@@ -1879,16 +1904,21 @@ gemv_cols_mfma2(GemvArgs a)
         uint16_t v[8];
     };
     auto finish_tile = [&](int it) {
-        // zero terms: zacc[jj] summed over the 16 lanes with the same `sub`; group 8*sub+jj -> LDS
+        // zero terms: zacc[jj] summed over the lanes with the same `sub`; group 8*sub+jj -> LDS
         float z[8];
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) z[jj] = zacc[jj];
-        const int first = scatter_reduce<8, 4, 1>(z, lane);  // lane bits 2..4
-        z[0] += __shfl_xor(z[0], 32);
+        int first;
+        if constexpr (UPR == 4) {
+            first = scatter_reduce<8, 4, 1>(z, lane);  // lane bits 2..4
+            z[0] += __shfl_xor(z[0], 32);
+        } else {
+            first = scatter_reduce<8, 8, 1>(z, lane);  // lane bits 3..5
+        }
         zl[8 * sub + first] = z[0];
-        float sum[2][NPOS];
+        float sum[NS][NPOS];
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
+        for (int s = 0; s < NS; s++) {
 #pragma unroll
             for (int p = 0; p < NPOS; p++) sum[s][p] = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
         }
@@ -1898,7 +1928,7 @@ gemv_cols_mfma2(GemvArgs a)
             float *mine = reinterpret_cast<float *>(atile);
             if (slice > 0) {
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
+                for (int s = 0; s < NS; s++) {
 #pragma unroll
                     for (int p = 0; p < NPOS; p++) mine[(s * NPOS + p) * kWave + lane] = sum[s][p];
                 }
@@ -1910,7 +1940,7 @@ gemv_cols_mfma2(GemvArgs a)
                     const float *other = reinterpret_cast<const float *>(other_tile);
                     const float *ozl = reinterpret_cast<const float *>(other_tile + AT);
 #pragma unroll
-                    for (int s = 0; s < 2; s++) {
+                    for (int s = 0; s < NS; s++) {
 #pragma unroll
                         for (int p = 0; p < NPOS; p++) sum[s][p] += other[(s * NPOS + p) * kWave + lane];
                     }
@@ -1923,17 +1953,19 @@ gemv_cols_mfma2(GemvArgs a)
             const int q = lane / 4;
             uint16_t *orow = reinterpret_cast<uint16_t *>(a.out) + sample * a.o_bs + m * a.o_rs + (int64_t)tile_g0(it) * 32;
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                const float zt = SPLIT ? zl[16 * s + q] : zl[2 * q + s];
-                // element of the quad's 8 that this lane's accumulators of set s belong to
-                const int elem = s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1)));
+            for (int s = 0; s < NS; s++) {
+                const int h = s / SPH, s2 = s % SPH;
+                // group of the tile / element (8 codes) of the tile that this lane's accumulators of set s belong to
+                const float zt = SPLIT ? zl[16 * h + q] : zl[32 * h + 2 * q + s2];
+                const int elem = SPLIT ? 64 * h + lane
+                                       : 128 * h + 8 * q + (s2 == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1))));
                 Out8 o;
 #pragma unroll
                 for (int p = 0; p < NPOS; p++) {
                     const float v = field_sum(sum[s][p], sum[s][p > 0 ? p - 1 : 0], p % FPB);
                     o.v[p] = f32_to_h16(fmaf(v, __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23), zt));
                 }
-                *reinterpret_cast<Out8 *>(orow + (SPLIT ? 64 * s + lane : 8 * q + elem) * 8) = o;
+                *reinterpret_cast<Out8 *>(orow + elem * 8) = o;
             }
         }
         wave_lds_fence();
@@ -2718,30 +2750,48 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     KVMIX_LAUNCH((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma<%d,%d>", BITS, NREP);
 }
 
-template <int BITS, bool NTC>
+template <int BITS, bool NTC, bool WIDE>
 static void launch_cols_mfma2_nt(GemvArgs &a, int64_t samples, hipStream_t st)
 {
-    if (!tile_fits(a.N / 32, 32) || !tile_fits(a.K, 16)) return;  // a 1024-code tile, a 16-row chunk
-    const int64_t tiles = (a.N / 32 + 31) / 32;
+    constexpr int TG = cols_mfma2_groups(WIDE);  // groups of 32 codes per tile
+    if (!tile_fits(a.N / 32, TG) || !tile_fits(a.K, 16)) return;  // a whole tile, a 16-row chunk
+    const int64_t tiles = (a.N / 32 + TG - 1) / TG;
     const int64_t batch = samples * a.M;
     // one tile per wave (several tiles per wave, so that one round of resident waves covers the problem, were
     // measured slower at every size).  Few tiles: 2 or 4 waves per tile, each with a share of the K rows (chunks of 16)
     const int64_t chunks = (a.K + 15) / 16;
     int ks = 1;
-    while (ks < kColsWaves && batch * tiles * ks * 2 <= kMfma2KsplitWaves && chunks >= ks * 4) ks *= 2;
+    while (!WIDE && ks < kColsWaves && batch * tiles * ks * 2 <= kMfma2KsplitWaves && chunks >= ks * 4) ks *= 2;
     a.ksplit = ks;
+    a.splits = 1;
+    const size_t lds_wave = cols_mfma2_lds(WIDE);
     if (ks > 1) {
-        a.splits = 1;
         const dim3 grid((unsigned)tiles, (unsigned)samples, (unsigned)a.M);  // one tile per block of ks waves
-        const size_t lds = (size_t)ks * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-        KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, ks), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
+        KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC, WIDE>), grid, dim3(kWave, ks), ks * lds_wave, st, a, "gemv_cols_mfma2<%d,%d,%d>", BITS,
+                     (int)NTC, (int)WIDE);
         return;
     }
     const int wpb = pick_waves_per_block(tiles);
-    a.splits = 1;
     const dim3 grid((unsigned)((tiles + wpb - 1) / wpb), (unsigned)samples, (unsigned)a.M);
-    const size_t lds = (size_t)wpb * (kColsMfma2Tile * sizeof(uint16_t) + 32 * sizeof(float));
-    KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma2<%d,%d>", BITS, (int)NTC);
+    KVMIX_LAUNCH((gemv_cols_mfma2<BITS, NTC, WIDE>), grid, dim3(kWave, wpb), wpb * lds_wave, st, a, "gemv_cols_mfma2<%d,%d,%d>", BITS,
+                 (int)NTC, (int)WIDE);
+}
+
+// Whether a launch takes the wide tiles (2048 codes per wave, two waves per SIMD) instead of the plain ones (1024
+// codes, three waves per SIMD): where the plain tiles would need more than one round of resident waves, the wide
+// ones get by with half as many waves that each keep twice the bytes in flight.  Measured, one library against
+// the other in one run (plain -> wide, us): T = 8k, B = 16: 4 bits 58.6 -> 56.5, 2 bits 40.2 -> 39.5; B = 24: 92.8 ->
+// 90.3, 71.4 -> 68.3; B = 32: 130.1 -> 124.9, 84.9 -> 84.2; B = 8 at T = 16k, 2 bits: 37.5 -> 35.0.  Behind where
+// one round of plain tiles covers the launch (B = 12: 44.4 -> 49.2, 29.2 -> 32.1) and on short rows (T = 4k, B = 64:
+// 136.6 -> 141.7, 88.0 -> 88.9).
+static bool cols_mfma2_wide(int bits, int64_t batch, int64_t N)
+{
+#ifdef KVMIX_EXPERIMENT
+    if (const char *e = getenv("KVMIX_DBG_WIDE")) return atoi(e) != 0 && N >= 2048;
+#endif
+    (void)bits;
+    const int64_t plain_tiles = (N / 32 + 31) / 32;
+    return N >= kMfma2WideMinCodes && batch * plain_tiles > (int64_t)kMfma2ResidentWaves;
 }
 
 template <int BITS>
@@ -2750,10 +2800,15 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     // non-temporal code loads: 2 and 4 bits (a wave's 1-bit row piece is 128 bytes and shares its cache lines
     // with the neighbours'), and only while the launch is at most three rounds of resident waves
     const int64_t tiles = (a.N / 32 + 31) / 32;
-    if (BITS >= 2 && samples * a.M * tiles <= 3 * (int64_t)kMfma2ResidentWaves)
-        launch_cols_mfma2_nt<BITS, true>(a, samples, st);
-    else
-        launch_cols_mfma2_nt<BITS, false>(a, samples, st);
+    const bool nt = BITS >= 2 && samples * a.M * tiles <= 3 * (int64_t)kMfma2ResidentWaves;
+    const bool wide = cols_mfma2_wide(BITS, samples * a.M, a.N);
+    if (wide) {
+        if (nt) launch_cols_mfma2_nt<BITS, true, true>(a, samples, st);
+        else launch_cols_mfma2_nt<BITS, false, true>(a, samples, st);
+    } else {
+        if (nt) launch_cols_mfma2_nt<BITS, true, false>(a, samples, st);
+        else launch_cols_mfma2_nt<BITS, false, false>(a, samples, st);
+    }
 }
 
 int plan_attn_slab_mfma(int64_t tokens, int64_t samples, unsigned grid[3], unsigned block[3])
@@ -2809,8 +2864,18 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // 110 -> 87 us; at T = 8k gemv_cols stays ahead)
         const bool one_bit_ok = MODE != 1 || (a.N <= 2 * 2048 &&
                                               samples * a.M * ((a.N / 32 + 31) / 32) >= (int64_t)kMfma1MaxWaves);
+        // ... and with the wide tiles (rows of kMfma2WideMinCodes codes and more): 4 bits up to kMfma2WideMaxWaves of
+        // them (beyond, gemv_cols is ahead: T = 8k, B = 20: 73.0 against 79.2 us, B = 48: 173 against 191), 2 bits at
+        // any batch (gemv_cols -> wide tiles, us: T = 8k, B = 20: 57.8 -> 53.6, B = 24: 69.3 -> 60.0, B = 32: 85.2 -> 79.8,
+        // B = 64: 169.7 -> 159.2; T = 16k, B = 12: 66.1 -> 59.3; T = 32k, B = 8: 78.1 -> 71.9)
+        int64_t wide_max = kMfma2WideMaxWaves;
+#ifdef KVMIX_EXPERIMENT
+        if (const char *e = getenv("KVMIX_DBG_WIDE_MAX")) wide_max = atoll(e);
+#endif
+        const bool wide_range = MODE != 1 && a.N >= kMfma2WideMinCodes &&
+                                (MODE == 2 || samples * a.M * ((a.N / 32 + 63) / 64) <= wide_max);
         if (one_bit_ok && heads_per_block(a.heads_per_kv) == 1 && a.N >= 1024 && a.K >= 16 &&
-            (MODE == 1 || samples * a.M * tiles2 <= (int64_t)kMfma2MaxWaves || a.N <= 2 * 2048)) {
+            (MODE == 1 || samples * a.M * tiles2 <= (int64_t)kMfma2MaxWaves || wide_range || a.N <= 2 * 2048)) {
             launch_cols_mfma2<MODE>(a, samples, st);
             return;
         }

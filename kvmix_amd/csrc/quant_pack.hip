@@ -24,7 +24,14 @@
 
 namespace kvmix {
 
-constexpr int kFlushValuePieces = 1;  // value half of the fused flush: 128-bit pieces per thread (more measured no faster)
+#ifndef KVMIX_FLUSH_VALUE_PIECES
+#define KVMIX_FLUSH_VALUE_PIECES 1
+#endif
+#ifndef KVMIX_FLUSH_IDX32
+#define KVMIX_FLUSH_IDX32 0
+#endif
+constexpr int kFlushValuePieces = KVMIX_FLUSH_VALUE_PIECES;  // value half of the fused flush: 128-bit pieces per thread (more measured no faster)
+constexpr bool kFlushIdx32 = KVMIX_FLUSH_IDX32 != 0;
 
 struct QuantArgs {
     const void *x;
@@ -622,10 +629,10 @@ __global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, 
     } else {
         const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
         switch (va.bits) {
-        case 1: rows_g32_f16_body<1, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
-        default: rows_g32_f16_body<4, kFlushValuePieces, false>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 1: rows_g32_f16_body<1, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
+        default: rows_g32_f16_body<4, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
         }
     }
 }

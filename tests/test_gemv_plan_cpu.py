@@ -26,8 +26,9 @@ def plan(bits, fmt, batch, kv_heads, rep, tokens, head_dim, side, group=32):
 def test_target_shape_b16_t8k(bits):
     # 2/4-bit Llama-2-7B KV at 8k context, batch 16 (8064 quantized tokens + the fp16 window)
     qk = plan(bits, REF, 16, 32, 1, 8064, 128, "qk")
-    assert qk["kernel"].startswith(f"gemv_cols_mfma2<{bits},") and qk["launches"] == 1
-    assert qk["grid"][1] == 512 and qk["block"] == (64, 4, 1)
+    # the wide tiles (2048 codes per wave): four waves cover a row, 2048 waves in all = one round at two per SIMD
+    assert qk["kernel"] == f"gemv_cols_mfma2<{bits},1,1>" and qk["launches"] == 1
+    assert qk["grid"][:2] == (1, 512) and qk["block"] == (64, 4, 1)
     pv = plan(bits, REF, 16, 32, 1, 8064, 128, "pv")
     assert pv["kernel"] == f"gemv_rows_mfma<{bits},1,1>" and pv["launches"] == 1 and pv["splits"] == 1
 
@@ -41,8 +42,13 @@ def test_config0_single_layer_b1_t4096():
 
 
 def test_config1_mixed_bits_b8_t8192():
-    assert plan(4, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<4,")
-    assert plan(2, REF, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<2,")
+    # one round of the plain tiles (1024 codes per wave) covers these launches
+    assert plan(4, REF, 8, 32, 1, 8064, 128, "qk")["kernel"] == "gemv_cols_mfma2<4,1,0>"
+    assert plan(2, REF, 8, 32, 1, 8064, 128, "qk")["kernel"] == "gemv_cols_mfma2<2,1,0>"
+    # large batches: 2 bits stay on the matrix cores with the wide tiles, 4 bits go to the vector-ALU kernel
+    assert plan(2, REF, 32, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols_mfma2<2,") and \
+        plan(2, REF, 32, 32, 1, 8064, 128, "qk")["kernel"].endswith(",1>")
+    assert plan(4, REF, 32, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols<4,")
     # the reference's 3-bit keys: 11 codes a word, 8063 = 733 * 11 tokens
     ref3 = plan(3, REF, 8, 32, 1, 8063, 128, "qk")
     # 128-word tiles, four waves a tile, each with a quarter of the channel rows
@@ -70,7 +76,7 @@ def test_config3_sweep_t4096_residual32(bits, batch):
         assert qk == "gemv_cols_mfma<1,1>"   # several tiles per wave: ahead while one round of waves covers the launch
     else:
         # non-temporal code loads (second argument) for 2-bit launches of up to three resident rounds of waves
-        assert qk == f"gemv_cols_mfma2<{bits},{int(bits == 2 and batch <= 64)}>"
+        assert qk.startswith(f"gemv_cols_mfma2<{bits},{int(bits == 2 and batch <= 64)},")
     assert plan(bits, REF, batch, 32, 1, 4064, 128, "pv")["kernel"] == f"gemv_rows_mfma<{bits},1,1>"
 
 
@@ -109,8 +115,9 @@ def _tile_units(kernel):
     m = re.match(r"gemv_cols<(\d+),(\d+),(\d+)>", kernel)
     if m:
         return (64 // int(m.group(2))) * int(m.group(3))
-    if kernel.startswith("gemv_cols_mfma2<"):
-        return 32
+    m = re.match(r"gemv_cols_mfma2<(\d+),(\d+),(\d+)>", kernel)
+    if m:
+        return 64 if int(m.group(3)) else 32   # (third argument: the wide tiles)
     if kernel.startswith("gemv_cols_mfma<"):
         return 16
     return 0

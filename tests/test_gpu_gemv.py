@@ -76,6 +76,13 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
     # a launch beyond one resident round of waves with short rows (the two-element kernel for every width)
     run_case(oracle, dev, bits, g, B=32, nh=32, nkv=32, K=32, N=32 * 127, seed=48)
     run_case(oracle, dev, bits, g, B=40, nh=32, nkv=32, K=48, N=32 * 127, seed=49)
+    if bits != 1:
+        # the wide tiles (2048 codes per wave; rows of 6144 codes and more, launches beyond one round of the plain
+        # tiles): a last tile moved back (197 groups = 3 tiles + 5 groups), K not a multiple of the chunk
+        from kvmix_amd import _lib
+        assert _lib.gemv_plan(g, bits, 0, 17 * 32, 1, 1, 24, 32 * 197)["kernel"].endswith(",1>")
+        run_case(oracle, dev, bits, g, B=17, nh=32, nkv=32, K=24, N=32 * 197, seed=50)
+        run_case(oracle, dev, bits, g, B=9, nh=64, nkv=64, K=16, N=32 * 192, seed=51)
     # p.V: chunks of 128 rows, K ragged; GQA with split-K; M = 2
     for K in (128, 129, 255, 1000):
         run_case(oracle, dev, bits, g, B=1, nh=2, nkv=2, K=K, N=128, seed=K)
