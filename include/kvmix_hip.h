@@ -322,14 +322,14 @@ int kvmix_decode_attention_fused(const kvmix_decode_attn_t *step, void *workspac
  * for the same sizes (KVMIX_ERR_NULL and KVMIX_ERR_WORKSPACE aside).
  */
 typedef struct kvmix_attn_plan {
-    int matrix;              /* 1: quantized positions [0, slab_begin) run on the matrix cores, one wave per tile */
+    int matrix;              /* 1: the positions [0, slab_begin) run on the matrix cores, one wave per tile */
     int launches;            /* kernel launches of the step, the merge included */
     int64_t matrix_tiles;    /* tiles of 1024 positions per query head (0 without the matrix-core kernel) */
-    int64_t slab_positions;  /* positions per slab of the vector-ALU slab kernel */
+    int64_t slab_positions;  /* positions per vector-ALU slab */
     int64_t slab_begin;      /* first position those slabs cover */
     int64_t slabs;           /* their number per query head */
-    unsigned matrix_grid[3], matrix_block[3];
-    unsigned slab_grid[3];
+    int64_t slab_blocks;     /* their blocks: trailing blocks of the matrix-core launch, or a launch of their own */
+    unsigned matrix_grid[3], matrix_block[3];   /* the matrix-core launch, the slabs' blocks included */
 } kvmix_attn_plan_t;
 int kvmix_decode_attention_fused_plan(const kvmix_decode_attn_t *step, kvmix_attn_plan_t *plan);
 

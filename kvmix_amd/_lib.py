@@ -103,7 +103,7 @@ class AttnPlan(ctypes.Structure):
     """kvmix_attn_plan_t"""
     _fields_ = [("matrix", ctypes.c_int), ("launches", ctypes.c_int), ("matrix_tiles", ctypes.c_int64),
                 ("slab_positions", ctypes.c_int64), ("slab_begin", ctypes.c_int64), ("slabs", ctypes.c_int64),
-                ("matrix_grid", ctypes.c_uint * 3), ("matrix_block", ctypes.c_uint * 3), ("slab_grid", ctypes.c_uint * 3)]
+                ("slab_blocks", ctypes.c_int64), ("matrix_grid", ctypes.c_uint * 3), ("matrix_block", ctypes.c_uint * 3)]
 
 
 class KVmixLibraryMissing(ImportError):
@@ -212,8 +212,8 @@ def attn_plan(step: DecodeAttn) -> dict:
     check(load().kvmix_decode_attention_fused_plan(ctypes.byref(step), ctypes.byref(plan)))
     return {"matrix": bool(plan.matrix), "launches": plan.launches, "matrix_tiles": plan.matrix_tiles,
             "slab_positions": plan.slab_positions, "slab_begin": plan.slab_begin, "slabs": plan.slabs,
-            "matrix_grid": tuple(plan.matrix_grid), "matrix_block": tuple(plan.matrix_block),
-            "slab_grid": tuple(plan.slab_grid)}
+            "slab_blocks": plan.slab_blocks, "matrix_grid": tuple(plan.matrix_grid),
+            "matrix_block": tuple(plan.matrix_block)}
 
 
 def strerror(code: int) -> str:

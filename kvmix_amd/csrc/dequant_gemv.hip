@@ -35,7 +35,7 @@
 // scheduling barriers -- otherwise the compiler sinks the prefetch loads to the end of the loop
 // body and every iteration starts by draining the load queue.
 
-#include "kvmix_common.h"
+#include "fused_slab.h"
 
 #include <atomic>
 #include <cstdarg>
@@ -2031,23 +2031,19 @@ constexpr int kSlabLds = kSlabKeyBytes + 1024 * 4;                            //
 static_assert(kRowsMfmaTile * 2 <= kSlabKeyBytes, "the value phase's A tile reuses the key phase's space");
 
 template <int KBITS, int VMODE>
-__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
-attn_slab_mfma(AttnSlabArgs a)
+__device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64_t bx, int64_t sample, float *lds)
 {
     static_assert(KBITS == 4 || KBITS == 2 || KBITS == 1, "key codes of 1, 2 or 4 bits");
     constexpr bool NTC = KBITS >= 2;  // (as gemv_cols_mfma2: a 1-bit row piece shares its lines with the neighbours')
     constexpr int NPOS = 8;
     constexpr int TG = 32;            // groups per tile
 
-    extern __shared__ float lds[];
     const int lane = threadIdx.x;
     const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const int nw = (int)blockDim.y;
     uint8_t *mine = reinterpret_cast<uint8_t *>(lds) + wy * kSlabLds;
     uint16_t *atile = reinterpret_cast<uint16_t *>(mine);
     float *pbuf = reinterpret_cast<float *>(mine + kSlabKeyBytes);  // [1024] probabilities of the slab
-    int64_t bx, sample;
-    xcd_swizzled_block(bx, sample, true);
     const int64_t kv = sample / a.heads_per_kv;
     const int ngroups = (int)(a.tokens / 32);
     const int tile = (int)bx * nw + wy;
@@ -2400,6 +2396,31 @@ attn_slab_mfma(AttnSlabArgs a)
             ml[0] = slab_m;
             ml[1] = slab_l;
         }
+    }
+}
+
+// The launch of a large single-pass step: blocks [0, mfma_blocks) are the matrix-core tiles above (mfma_nx blocks per
+// query head, XCD-swizzled), the rest are slabs of the vector-ALU kind (fused_slab.h, 8 lanes per key row = 256
+// threads) over the positions the tiles do not cover: the fp16 tails, and quantized positions where keys and values
+// are quantized to different lengths.  One launch instead of two; attn_fused_merge follows.
+// block = (64, 4); dynamic LDS = kStepLds.
+constexpr size_t kStepLds = 4 * kSlabLds > fused::SlabCfg<8>::lds_floats(1) * sizeof(float) ? 4 * kSlabLds
+                                                                                           : fused::SlabCfg<8>::lds_floats(1) * sizeof(float);
+template <int KBITS, int VMODE>
+__global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
+attn_step_mfma(AttnSlabArgs m, fused::FusedArgs f, unsigned mfma_blocks, unsigned mfma_nx)
+{
+    extern __shared__ float lds[];
+    if (blockIdx.x < mfma_blocks) {
+        // consecutive logical blocks on one XCD (xcd_swizzled_block, for a part of a one-dimensional grid; the XCD
+        // of a block is its index in the whole launch modulo 8, and the tiles come first)
+        const int64_t n = mfma_blocks, l = blockIdx.x;
+        const int64_t xcd = l % kXcds, slot = l / kXcds, per = n / kXcds, rem = n % kXcds;
+        const int64_t j = xcd * per + (xcd < rem ? xcd : rem) + slot;
+        attn_slab_mfma_body<KBITS, VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
+    } else {
+        fused::attn_fused_slab_body<1, 8>(f, (int64_t)blockIdx.x - mfma_blocks, (int64_t)gridDim.x - mfma_blocks,
+                                          (int)(threadIdx.y * kWave + threadIdx.x), lds);
     }
 }
 
@@ -2811,25 +2832,27 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     }
 }
 
-int plan_attn_slab_mfma(int64_t tokens, int64_t samples, unsigned grid[3], unsigned block[3])
+int plan_attn_slab_mfma(int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3])
 {
     const int64_t tiles = (tokens / 32 + 31) / 32;
-    if (tokens < 1024 || tokens % 32 != 0 || samples <= 0 || samples > 65535 || tiles > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    const int wpb = pick_waves_per_block(tiles);
-    grid[0] = (unsigned)((tiles + wpb - 1) / wpb), grid[1] = (unsigned)samples, grid[2] = 1;
-    block[0] = kWave, block[1] = (unsigned)wpb, block[2] = 1;
+    if (tokens < 1024 || tokens % 32 != 0 || samples <= 0 || tail_blocks < 0) return KVMIX_ERR_SHAPE;
+    const int64_t nx = (tiles + kColsWaves - 1) / kColsWaves;  // blocks of four tiles per query head
+    if (nx * samples + tail_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    grid[0] = (unsigned)(nx * samples + tail_blocks), grid[1] = 1, grid[2] = 1;
+    block[0] = kWave, block[1] = kColsWaves, block[2] = 1;
     return KVMIX_OK;
 }
 
-int launch_attn_slab_mfma(const AttnSlabArgs &a, int k_bits, int v_mode, int64_t samples, hipStream_t stream)
+int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, int v_mode, int64_t samples,
+                          int64_t tail_blocks, hipStream_t stream)
 {
     unsigned g[3], b[3];
-    const int prc = plan_attn_slab_mfma(a.tokens, samples, g, b);
+    const int prc = plan_attn_slab_mfma(a.tokens, samples, tail_blocks, g, b);
     if (prc != KVMIX_OK) return prc;
-    const int wpb = (int)b[1];
-    const dim3 grid(g[0], g[1]), block(b[0], b[1]);
-    const size_t lds = (size_t)wpb * kSlabLds;
-#define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_slab_mfma<KB_, VM_>), grid, block, lds, stream, a)
+    const dim3 grid(g[0]), block(b[0], b[1]);
+    const unsigned mfma_blocks = (unsigned)(g[0] - tail_blocks), mfma_nx = (unsigned)(mfma_blocks / samples);
+    const size_t lds = kStepLds;
+#define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_step_mfma<KB_, VM_>), grid, block, lds, stream, a, f, mfma_blocks, mfma_nx)
 #define KVMIX_SLAB_V(KB_)                          \
     switch (v_mode) {                              \
     case 1: KVMIX_SLAB(KB_, 1); break;             \

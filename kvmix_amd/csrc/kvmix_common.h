@@ -137,12 +137,6 @@ struct AttnSlabArgs {
     int slabs;                // slabs of a row in the workspace (these tiles first, the tail's slabs after them)
     float inv_sqrt_d;
 };
-// k_bits in {1, 2, 4}; v_mode in {1, 2, 4, 30 (dense 3-bit)}
-int launch_attn_slab_mfma(const AttnSlabArgs &a, int k_bits, int v_mode, int64_t samples, hipStream_t stream);
-// grid and block of that launch for `tokens` quantized positions and `samples` query heads (KVMIX_ERR_SHAPE for
-// sizes the kernel does not take: fewer positions than one tile, not whole groups, too many rows for a grid)
-int plan_attn_slab_mfma(int64_t tokens, int64_t samples, unsigned grid[3], unsigned block[3]);
-
 inline int launch_status()
 {
     return hipGetLastError() == hipSuccess ? KVMIX_OK : KVMIX_ERR_LAUNCH;

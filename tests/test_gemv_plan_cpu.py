@@ -159,11 +159,15 @@ def _step(batch, heads, kv_heads, k_bits, k_fmt, k_tokens, v_bits, v_fmt, v_toke
 
 
 def test_attention_step_plans_of_the_measured_shapes():
-    # B = 16, T = 8192, 4-bit keys and values quantized to the same length: matrix cores over [0, 8064), the two
-    # 128-token fp16 tails as one further slab, and the merge
+    # B = 16, T = 8192, 4-bit keys and values: matrix cores over [0, 8064) (two blocks of four tiles per query head),
+    # the two 128-token fp16 tails as one slab of 256 positions in a trailing block of the same launch, and the merge
     p = _lib.attn_plan(_step(16, 32, 32, 4, REF, 8064, 4, REF, 8064, 8192))
-    assert p["matrix"] and p["matrix_tiles"] == 8 and p["slab_begin"] == 8064 and p["slabs"] == 1 and p["launches"] == 3
-    assert p["matrix_grid"][:2] == (2, 512) and p["matrix_block"] == (64, 4, 1)
+    assert p["matrix"] and p["matrix_tiles"] == 8 and p["slab_begin"] == 8064 and p["launches"] == 2
+    assert (p["slabs"], p["slab_positions"], p["slab_blocks"]) == (1, 256, 512)
+    assert p["matrix_grid"] == (2 * 512 + 512, 1, 1) and p["matrix_block"] == (64, 4, 1)
+    # keys and values quantized to different lengths: tiles over what both have, slabs over the rest
+    p = _lib.attn_plan(_step(16, 32, 32, 2, REF, 8064, 4, REF, 7968, 8192))
+    assert p["matrix"] and p["slab_begin"] == 7968 and p["slabs"] == 1 and p["launches"] == 2
     # configs[4]'s size: the vector-ALU slab kernel from position 0
     p = _lib.attn_plan(_step(4, 32, 32, 4, REF, 2176, 4, REF, 2176, 2304))
     assert not p["matrix"] and p["slab_begin"] == 0 and p["slabs"] == 5 and p["launches"] == 2
@@ -197,12 +201,12 @@ def test_no_attention_step_is_given_a_tile_longer_than_its_quantized_part():
                                 continue
                             assert rc == 0, (rc, k_bits, k_fmt, v_bits, batch, k_tokens, v_tokens, width)
                             if plan.matrix:
-                                assert k_tokens >= 1024 and k_tokens % 32 == 0 and k_tokens == v_tokens
-                                assert batch * heads <= 65535
-                                assert plan.matrix_tiles == (k_tokens + 1023) // 1024
-                                assert plan.matrix_grid[0] * plan.matrix_block[1] >= plan.matrix_tiles
-                                assert plan.matrix_grid[1] == batch * heads and 1 <= plan.matrix_block[1] <= 4
-                                assert plan.slab_begin == k_tokens
+                                both = min(k_tokens, v_tokens)
+                                assert both >= 1024 and both % 32 == 0 and unit == 32
+                                assert plan.slab_begin == both and plan.matrix_tiles == (both + 1023) // 1024
+                                blocks_per_head = (plan.matrix_grid[0] - plan.slab_blocks) // (batch * heads)
+                                assert blocks_per_head * plan.matrix_block[1] >= plan.matrix_tiles and plan.matrix_block[1] == 4
+                                assert plan.matrix_grid[0] == blocks_per_head * batch * heads + plan.slabs * batch * heads
                             else:
                                 assert plan.slab_begin == 0 and plan.matrix_tiles == 0
                             assert plan.slab_begin + plan.slabs * plan.slab_positions >= width

@@ -255,3 +255,34 @@ def test_matrix_core_slabs_with_short_rows_and_device_side_lengths(dev):
     got2, _ = ops.decode_attention(q, kq, vq, kwin, vwin, kg, k_bits, 32, v_bits, k_tail_len=klen, v_tail_len=klen.clone(),
                                    single_pass=True, **fmt)
     assert torch.equal(got2, got)
+
+
+@pytest.mark.parametrize("k_bits,v_bits,tk,tv", [(4, 2, 8064, 7968), (2, 4, 4000 // 32 * 32, 4096), (1, 3, 4096, 4096 + 32),
+                                                 (4, 4, 8064, 8064)])
+def test_matrix_core_steps_with_keys_and_values_quantized_to_different_lengths(dev, k_bits, v_bits, tk, tv):
+    """The matrix-core tiles cover the positions quantized on both sides; what lies between the two quantized lengths
+    (codes on one side, the fp16 tail on the other) and the tails run as vector-ALU slabs in the same launch.  Against
+    the four-launch step and, for two rows, fp64 attention over the dequantized cache; the library is asked first
+    whether these sizes take the matrix-core form, with two launches (tiles + slabs, merge)."""
+    from kvmix_amd import ops, _lib
+    from helpers import dequantize_torch
+
+    gen = torch.Generator(device=dev).manual_seed(300 + tk % 97 + tv % 89)
+    rng = np.random.default_rng(tk + tv)
+    B, nkv, rep = 2, 32, 2
+    n = max(tk, tv) + 61
+    plan = _lib.attn_plan(_lib.attn_step_descriptor(B, nkv * rep, nkv, 128, k_bits, 0, 32, tk, v_bits, 1 if v_bits == 3 else 0, 32, tv,
+                                                   n - tk, n - tv))
+    assert plan["matrix"] and plan["launches"] == 2 and plan["slab_begin"] == min(tk, tv), plan
+    q, kq, vq, k_tail, v_tail, kg, mask, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tv, n, mask_rng=rng)
+    out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, **fmt)
+    out_s, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
+    vm = v_magnitude(vq, v_tail, v_bits)
+    check(out_s, out_f, vm)
+    sl = slice(B - 1, B)
+    kd = dequantize_torch(kq[0][sl, :2], kq[1][sl, :2], kq[2][sl, :2], k_bits, 32).double()
+    vd = dequantize_torch(vq[0][sl, :2], vq[1][sl, :2], vq[2][sl, :2], v_bits, 32, dense3=v_bits == 3).double()
+    keys = torch.cat([kd.transpose(2, 3), k_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    logits = (q[sl, :2 * rep].double() @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
+    check(out_s[sl, :2 * rep], torch.softmax(logits, -1) @ vals, vm)
