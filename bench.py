@@ -504,9 +504,12 @@ def attention_step_extra(torch, dev, shapes=None):
     H, D, R = 32, 128, 128
     res = {}
     side = torch.cuda.Stream()
+    # (3-bit keys: the reference's words of 11 codes; 3-bit values: the dense stream)
     for (B, T, kb, vb) in shapes or [(1, 4096, 4, 4), (4, 2304, 4, 4), (4, 2304, 3, 2), (4, 2304, 2, 2), (8, 8192, 4, 4),
-                                     (16, 8192, 4, 4)]:
+                                     (16, 8192, 4, 4), (8, 8192, 2, 2), (16, 8192, 2, 2), (8, 8192, 3, 2), (16, 8192, 3, 2),
+                                     (8, 8192, 2, 4), (16, 8192, 2, 4), (8, 8192, 3, 3), (16, 8192, 3, 3)]:
         kg = 11 if kb == 3 else 32
+        vfmt = ops.FMT_DENSE3 if vb == 3 else ops.FMT_REF
         tk, tv = ((T - R) // kg) * kg, ((T - R) // 32) * 32
         kbytes = (1024 / 11 if kb == 3 else 16 * kb + 16) * tk
         nbytes = B * H * (kbytes + (16 * vb + 16) * tv + (2 * T - tk - tv) * 2 * D)
@@ -524,7 +527,7 @@ def attention_step_extra(torch, dev, shapes=None):
         for name, single in (("four_launch", False), ("single_pass", True)):
             def fn(i):
                 kq, vq, kt, vt = sets[i % nsets]
-                return ops.decode_attention(q, kq, vq, kt, vt, kg, kb, 32, vb, single_pass=single)
+                return ops.decode_attention(q, kq, vq, kt, vt, kg, kb, 32, vb, v_fmt=vfmt, single_pass=single)
             iters = max(100, 2 * nsets)
             with torch.cuda.stream(side):
                 for i in range(max(nsets, 20)):
@@ -544,9 +547,9 @@ def attention_step_extra(torch, dev, shapes=None):
             us = s.elapsed_time(e) * 1e3 / iters
             del graph
             entry[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
-        entry["chosen"] = "single_pass" if ops.prefer_single_pass(B, H, H, D, T, kb, 0, kg, vb, 0, 32, k_tokens=tk,
+        entry["chosen"] = "single_pass" if ops.prefer_single_pass(B, H, H, D, T, kb, 0, kg, vb, vfmt, 32, k_tokens=tk,
                                                                    v_tokens=tv) else "four_launch"
-        res[f"B{B}_T{T}_k{kb}v{vb}"] = entry
+        res[f"B{B}_T{T}_k{'ref3' if kb == 3 else kb}v{'dense3' if vb == 3 else vb}"] = entry
         del sets
         torch.cuda.empty_cache()
     return res

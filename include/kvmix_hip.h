@@ -323,8 +323,11 @@ int kvmix_decode_attention_fused(const kvmix_decode_attn_t *step, void *workspac
  */
 typedef struct kvmix_attn_plan {
     int matrix;              /* 1: the positions [0, slab_begin) run on the matrix cores, one wave per tile */
+    int recommended;         /* 1: at these sizes the single pass is the faster form (measured), 0: the four launches
+                              * of kvmix_decode_attention are */
     int launches;            /* kernel launches of the step, the merge included */
-    int64_t matrix_tiles;    /* tiles of 1024 positions per query head (0 without the matrix-core kernel) */
+    int64_t matrix_tiles;    /* tiles of 1024 positions (1408 with the reference's 3-bit keys) per query head; 0
+                              * without the matrix-core kernel */
     int64_t slab_positions;  /* positions per vector-ALU slab */
     int64_t slab_begin;      /* first position those slabs cover */
     int64_t slabs;           /* their number per query head */

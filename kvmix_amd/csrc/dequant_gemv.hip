@@ -2011,6 +2011,172 @@ gemv_cols_mfma2(GemvArgs a)
     finish_tile(items - 1);
 }
 
+// The value phase of a matrix-core slab: out[128] += sum over the slab's NCH * 128 positions [t_first, ...) of
+// p[position] * value[position][:], as gemv_rows_mfma does it (chunks of 128 rows, p * scale * 2^90 in three bf16
+// parts as the A operand), with p taken from the wave's LDS row `pbuf` (position order, fp32) instead of an fp16
+// vector in memory.  (m, l) of the slab and its 128 unnormalised outputs go to the workspace as slab `tile` of the
+// row.  `atile`: the wave's A tile (kRowsMfmaTile bf16).
+template <int VMODE, int NCH>
+__device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t kv, int64_t sample, int tile, int t_first,
+                                                 uint16_t *atile, const float *pbuf, float slab_m, float slab_l)
+{
+    constexpr int NPOS = 8;
+    constexpr int BITS = VMODE;
+    using Elem = typename CodeElem<BITS>::type;
+    constexpr int EB = BITS == 30 ? 3 : BITS, FB = BITS == 30 ? 3 : BITS;
+    constexpr int LPR = 4, EPR = 16, RL = kWave / EPR, RKB = 4 * RL, CH = 128, KB = CH / RKB, FPB = 8 / FB;
+    const int lane = threadIdx.x;
+    const int rs = lane / EPR, wi = lane % EPR;
+    const int t_end = t_first + NCH * 128;
+    const uint8_t *cp = reinterpret_cast<const uint8_t *>(a.v_code + kv * a.vc_bs) +
+                        (BITS == 30 ? (wi / 4) * 12 + (wi % 4 < 2 ? wi % 4 : 2) * 4 : wi * EB);
+    [[maybe_unused]] const uint32_t sh3 = (uint32_t)(24 * (wi % 4)) % 32u;
+    const uint16_t *sp = a.v_scale + kv * a.vsz_bs;
+    const uint16_t *zp = a.v_zero + kv * a.vsz_bs;
+
+    f32x4_t acc[NPOS];
+    float zacc[LPR];
+#pragma unroll
+    for (int p = 0; p < NPOS; p++) acc[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < LPR; g++) zacc[g] = 0.f;
+    auto cell = [](int t, int l) { return ((4 * t + l / EPR) * 17 + (l % EPR)) * 4 + (t >> 2) * 4; };
+    const int row0 = 2 * lane;
+    int aoff[2];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const int r = row0 + e;
+        aoff[e] = cell(r / RKB, (r % RL) * EPR) + (r % RKB) / RL;
+    }
+    Half8 s8, z8;
+    Elem w[KB][4];
+    // (a chunk past the slab's end -- the prefetch of the last step -- is the last chunk again)
+    auto chunk_base = [&](int k0) { return k0 + CH <= t_end ? k0 : max(t_end - CH, 0); };
+    auto load_small = [&](int k0) {
+        const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
+        s8 = ld_stream<Half8>(sp + kr * LPR);
+        z8 = ld_stream<Half8>(zp + kr * LPR);
+    };
+    auto load_codes = [&](int k0, int t) {
+        const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
+    };
+    auto stage = [&](int k0) {
+        const float2 pv = *reinterpret_cast<const float2 *>(pbuf + (k0 - t_first) + row0);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int q = e / LPR, g = e % LPR;
+            const float xv = q == 0 ? pv.x : pv.y;
+            zacc[g] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[g]);
+            // p * scale * 2^90 in three bf16 parts by truncation (24 of the product's bits)
+            const float v0 = (xv * 1237940039285380274899124224.0f) * h16_to_f32(s8.v[e]);
+            const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
+            const float v1 = v0 - __uint_as_float(b0);
+            const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
+            const float v2 = v1 - __uint_as_float(b1);
+            const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+#pragma unroll
+            for (int pt = 0; pt < 3; pt++) atile[aoff[q] + g * 16 + pt * 4] = (uint16_t)(part[pt] >> 16);
+        }
+    };
+    auto compute = [&](int t) {
+        const bf16x4_t av = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, lane));
+        if constexpr (BITS == 30) {
+            uint32_t v[4], u[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t lo = __builtin_amdgcn_mov_dpp(w[t][k], 0x90, 0xf, 0xf, false);
+                const uint32_t hi = __builtin_amdgcn_mov_dpp(w[t][k], 0xA4, 0xf, 0xf, false);
+                v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
+                u[k] = v[k] >> 4;
+            }
+#pragma unroll
+            for (int mm = 0; mm < 4; mm++) {
+                const bool from_u = mm == 1 || mm == 2;
+                const uint32_t b = from_u ? (uint32_t)(mm - 1) : (mm == 0 ? 0u : 2u);
+                const uint32_t sel = 0x0c000c00u | b | ((4u + b) << 16);
+                const uint32_t *src = from_u ? u : v;
+                const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
+                const int o0 = mm % 2 == 0 ? 0 : 2;
+#pragma unroll
+                for (int f = 0; f < 2; f++) {
+                    const uint32_t mask = 0x00070007u << (o0 + 3 * f);
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+                    acc[mm * 2 + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[mm * 2 + f], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < EB; b++) {
+                const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[t][1], (uint32_t)w[t][0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[t][3], (uint32_t)w[t][2], sel);
+#pragma unroll
+                for (int f = 0; f < FPB; f++) {
+                    const bf16x4_t bv =
+                        __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
+                    acc[b * FPB + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[b * FPB + f], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    load_small(t_first);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < KB; t++) {
+        load_codes(t_first, t);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int i = lane; i < kRowsMfmaTile / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+    wave_lds_fence();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+    for (int k0 = t_first; k0 < t_end; k0 += CH) {
+        stage(k0);
+        wave_lds_fence();
+        load_small(k0 + CH);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < KB; t++) {
+            compute(t);
+            load_codes(k0 + CH, t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wave_lds_fence();
+    }
+
+    // zero term of the lane's group; code sums; the four row slots (lane bits 4, 5) meet
+    float z[LPR];
+#pragma unroll
+    for (int g = 0; g < LPR; g++) z[g] = zacc[g];
+    scatter_reduce<LPR, 8, 0>(z, lane);
+    z[0] += __shfl_xor(z[0], 1);
+    z[0] += __shfl_xor(z[0], 2);
+    z[0] += __shfl_xor(z[0], 16);
+    z[0] += __shfl_xor(z[0], 32);
+    float sums[NPOS], flat[NPOS];
+#pragma unroll
+    for (int p = 0; p < NPOS; p++) sums[p] = (acc[p][0] + acc[p][1]) + acc[p][2];
+#pragma unroll
+    for (int p = 0; p < NPOS; p++) {
+        const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
+        const float sum = BITS == 30 ? sums[p] : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+        flat[p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
+    }
+    const int first = scatter_reduce<NPOS, 16, 1>(flat, lane);  // two of the lane's eight columns are left
+    float *wo = a.ws_o + ((int64_t)sample * a.slabs + tile) * 128 + wi * NPOS + first;
+    wo[0] = flat[0] + z[0];
+    wo[1] = flat[1] + z[0];
+    if (lane == 0) {
+        float *ml = a.ws_ml + ((int64_t)sample * a.slabs + tile) * 2;
+        ml[0] = slab_m;
+        ml[1] = slab_l;
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // attn_slab_mfma<KBITS, VMODE>   the single-pass decode step over the quantized positions, on the matrix
 // cores: one wave = one slab of 1024 positions of one query head (D = 128).
@@ -2241,171 +2407,167 @@ __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64
         wave_lds_fence();
     }
 
-    // ---- 2. p.V over the slab's 1024 positions: gemv_rows_mfma's chunks ---------------------------------
+    // ---- 2. p.V over the slab's 1024 positions ------------------------------------------------------------
+    slab_value_phase<VMODE, 8>(a, kv, sample, tile, g_first * 32, atile, pbuf, slab_m, slab_l);
+}
+
+// ---------------------------------------------------------------------------------------
+// attn_slab_ref3_body<VMODE>   the same slab for keys in the reference's 3-bit words (11 codes and an own scale and
+// zero per word): one wave = 128 words = 1408 positions of one query head (4 * lcm(11, 32): whole words of the keys
+// and whole 128-row chunks of the values).
+//   1. logits as gemv_cols3 computes them, one head per pass and no K slicing: a lane owns two words of every
+//      channel row (8 + 4 + 4 bytes per row straight to registers, eight rows in flight), codes multiplied in as
+//      fp32 bit patterns; the query, times 2^90, sits in the wave's LDS.
+//   2. 3. as above, the value phase over eleven chunks.
+//   `tokens` is a multiple of 352 here; the last tile is moved back to end there.
+// ---------------------------------------------------------------------------------------
+constexpr int kSlabRef3Words = 128;                       // words per tile and channel row
+constexpr int kSlabRef3Tile = kSlabRef3Words * 11;        // positions per tile
+constexpr int kSlabRef3ABytes = (kRowsMfmaTile * 2 + 15) / 16 * 16;
+constexpr int kSlabRef3Lds = 128 * 4 + kSlabRef3ABytes + kSlabRef3Tile * 4;   // query, A tile of the value phase, probabilities
+
+template <int VMODE>
+__device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64_t bx, int64_t sample, float *lds)
+{
+    constexpr int K = 128, U = 8, UPL = 2, VALS = 11, TW = kSlabRef3Words;
+    const int lane = threadIdx.x;
+    const int wy = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int nw = (int)blockDim.y;
+    uint8_t *mine = reinterpret_cast<uint8_t *>(lds) + wy * kSlabRef3Lds;
+    float *xs = reinterpret_cast<float *>(mine);                                  // [128] query * 2^90
+    uint16_t *atile = reinterpret_cast<uint16_t *>(mine + K * 4);
+    float *pbuf = reinterpret_cast<float *>(mine + K * 4 + kSlabRef3ABytes);      // [1408] probabilities of the slab
+    const int64_t kv = sample / a.heads_per_kv;
+    const int nwords = (int)(a.tokens / VALS);
+    const int tile = (int)bx * nw + wy;
+    if (nwords < TW) return;  // (never launched so: a slab longer than the row would leave the operands)
+    if (tile * TW >= nwords) return;
+    const int w_first = tile * TW + TW <= nwords ? tile * TW : max(nwords - TW, 0);  // (the last tile ends at `tokens`)
+    const int shift = tile * TW - w_first;                                             // its first words are the neighbour's
+    float slab_m, slab_l;
     {
-        constexpr int BITS = VMODE;
-        using Elem = typename CodeElem<BITS>::type;
-        constexpr int EB = BITS == 30 ? 3 : BITS, FB = BITS == 30 ? 3 : BITS;
-        constexpr int LPR = 4, EPR = 16, RL = kWave / EPR, RKB = 4 * RL, CH = 128, KB = CH / RKB, FPB = 8 / FB;
-        const int rs = lane / EPR, wi = lane % EPR;
-        const int t_first = g_first * 32, t_end = t_first + 1024;
-        const uint8_t *cp = reinterpret_cast<const uint8_t *>(a.v_code + kv * a.vc_bs) +
-                            (BITS == 30 ? (wi / 4) * 12 + (wi % 4 < 2 ? wi % 4 : 2) * 4 : wi * EB);
-        [[maybe_unused]] const uint32_t sh3 = (uint32_t)(24 * (wi % 4)) % 32u;
-        const uint16_t *sp = a.v_scale + kv * a.vsz_bs;
-        const uint16_t *zp = a.v_zero + kv * a.vsz_bs;
-
-        f32x4_t acc[NPOS];
-        float zacc[LPR];
-#pragma unroll
-        for (int p = 0; p < NPOS; p++) acc[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int g = 0; g < LPR; g++) zacc[g] = 0.f;
-        auto cell = [](int t, int l) { return ((4 * t + l / EPR) * 17 + (l % EPR)) * 4 + (t >> 2) * 4; };
-        const int row0 = 2 * lane;
-        int aoff[2];
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const int r = row0 + e;
-            aoff[e] = cell(r / RKB, (r % RL) * EPR) + (r % RKB) / RL;
-        }
-        Half8 s8, z8;
-        Elem w[KB][4];
-        // (a chunk past the slab's end -- the prefetch of the last step -- is the last chunk again)
-        auto chunk_base = [&](int k0) { return k0 + CH <= t_end ? k0 : max(t_end - CH, 0); };
-        auto load_small = [&](int k0) {
-            const uint32_t kr = (uint32_t)(chunk_base(k0) + row0);
-            s8 = ld_stream<Half8>(sp + kr * LPR);
-            z8 = ld_stream<Half8>(zp + kr * LPR);
-        };
-        auto load_codes = [&](int k0, int t) {
-            const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
-#pragma unroll
-            for (int k = 0; k < 4; k++) w[t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
-        };
-        auto stage = [&](int k0) {
-            const float2 pv = *reinterpret_cast<const float2 *>(pbuf + (k0 - t_first) + row0);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int q = e / LPR, g = e % LPR;
-                const float xv = q == 0 ? pv.x : pv.y;
-                zacc[g] = fmaf(xv, h16_to_f32(z8.v[e]), zacc[g]);
-                // p * scale * 2^90 in three bf16 parts by truncation (24 of the product's bits)
-                const float v0 = (xv * 1237940039285380274899124224.0f) * h16_to_f32(s8.v[e]);
-                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
-                const float v1 = v0 - __uint_as_float(b0);
-                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
-                const float v2 = v1 - __uint_as_float(b1);
-                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
-#pragma unroll
-                for (int pt = 0; pt < 3; pt++) atile[aoff[q] + g * 16 + pt * 4] = (uint16_t)(part[pt] >> 16);
-            }
-        };
-        auto compute = [&](int t) {
-            const bf16x4_t av = *reinterpret_cast<const bf16x4_t *>(atile + cell(t, lane));
-            if constexpr (BITS == 30) {
-                uint32_t v[4], u[4];
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint32_t lo = __builtin_amdgcn_mov_dpp(w[t][k], 0x90, 0xf, 0xf, false);
-                    const uint32_t hi = __builtin_amdgcn_mov_dpp(w[t][k], 0xA4, 0xf, 0xf, false);
-                    v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
-                    u[k] = v[k] >> 4;
-                }
-#pragma unroll
-                for (int mm = 0; mm < 4; mm++) {
-                    const bool from_u = mm == 1 || mm == 2;
-                    const uint32_t b = from_u ? (uint32_t)(mm - 1) : (mm == 0 ? 0u : 2u);
-                    const uint32_t sel = 0x0c000c00u | b | ((4u + b) << 16);
-                    const uint32_t *src = from_u ? u : v;
-                    const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
-                    const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
-                    const int o0 = mm % 2 == 0 ? 0 : 2;
-#pragma unroll
-                    for (int f = 0; f < 2; f++) {
-                        const uint32_t mask = 0x00070007u << (o0 + 3 * f);
-                        const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
-                        acc[mm * 2 + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[mm * 2 + f], 0, 0, 0);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int b = 0; b < EB; b++) {
-                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-                    const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[t][1], (uint32_t)w[t][0], sel);
-                    const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[t][3], (uint32_t)w[t][2], sel);
-#pragma unroll
-                    for (int f = 0; f < FPB; f++) {
-                        const bf16x4_t bv =
-                            __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
-                        acc[b * FPB + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[b * FPB + f], 0, 0, 0);
-                    }
-                }
-            }
-        };
-
-        load_small(t_first);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < KB; t++) {
-            load_codes(t_first, t);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        for (int i = lane; i < kRowsMfmaTile / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
+        const uint16_t *qp = a.q + sample * a.q_bs;
+        for (int i = lane; i < K; i += kWave) xs[i] = h16_to_f32(qp[i]) * 1237940039285380274899124224.0f;  // 2^90
         wave_lds_fence();
-        __builtin_amdgcn_sched_barrier(0);
+
+        float acc[UPL][VALS], zsum[UPL];
+#pragma unroll
+        for (int j = 0; j < UPL; j++) {
+            zsum[j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < VALS; i++) acc[j][i] = 0.f;
+        }
+        struct __attribute__((packed, aligned(2))) Half2x {
+            uint16_t v[UPL];
+        };
+        Words<UPL> cw[U];
+        Half2x sw[U], zw[U];
+        // uniform bases and 32-bit byte offsets per lane, one running offset per array (gemv_cols3's walk)
+        const uint8_t *cb = reinterpret_cast<const uint8_t *>(a.k_code + kv * a.kc_bs);
+        const uint8_t *sb = reinterpret_cast<const uint8_t *>(a.k_scale + kv * a.ksz_bs);
+        const uint8_t *zb = reinterpret_cast<const uint8_t *>(a.k_zero + kv * a.ksz_bs);
+        const uint32_t unit0 = (uint32_t)(w_first + lane * UPL);
+        uint32_t co = unit0 * 4u, so = unit0 * 2u;
+        const uint32_t c_step = (uint32_t)a.kc_rs * 4u, s_step = (uint32_t)a.ksz_rs * 2u;
+        auto next_row = [&](int u) {
+            cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cb + co);
+            sw[u] = ld_stream<Half2x, KVMIX_COLS3_NT_SZ>(sb + so);
+            zw[u] = ld_stream<Half2x, KVMIX_COLS3_NT_SZ>(zb + so);
+            co += c_step;
+            so += s_step;
+        };
+        float xr[U];
+        auto compute_row = [&](int u) {
+            const float xv = xr[u];
+#pragma unroll
+            for (int j = 0; j < UPL; j++) {
+                const half2_t sz = __builtin_bit_cast(half2_t, (uint32_t)sw[u].v[j] | ((uint32_t)zw[u].v[j] << 16));
+                // (a masked field of the word is code * 2^(offset - 149) as an fp32 pattern: see gemv_cols3)
+                const uint32_t w = cw[u].v[j], hi = w >> 24;
+                float f[VALS];
+#pragma unroll
+                for (int i = 0; i < 8; i++) f[i] = __uint_as_float(w & (7u << (3 * i)));
+                f[8] = __uint_as_float(hi & 0x07u);
+                f[9] = __uint_as_float(hi & 0x38u);
+                f[10] = __uint_as_float(hi & 0xC0u);
+                zsum[j] = fmaf(xv, (float)sz.y, zsum[j]);
+                const float mq = fmaf(xv, (float)sz.x, 0.f);
+#pragma unroll
+                for (int i = 0; i < VALS; i++) acc[j][i] = fmaf(mq, f[i], acc[j][i]);
+            }
+        };
+        constexpr int steps = K / U;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            next_row(u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll 1
-        for (int k0 = t_first; k0 < t_end; k0 += CH) {
-            stage(k0);
-            wave_lds_fence();
-            load_small(k0 + CH);
+        for (int st = 0; st < steps - 1; st++) {
+#pragma unroll
+            for (int u = 0; u < U; u++) xr[u] = xs[st * U + u];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int t = 0; t < KB; t++) {
-                compute(t);
-                load_codes(k0 + CH, t);
+            for (int u = 0; u < U; u++) {
+                compute_row(u);
+                next_row(u);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            wave_lds_fence();
         }
+#pragma unroll
+        for (int u = 0; u < U; u++) xr[u] = xs[(steps - 1) * U + u];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; u++) compute_row(u);
 
-        // zero term of the lane's group; code sums; the four row slots (lane bits 4, 5) meet
-        float z[LPR];
+        // the logits of this lane's 22 positions: fp16 rounding, 1/sqrt(D), mask as in the reference
+        const float *mrow = a.mask ? a.mask + (sample / a.heads) * a.mask_bs + (int64_t)w_first * VALS : nullptr;
+        float x[UPL][VALS];
+        float mx = -INFINITY;
 #pragma unroll
-        for (int g = 0; g < LPR; g++) z[g] = zacc[g];
-        scatter_reduce<LPR, 8, 0>(z, lane);
-        z[0] += __shfl_xor(z[0], 1);
-        z[0] += __shfl_xor(z[0], 2);
-        z[0] += __shfl_xor(z[0], 16);
-        z[0] += __shfl_xor(z[0], 32);
-        float sums[NPOS], flat[NPOS];
+        for (int j = 0; j < UPL; j++) {
+            const int wj = lane * UPL + j;  // word of the tile
 #pragma unroll
-        for (int p = 0; p < NPOS; p++) sums[p] = (acc[p][0] + acc[p][1]) + acc[p][2];
-#pragma unroll
-        for (int p = 0; p < NPOS; p++) {
-            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
-            const float sum = BITS == 30 ? sums[p] : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
-            flat[p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
+            for (int i = 0; i < VALS; i++) {
+                const float dot = fmaf(acc[j][i], cols3_out_scale(i), zsum[j] * kCols3ZeroDown);
+                float lg = h16_to_f32(f32_to_h16(dot)) * a.inv_sqrt_d;
+                if (mrow) lg = fmaxf(lg + mrow[wj * VALS + i], -3.4028234663852886e38f);
+                x[j][i] = wj >= shift ? lg : -INFINITY;
+                mx = fmaxf(mx, x[j][i]);
+            }
         }
-        const int first = scatter_reduce<NPOS, 16, 1>(flat, lane);  // two of the lane's eight columns are left
-        float *wo = a.ws_o + ((int64_t)sample * a.slabs + tile) * 128 + wi * NPOS + first;
-        wo[0] = flat[0] + z[0];
-        wo[1] = flat[1] + z[0];
-        if (lane == 0) {
-            float *ml = a.ws_ml + ((int64_t)sample * a.slabs + tile) * 2;
-            ml[0] = slab_m;
-            ml[1] = slab_l;
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < UPL; j++) {
+#pragma unroll
+            for (int i = 0; i < VALS; i++) {
+                const float e = x[j][i] == -INFINITY ? 0.f : expf(x[j][i] - mx);
+                sum += e;
+                pbuf[(lane * UPL + j) * VALS + i] = e;
+            }
         }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+        slab_m = mx;
+        slab_l = sum;
+        wave_lds_fence();
     }
+    slab_value_phase<VMODE, kSlabRef3Tile / 128>(a, kv, sample, tile, w_first * VALS, atile, pbuf, slab_m, slab_l);
 }
 
 // The launch of a large single-pass step: blocks [0, mfma_blocks) are the matrix-core tiles above (mfma_nx blocks per
 // query head, XCD-swizzled), the rest are slabs of the vector-ALU kind (fused_slab.h, 8 lanes per key row = 256
 // threads) over the positions the tiles do not cover: the fp16 tails, and quantized positions where keys and values
 // are quantized to different lengths.  One launch instead of two; attn_fused_merge follows.
-// block = (64, 4); dynamic LDS = kStepLds.
-constexpr size_t kStepLds = 4 * kSlabLds > fused::SlabCfg<8>::lds_floats(1) * sizeof(float) ? 4 * kSlabLds
-                                                                                           : fused::SlabCfg<8>::lds_floats(1) * sizeof(float);
+// KBITS: 1, 2, 4, or 3 = the reference's 3-bit words (tiles of 1408 positions).  block = (64, 4); dynamic LDS = step_lds(KBITS).
+constexpr size_t step_lds(int k_mode)
+{
+    const size_t tiles = (size_t)kColsWaves * (k_mode == 3 ? kSlabRef3Lds : kSlabLds);
+    const size_t slab = fused::SlabCfg<8>::lds_floats(1) * sizeof(float);
+    return tiles > slab ? tiles : slab;
+}
 template <int KBITS, int VMODE>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
 attn_step_mfma(AttnSlabArgs m, fused::FusedArgs f, unsigned mfma_blocks, unsigned mfma_nx)
@@ -2417,7 +2579,10 @@ attn_step_mfma(AttnSlabArgs m, fused::FusedArgs f, unsigned mfma_blocks, unsigne
         const int64_t n = mfma_blocks, l = blockIdx.x;
         const int64_t xcd = l % kXcds, slot = l / kXcds, per = n / kXcds, rem = n % kXcds;
         const int64_t j = xcd * per + (xcd < rem ? xcd : rem) + slot;
-        attn_slab_mfma_body<KBITS, VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
+        if constexpr (KBITS == 3)
+            attn_slab_ref3_body<VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
+        else
+            attn_slab_mfma_body<KBITS, VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
     } else {
         fused::attn_fused_slab_body<1, 8>(f, (int64_t)blockIdx.x - mfma_blocks, (int64_t)gridDim.x - mfma_blocks,
                                           (int)(threadIdx.y * kWave + threadIdx.x), lds);
@@ -2832,10 +2997,11 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     }
 }
 
-int plan_attn_slab_mfma(int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3])
+int plan_attn_slab_mfma(int k_mode, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3])
 {
-    const int64_t tiles = (tokens / 32 + 31) / 32;
-    if (tokens < 1024 || tokens % 32 != 0 || samples <= 0 || tail_blocks < 0) return KVMIX_ERR_SHAPE;
+    const int64_t tile = k_mode == 3 ? kSlabRef3Tile : 1024, unit = k_mode == 3 ? 352 : 32;
+    const int64_t tiles = (tokens + tile - 1) / tile;
+    if (tokens < tile || tokens % unit != 0 || samples <= 0 || tail_blocks < 0) return KVMIX_ERR_SHAPE;
     const int64_t nx = (tiles + kColsWaves - 1) / kColsWaves;  // blocks of four tiles per query head
     if (nx * samples + tail_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
     grid[0] = (unsigned)(nx * samples + tail_blocks), grid[1] = 1, grid[2] = 1;
@@ -2847,11 +3013,11 @@ int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int 
                           int64_t tail_blocks, hipStream_t stream)
 {
     unsigned g[3], b[3];
-    const int prc = plan_attn_slab_mfma(a.tokens, samples, tail_blocks, g, b);
+    const int prc = plan_attn_slab_mfma(k_bits, a.tokens, samples, tail_blocks, g, b);
     if (prc != KVMIX_OK) return prc;
     const dim3 grid(g[0]), block(b[0], b[1]);
     const unsigned mfma_blocks = (unsigned)(g[0] - tail_blocks), mfma_nx = (unsigned)(mfma_blocks / samples);
-    const size_t lds = kStepLds;
+    const size_t lds = step_lds(k_bits);
 #define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_step_mfma<KB_, VM_>), grid, block, lds, stream, a, f, mfma_blocks, mfma_nx)
 #define KVMIX_SLAB_V(KB_)                          \
     switch (v_mode) {                              \
@@ -2864,6 +3030,7 @@ int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int 
     switch (k_bits) {
     case 1: KVMIX_SLAB_V(1) break;
     case 2: KVMIX_SLAB_V(2) break;
+    case 3: KVMIX_SLAB_V(3) break;
     case 4: KVMIX_SLAB_V(4) break;
     default: return KVMIX_ERR_UNSUPPORTED;
     }

@@ -115,12 +115,14 @@ static int64_t fused_slabs(const kvmix_decode_attn_t *p)
     return (fused_width(p) + s - 1) / s;
 }
 
-// How a row's positions are divided into slabs.  Large steps with keys of 1, 2 or 4 bits take the positions that
-// are quantized on both sides, [0, min(k_tokens, v_tokens)), through the matrix-core tiles (attn_slab_mfma_body: 1024
-// positions per wave, the formats of gemv_cols_mfma2 and gemv_rows_mfma) and the rest -- the fp16 tails, and the few
+// How a row's positions are divided into slabs.  Large steps with keys of 1, 2 or 4 bits or in the reference's 3-bit
+// words take the positions that are quantized on both sides, [0, min(k_tokens, v_tokens)), through the matrix-core
+// tiles (attn_slab_mfma_body: 1024 positions per wave, the formats of gemv_cols_mfma2 and gemv_rows_mfma;
+// attn_slab_ref3_body: 1408 positions, gemv_cols3's arithmetic for the keys) and the rest -- the fp16 tails, and the few
 // positions quantized on one side only when keys and values are quantized to different lengths -- through slabs of
 // the vector-ALU kind that run as trailing blocks of the same launch (256 threads, 256 positions each); everything
 // else goes through attn_fused_slab (512 threads) from position 0.
+constexpr int64_t kSmallStepEntries = 1 << 19, kSmallStepEntriesRef3 = 360000;  // (see kvmix_decode_attention_fused_plan)
 constexpr int64_t kSlabMfmaMinWaves = 512;  // (measured: 512 waves 34 against 38 us, 256 waves 33 against 25 us)
 struct FusedLayout {
     bool mfma;
@@ -136,9 +138,12 @@ static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
     FusedLayout l{false, 0, fused_slabs(p), 0, fused_slab(p)};
     const int km = fused_key_mode(p), vm = fused_value_mode(p);
     const int vbits = vm == 3 ? 3 : vm;
-    const int64_t both = (p->k_tokens < p->v_tokens ? p->k_tokens : p->v_tokens) / 32 * 32;  // quantized on both sides
-    const int64_t tiles = (both / 32 + 31) / 32;
-    if (both >= 1024 && (km == 1 || km == 2 || km == 4) && vm != 0 &&
+    // positions quantized on both sides, in whole words of the keys and whole groups of the values; tiles of 1024
+    // positions, or 1408 with the reference's 3-bit keys
+    const int64_t unit = km == 3 ? 352 : 32, tile = km == 3 ? 1408 : 1024;
+    const int64_t both = (p->k_tokens < p->v_tokens ? p->k_tokens : p->v_tokens) / unit * unit;
+    const int64_t tiles = (both + tile - 1) / tile;
+    if (both >= tile && (km == 1 || km == 2 || km == 3 || km == 4) && vm != 0 &&
         p->v_code_row_stride == kFusedD * vbits / 32 && p->v_sz_row_stride == kFusedD / 32 &&
         (kFusedD + 1) * p->k_code_row_stride < (1ll << 29) && (kFusedD + 1) * p->k_sz_row_stride < (1ll << 30) &&
         // (the value phase forms 32-bit byte offsets of code rows and 32-bit element offsets of scale rows)
@@ -147,7 +152,7 @@ static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
         l.mfma = true;
         l.tiles = tiles;
         l.t_begin = both;
-        l.slab = SlabCfg<8>::kSlabG32;
+        l.slab = km == 3 ? SlabCfg<8>::kSlabRef3 : SlabCfg<8>::kSlabG32;
         l.tail_slabs = (fused_width(p) - both + l.slab - 1) / l.slab;
     }
     return l;
@@ -217,13 +222,24 @@ extern "C" int kvmix_decode_attention_fused_plan(const kvmix_decode_attn_t *p, k
     if (rc != KVMIX_OK || p->samples == 0) return rc;
     const FusedLayout lay = fused_layout(p);
     plan->matrix = lay.mfma ? 1 : 0;
+    // Which form is faster (MI355X, Llama-2-7B heads, graph-replayed; four launches -> single pass, us): the
+    // vector-ALU slabs up to about 2^19 (query head x position) entries -- 1 x 4096: 29 -> 19, 4 x 2304: 31 -> 27..30 --
+    // earlier with the reference's 3-bit keys; beyond that only on the matrix cores, with keys of 1, 2 or 4 bits
+    // (8 x 8192: 4/4 bits 71 -> 61, 2/2 bits 54 -> 45, 2/4 bits 63 -> 52; 16 x 8192: 129 -> 116, 90 -> 80, 110 -> 98).
+    // The reference's 3-bit keys on the matrix-core tiles are correct but behind there (8 x 8192, 2-bit values:
+    // 69 -> 72, 16 x 8192: 124 -> 140): the key phase of a tile is one wave's vector arithmetic over all 128 rows.
+    {
+        const int64_t entries = p->samples * fused_width(p);
+        const bool ref3 = p->k_tokens > 0 && fused_key_mode(p) == 3;
+        plan->recommended = entries <= (ref3 ? kSmallStepEntriesRef3 : kSmallStepEntries) ? 1 : (lay.mfma && !ref3 ? 1 : 0);
+    }
     plan->matrix_tiles = lay.tiles;
     plan->slab_positions = lay.slab;
     plan->slab_begin = lay.t_begin;
     plan->slabs = lay.tail_slabs;
     if (lay.mfma) {
         // one launch: the tiles' blocks, then the slabs' blocks
-        const int prc = plan_attn_slab_mfma(lay.t_begin, p->samples, lay.tail_slabs * p->samples, plan->matrix_grid, plan->matrix_block);
+        const int prc = plan_attn_slab_mfma(fused_key_mode(p), lay.t_begin, p->samples, lay.tail_slabs * p->samples, plan->matrix_grid, plan->matrix_block);
         if (prc != KVMIX_OK) return prc;
         plan->slab_blocks = lay.tail_slabs * p->samples;
         plan->launches++;

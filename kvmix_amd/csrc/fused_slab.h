@@ -501,12 +501,13 @@ __device__ __forceinline__ void attn_fused_slab_body(const FusedArgs &a, int64_t
 
 // The launch of a large single-pass step (attn_step_mfma in dequant_gemv.hip): matrix-core tiles over the quantized
 // positions [0, a.tokens) plus `tail_blocks` vector-ALU slabs (8 lanes per key row, 256 threads; `f` describes them:
-// f.t_begin = a.tokens, f.slab0 = the number of tiles) over the rest.  k_bits in {1, 2, 4}; v_mode in {1, 2, 4, 30
-// (dense 3-bit)}.
+// f.t_begin = a.tokens, f.slab0 = the number of tiles) over the rest.  k_bits in {1, 2, 4} (tiles of 1024 positions,
+// a.tokens a multiple of 32) or 3 = the reference's 3-bit words (tiles of 1408, a.tokens a multiple of 352); v_mode
+// in {1, 2, 4, 30 (dense 3-bit)}.
 int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, int v_mode, int64_t samples,
                           int64_t tail_blocks, hipStream_t stream);
 // grid and block of that launch (KVMIX_ERR_SHAPE for sizes the kernel does not take: fewer positions than one tile,
 // not whole groups, too many blocks for a grid)
-int plan_attn_slab_mfma(int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3]);
+int plan_attn_slab_mfma(int k_mode, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3]);
 
 }  // namespace kvmix

@@ -277,36 +277,24 @@ def quantized_gemm(group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: 
     return out
 
 
-# Up to this many (batch x query head x position) entries the single-pass step is the faster one
-# (measured on MI355X, Llama-2-7B heads: 12-20 us against 20-30 us at 1-4 sequences of 2k-4k tokens;
-# equal at about 2^19 entries, i.e. 1024 blocks).  Keys in the reference's 3-bit words break even earlier.
-# Beyond that it is the faster one again where the library runs the quantized positions on the matrix cores
-# (16 x 8k 120 against 131 us, 4 x 8k 40 against 51 us); which steps those are is the library's decision and is
-# asked of it (kvmix_decode_attention_fused_plan), not repeated here.
-SINGLE_PASS_MAX_ENTRIES = 1 << 19
-SINGLE_PASS_MAX_ENTRIES_REF3 = 360_000
-
-
 def prefer_single_pass(batch: int, heads: int, kv_heads: int, head_dim: int, width: int, k_bits: int, k_fmt: int,
                        k_group: int, v_bits: int, v_fmt: int, v_group: int, k_tokens: int = None,
                        v_tokens: int = None) -> bool:
     """Policy for callers that do not need the probabilities: whether the single-pass step is both
-    available for this layout and the faster of the two at this size.  k_tokens / v_tokens: the quantized
-    lengths, where the caller knows them (they decide whether a large step can use the matrix cores: the
-    library is asked, kvmix_decode_attention_fused_plan)."""
+    available for this layout and the faster of the two at this size.  The library holds the measured rule
+    (kvmix_decode_attention_fused_plan: `recommended`); k_tokens / v_tokens are the quantized lengths, where the
+    caller knows them (they decide whether a large step can use the matrix cores; without them a step is
+    taken to have nothing quantized on both sides)."""
     if kv_heads <= 0 or heads % kv_heads != 0:
         return False
     if not single_pass_supported(head_dim, heads // kv_heads, k_bits, k_fmt, k_group, v_bits, v_fmt, v_group):
         return False
-    limit = SINGLE_PASS_MAX_ENTRIES_REF3 if (k_bits == 3 and k_fmt == _lib.FMT_REF) else SINGLE_PASS_MAX_ENTRIES
-    if batch * heads * width <= limit:
-        return True
     if k_tokens is None or v_tokens is None or width < max(k_tokens, v_tokens):
-        return False
+        k_tokens = v_tokens = 0
     step = _lib.attn_step_descriptor(batch, heads, kv_heads, head_dim, k_bits, k_fmt, k_group, k_tokens, v_bits, v_fmt,
                                      v_group, v_tokens, width - k_tokens, width - v_tokens)
     try:
-        return _lib.attn_plan(step)["matrix"]
+        return _lib.attn_plan(step)["recommended"]
     except RuntimeError:
         return False
 

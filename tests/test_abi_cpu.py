@@ -232,7 +232,11 @@ def test_single_pass_policy_knows_the_matrix_core_steps():
     large_unknown = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32)
     large = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32, k_tokens=8064, v_tokens=8064)
     uneven = ops.prefer_single_pass(16, 32, 32, 128, 8192, 4, 0, 32, 4, 0, 32, k_tokens=8064, v_tokens=8032)
-    ref3 = ops.prefer_single_pass(16, 32, 32, 128, 8192, 3, 0, 11, 4, 0, 32, k_tokens=8063, v_tokens=8063)
+    ref3 = ops.prefer_single_pass(16, 32, 32, 128, 8192, 3, 0, 11, 4, 0, 32, k_tokens=8063, v_tokens=8064)
     few = ops.prefer_single_pass(2, 32, 32, 128, 16384, 4, 0, 32, 4, 0, 32, k_tokens=2048, v_tokens=2048)
-    # (keys and values quantized to different lengths still take the matrix cores over what both have)
+    # (keys and values quantized to different lengths take the matrix cores over the positions both sides have
+    # quantized; the reference's 3-bit keys can, but the four launches are the faster form at that size)
     assert (small, large_unknown, large, uneven, ref3, few) == (True, False, True, True, False, False)
+    from kvmix_amd import _lib
+    plan = _lib.attn_plan(_lib.attn_step_descriptor(16, 32, 32, 128, 3, 0, 11, 8063, 4, 0, 32, 8064, 129, 128))
+    assert plan["matrix"] and not plan["recommended"]

@@ -168,6 +168,11 @@ def test_attention_step_plans_of_the_measured_shapes():
     # keys and values quantized to different lengths: tiles over what both have, slabs over the rest
     p = _lib.attn_plan(_step(16, 32, 32, 2, REF, 8064, 4, REF, 7968, 8192))
     assert p["matrix"] and p["slab_begin"] == 7968 and p["slabs"] == 1 and p["launches"] == 2
+    # the reference's 3-bit keys (733 words = 8063 tokens) with 2-bit values (8064): tiles of 1408 positions over
+    # [0, 7744) = 22 * 352, two slabs of 352 over the remaining quantized positions and the tails
+    p = _lib.attn_plan(_step(8, 32, 32, 3, REF, 8063, 2, REF, 8064, 8192))
+    assert p["matrix"] and (p["matrix_tiles"], p["slab_begin"], p["slab_positions"], p["slabs"]) == (6, 7744, 352, 2)
+    assert p["matrix_grid"][0] == 2 * 256 + 2 * 256 and p["launches"] == 2
     # configs[4]'s size: the vector-ALU slab kernel from position 0
     p = _lib.attn_plan(_step(4, 32, 32, 4, REF, 2176, 4, REF, 2176, 2304))
     assert not p["matrix"] and p["slab_begin"] == 0 and p["slabs"] == 5 and p["launches"] == 2
@@ -201,9 +206,13 @@ def test_no_attention_step_is_given_a_tile_longer_than_its_quantized_part():
                                 continue
                             assert rc == 0, (rc, k_bits, k_fmt, v_bits, batch, k_tokens, v_tokens, width)
                             if plan.matrix:
-                                both = min(k_tokens, v_tokens)
-                                assert both >= 1024 and both % 32 == 0 and unit == 32
-                                assert plan.slab_begin == both and plan.matrix_tiles == (both + 1023) // 1024
+                                # tiles of 1024 positions over what both sides have quantized; with the reference's
+                                # 3-bit keys tiles of 1408 over whole multiples of lcm(11, 32) = 352
+                                step, tile = (352, 1408) if unit == 11 else (32, 1024)
+                                both = min(k_tokens, v_tokens) // step * step
+                                assert both >= tile and (k_fmt, k_bits) != (DENSE3, 3)
+                                assert plan.slab_begin == both and plan.matrix_tiles == (both + tile - 1) // tile
+                                assert plan.slab_positions == (352 if unit == 11 else 256)
                                 blocks_per_head = (plan.matrix_grid[0] - plan.slab_blocks) // (batch * heads)
                                 assert blocks_per_head * plan.matrix_block[1] >= plan.matrix_tiles and plan.matrix_block[1] == 4
                                 assert plan.matrix_grid[0] == blocks_per_head * batch * heads + plan.slabs * batch * heads

@@ -286,3 +286,33 @@ def test_matrix_core_steps_with_keys_and_values_quantized_to_different_lengths(d
     vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
     logits = (q[sl, :2 * rep].double() @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
     check(out_s[sl, :2 * rep], torch.softmax(logits, -1) @ vals, vm)
+
+
+@pytest.mark.parametrize("v_bits,tk,tv", [(2, 8063, 8064), (3, 733 * 11 - 11 * 40, 8064), (4, 1408 + 352, 1408 + 352 + 32), (1, 3 * 1408, 3 * 1408)])
+def test_matrix_core_steps_with_the_reference_three_bit_keys(dev, v_bits, tk, tv):
+    """Keys in the reference's 3-bit words, the format its profiler assigns to most layers: tiles of 1408 positions
+    (128 words a row) over the whole multiples of 352 positions that keys and values both have quantized, a last
+    tile that is moved back, vector-ALU slabs over the rest.  Against the four-launch step and, for two rows, fp64
+    attention over the dequantized cache."""
+    from kvmix_amd import ops, _lib
+    from helpers import dequantize_torch
+
+    gen = torch.Generator(device=dev).manual_seed(500 + tk % 97 + v_bits)
+    rng = np.random.default_rng(tk + v_bits)
+    B, nkv, rep = 4, 32, 2
+    n = max(tk, tv) + 77
+    plan = _lib.attn_plan(_lib.attn_step_descriptor(B, nkv * rep, nkv, 128, 3, 0, 11, tk, v_bits, 1 if v_bits == 3 else 0, 32, tv,
+                                                   n - tk, n - tv))
+    assert plan["matrix"] and plan["launches"] == 2 and plan["slab_begin"] == min(tk, tv) // 352 * 352, plan
+    q, kq, vq, k_tail, v_tail, kg, mask, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, 3, v_bits, tk, tv, n, mask_rng=rng)
+    out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, 3, 32, v_bits, attention_mask=mask, **fmt)
+    out_s, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, 3, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
+    vm = v_magnitude(vq, v_tail, v_bits)
+    check(out_s, out_f, vm)
+    sl = slice(B - 1, B)
+    kd = dequantize_torch(kq[0][sl, :2], kq[1][sl, :2], kq[2][sl, :2], 3, 11).double()
+    vd = dequantize_torch(vq[0][sl, :2], vq[1][sl, :2], vq[2][sl, :2], v_bits, 32, dense3=v_bits == 3).double()
+    keys = torch.cat([kd.transpose(2, 3), k_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    logits = (q[sl, :2 * rep].double() @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
+    check(out_s[sl, :2 * rep], torch.softmax(logits, -1) @ vals, vm)
