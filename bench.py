@@ -233,11 +233,79 @@ def cpu_baseline(layers, kbits, vbits, B, H, D, T, R, sample_layers=None, budget
             O.quantized_gemm(32, p, vc, vs, vz, L.vb, mode=O.GEMM_SEQUENTIAL)
         total_t += time.perf_counter() - t0
         total_bytes += L.bytes_qk + L.bytes_pv + L.bytes_fk + L.bytes_fv
-    return {"value": round(total_bytes / total_t / 1e9, 3), "unit": "GB/s", "cores": int(O.num_threads()),
-            "kind": "port",
-            "sample": f"layers 0..{done - 1} of the step at full batch (one flush + q.K^T + p.V each, "
-                      f"{total_bytes / 1e9:.2f} GB algorithmic), {total_t:.1f} s of CPU time, "
-                      f"C oracle with OpenMP on {int(O.num_threads())} threads"}
+    res = {"value": round(total_bytes / total_t / 1e9, 3), "unit": "GB/s", "cores": int(O.num_threads()),
+           "kind": "port",
+           "sample": f"layers 0..{done - 1} of the step at full batch (one flush + q.K^T + p.V each, "
+                     f"{total_bytes / 1e9:.2f} GB algorithmic), {total_t:.1f} s of CPU time, "
+                     f"C oracle with OpenMP on {int(O.num_threads())} threads"}
+    try:
+        res["torch_cpu"] = torch_cpu_baseline(layers, int(O.num_threads()))
+    except Exception as ex:  # (the C port above is the figure of record; this leg must not take it down)
+        res["torch_cpu"] = {"error": f"{type(ex).__name__}: {ex}"}
+    return res
+
+
+def torch_cpu_baseline(layers, threads, batch_slice=2, reps=5, warm=2):
+    """The same work as vectorised PyTorch on the CPU: quantize = fp32 min / max / scale / round-half-away / pack
+    with tensor ops, GEMV = unpack with shifts and masks, dequantize to fp32, torch.matmul
+    (quant_cuda/csrc/quantization_cuda.cu:540-721, dequantization_gemv_cuda.cu:7-124 restated on tensors).  One layer
+    of each reference-layout bit width present in the step (2/2 and 4/4 bits), the first `batch_slice` batch entries
+    of it, `reps` repetitions after `warm` warm-ups, all host threads."""
+    import torch
+
+    torch.set_num_threads(threads)
+
+    def unpack(code, bits):
+        shifts = torch.arange(0, 32, bits, dtype=torch.int32)
+        return ((code.unsqueeze(-1) >> shifts) & ((1 << bits) - 1)).flatten(-2)
+
+    def dequant(code, scale, zero, bits, g=32):
+        return unpack(code, bits).float() * scale.float().repeat_interleave(g, -1) + zero.float().repeat_interleave(g, -1)
+
+    def quantize(x, bits, g=32):
+        qmax = (1 << bits) - 1
+        xf = x.float().unflatten(-1, (-1, g))
+        mn, mx = xf.amin(-1, keepdim=True), xf.amax(-1, keepdim=True)
+        scale = (mx - mn) / qmax
+        q = torch.nan_to_num(torch.floor((xf - mn) / scale + 0.5), nan=0.0).clamp_(0, qmax).to(torch.int32).flatten(-2)
+        shifts = torch.arange(0, 32, bits, dtype=torch.int32)
+        words = (q.unflatten(-1, (-1, 32 // bits)) << shifts).sum(-1, dtype=torch.int32)
+        return words, ((mx - mn) * (1.0 / qmax)).half().squeeze(-1), mn.half().squeeze(-1)
+
+    out = {}
+    total_bytes = total_t = 0.0
+    for L in layers:
+        if (L.kb, L.vb) not in ((2, 2), (4, 4)) or f"k{L.kb}v{L.vb}" in out:
+            continue
+        n = min(batch_slice, L.q.shape[0])
+        frac = n / L.q.shape[0]
+        kc, ks, kz = (t[:n].cpu() for t in (L.kc, L.ks, L.kz))
+        vc, vs, vz = (t[:n].cpu() for t in (L.vc, L.vs, L.vz))
+        q, p = L.q[:n].cpu().float(), L.p[:n].cpu().float()
+        ktail, vtail = L.ktail[:n].cpu().transpose(2, 3).contiguous(), L.vtail[:n].cpu()
+
+        def step():
+            quantize(ktail, L.kb)
+            quantize(vtail, L.vb)
+            a = torch.matmul(q, dequant(kc, ks, kz, L.kb)).half()
+            b = torch.matmul(p, dequant(vc, vs, vz, L.vb)).half()
+            return a, b
+
+        for _ in range(warm):
+            step()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            step()
+        dt = (time.perf_counter() - t0) / reps
+        nbytes = (L.bytes_qk + L.bytes_pv + L.bytes_fk + L.bytes_fv) * frac
+        out[f"k{L.kb}v{L.vb}"] = {"ms": round(dt * 1e3, 1), "GBps": round(nbytes / dt / 1e9, 3)}
+        total_bytes += nbytes
+        total_t += dt
+    out["value"] = round(total_bytes / total_t / 1e9, 3) if total_t else None
+    out["unit"], out["cores"] = "GB/s", threads
+    out["sample"] = (f"one 2/2-bit and one 4/4-bit layer of the step, first {batch_slice} of its batch entries (flush + q.K^T + p.V), "
+                     f"{reps} repetitions after {warm} warm-ups, torch {torch.__version__} on {threads} threads")
+    return out
 
 
 def mha_pair_times(torch, lib, dev, stream, B, Tq, bits, nsets=3, warm=30, iters=100, H=32, D=128):
@@ -884,6 +952,7 @@ def print_result(result, args, torch, _lib, lib, dev, layers, kbits, vbits, B, H
             result[key] = fn()
         except Exception as ex:
             result[key] = {"error": f"{type(ex).__name__}: {ex}"}
+            result.setdefault("extras_failed", []).append(key)  # (the headline stands; what broke is named on the line)
         torch.cuda.empty_cache()
 
     st = torch.cuda.current_stream().cuda_stream

@@ -157,14 +157,18 @@ class GraphDecoder(Decoder):
     fixed-size tail window through an indexed copy, and the attention step reads the tail lengths
     from the counters, so that the window's unused slots get probability zero.  A step in which some layer flushes runs eagerly (the flush changes the packed
     lengths, which are launch arguments), after which the graph is captured again.
-    Needs in-place caches (PackedKVCache) with a fixed residual window."""
+    Needs in-place caches (PackedKVCache) that all follow the same kind of flush policy: one fixed residual window,
+    or the reference's ratio rule (models/modeling_llama_KVmix.py:119-127,152-155: residual_length None) -- there the
+    tails stay short (a flush every group / (1 - ratio) tokens per layer, every 14 tokens with the reference's
+    3-bit keys), so a graph lives for fewer steps and the window is sized at every capture."""
 
     def __init__(self, cfg: DecoderConfig, weights: dict, attention: Sequence, caches: List):
         super().__init__(cfg, weights, attention, caches)
         windows = {c.residual_length for c in caches}
-        if None in windows or len(windows) != 1:
-            raise RuntimeError("GraphDecoder needs in-place caches that share one fixed residual window")
-        self.window = windows.pop()
+        if len(windows) != 1:
+            raise RuntimeError("GraphDecoder needs in-place caches that share one flush policy: one fixed residual "
+                               "window, or the ratio rule for all")
+        self.window = windows.pop()   # None: the ratio rule, the window is set at every capture
         self._graph = None
         self._stale = True
         self._warm = False
@@ -231,12 +235,29 @@ class GraphDecoder(Decoder):
             live.fill_(n + 1)
         self._len = [(self._counters[nk], self._counters[nv]) for nk, nv in lengths]
 
+    def _ratio_window(self) -> int:
+        """Slots the tail windows need until the next flush under the ratio rule: every tail grows one token a
+        step until the first length at which its rule flushes; that step runs eagerly, so the replayed steps
+        write slots below it.  (A multiple of 8, so that windows change less often between captures.)"""
+        from .cache import flush_length
+
+        need = 1
+        for c in self.caches:
+            for tail, ratio, group in ((c._k_tail, c.k_residual_ratio, c.Kgroup_size), (c._v_tail, c.v_residual_ratio, c.Vgroup_size)):
+                n = tail.len + 1
+                while flush_length(n, ratio, group) == 0:
+                    n += 1
+                need = max(need, n)
+        return (need + 7) // 8 * 8
+
     def _capture(self, ids: torch.Tensor) -> None:
         dev = ids.device
         if self._ids is None:
             self._ids = torch.zeros_like(ids)
             self._pos = torch.zeros(1, dtype=torch.int64, device=dev)
         self._ids.copy_(ids)
+        if self.caches[0].residual_length is None:
+            self.window = self._ratio_window()
         self._sync_counters()  # (also settles where the tail windows lie before anything is recorded)
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))

@@ -302,10 +302,53 @@ def test_graph_replayed_steps_match_eager_steps(dev):
     assert float((diff != 0).sum()) / diff.numel() < 0.2
 
 
-def test_graph_decoder_needs_a_fixed_window(dev):
+def test_graph_decoder_needs_one_flush_policy(dev):
     from kvmix_amd.decoder import DecoderConfig, GraphDecoder, kvmix_layers
 
-    cfg = DecoderConfig(hidden_size=256, num_layers=1, num_heads=2, num_kv_heads=2, intermediate_size=256, vocab_size=10)
-    atts, caches = kvmix_layers(cfg, [4], [4], residual_length=None)
-    with pytest.raises(RuntimeError, match="fixed residual window"):
-        GraphDecoder(cfg, {}, atts, caches)
+    cfg = DecoderConfig(hidden_size=256, num_layers=2, num_heads=2, num_kv_heads=2, intermediate_size=256, vocab_size=10)
+    atts, caches = kvmix_layers(cfg, [4, 4], [4, 4], residual_length=None)
+    _, fixed = kvmix_layers(cfg, [4, 4], [4, 4], residual_length=64)
+    with pytest.raises(RuntimeError, match="one flush policy"):
+        GraphDecoder(cfg, {}, atts, [caches[0], fixed[1]])
+
+
+def test_graph_replayed_steps_under_the_ratio_flush_rule(dev):
+    """The reference's own flush rule (keep int(ratio * L) tail tokens, quantize the rest in whole groups:
+    models/modeling_llama_KVmix.py:119-127,152-155) under graph replay: the tails stay short and flush every few
+    steps (every 14 tokens with the reference's 3-bit keys), every flushing step runs eagerly and the graph is
+    captured again with a window sized for the tails of that moment.  Against the eager decoder fed the same
+    tokens: every step's logits, and the caches -- the same quantized lengths everywhere, layer 0 bit for bit."""
+    from kvmix_amd.decoder import Decoder, DecoderConfig, GraphDecoder, init_weights, kvmix_layers
+
+    cfg = DecoderConfig(hidden_size=512, num_layers=4, num_heads=4, num_kv_heads=2, intermediate_size=1024, vocab_size=1000)
+    kbits, vbits = [4, 3, 2, 1], [2, 4, 3, 1]
+    B, T, new = 2, 150, 120
+    weights = init_weights(cfg, dev)
+    gen = torch.Generator(device="cpu").manual_seed(43)
+    prompt = torch.randint(0, cfg.vocab_size, (B, T), generator=gen).to(dev)
+
+    atts, caches = kvmix_layers(cfg, kbits, vbits, residual_length=None, capacity=T + new)
+    gd = GraphDecoder(cfg, weights, atts, caches)
+    seen = []
+    def keep(step, lg):
+        seen.append(lg.clone())
+        torch.cuda.synchronize()
+
+    tokens = gd.generate(prompt, new, keep)
+    assert gd.graph_steps + gd.eager_steps == new and gd.graph_steps > 0.5 * new and gd.captures >= 5, \
+        (gd.graph_steps, gd.eager_steps, gd.captures)
+
+    atts2, caches2 = kvmix_layers(cfg, kbits, vbits, residual_length=None, capacity=T + new)
+    ed = Decoder(cfg, weights, atts2, caches2)
+    ids = torch.cat([prompt, tokens], dim=1)
+    for step in range(new):
+        lg = ed.forward(ids[:, :T] if step == 0 else ids[:, T + step - 1:T + step])
+        assert float((lg - seen[step]).abs().max()) <= 0.01 * float(lg.std()), step
+    for li in range(cfg.num_layers):
+        a, b = caches[li].as_tuple(), caches2[li].as_tuple()
+        assert a[-1] == b[-1] == T + new - 1
+        assert (caches[li].k_tokens, caches[li].v_tokens) == (caches2[li].k_tokens, caches2[li].v_tokens)
+        for x, y in zip(a[:-1], b[:-1]):
+            assert x.shape == y.shape
+            if li == 0:
+                assert torch.equal(x, y)
