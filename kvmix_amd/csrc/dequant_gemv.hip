@@ -2759,6 +2759,9 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
         if (lean < want) want = lean;
     }
     if (want < 1) want = 1;
+#ifdef KVMIX_EXPERIMENT
+    if (const char *e = getenv("KVMIX_DBG_ROWS_WAVES")) want = atoll(e);
+#endif
     int64_t waves = want < max_waves ? want : max_waves;
     if (waves < 4) waves = 4;  // the block epilogue wants 128+ threads; idle waves are cheap
     int64_t splits = (want + waves - 1) / waves;

@@ -491,13 +491,18 @@ __device__ __forceinline__ void key_tokens_body(const KeyTokArgs &a, int64_t gi,
 // the reference 3-bit format 44 + 22 + 22 bytes instead of 33 separate stores from different blocks).
 // Units: (outer, chunk, channel half), channel half fastest.  Every thread of the block must call it
 // (block barriers).
-constexpr int kKeySlabChannels = 64;
+#ifndef KVMIX_KEY_SLAB_CHANNELS
+#define KVMIX_KEY_SLAB_CHANNELS 64
+#endif
+constexpr int kKeySlabChannels = KVMIX_KEY_SLAB_CHANNELS;
+constexpr int kKeySlabParts = 128 / kKeySlabChannels;       // channel parts of a head
+constexpr int kKeySlabThreadGroups = 256 / kKeySlabChannels; // groups of a chunk packed at a time
 template <int MODE>
 constexpr int key_slab_groups() { return MODE == 3 ? 11 : 4; }   // 121 or 128 tokens: a 16 KB tile
 static inline int64_t key_slab_units(int mode, int64_t outer, int64_t k_groups)
 {
     const int gc = mode == 3 ? key_slab_groups<3>() : key_slab_groups<4>();
-    return outer * ((k_groups + gc - 1) / gc) * (128 / kKeySlabChannels);
+    return outer * ((k_groups + gc - 1) / gc) * kKeySlabParts;
 }
 // what the slab path asks of the operand: D = 128, token rows that 128-bit loads can fetch
 static inline bool key_rows_tileable(const KeyTokArgs &a)
@@ -512,12 +517,12 @@ __device__ __forceinline__ void key_tokens_slab_body(const KeyTokArgs &a, int64_
 {
     constexpr int GC = key_slab_groups<MODE>(), CH = kKeySlabChannels, PPR = CH / 8;  // 16-byte pieces per tile row
     constexpr int WORDS = key_group_words<G, MODE>();
-    constexpr int JMAX = (GC + 3) / 4;  // groups per thread
+    constexpr int NGQ = kKeySlabThreadGroups, JMAX = (GC + NGQ - 1) / NGQ;  // groups per thread
     static_assert(GC * G * CH <= kKeySlabTile, "the tile of a chunk");
     const int tid = threadIdx.x;
     const uint32_t chunks = (uint32_t)((k_groups + GC - 1) / GC);
     const uint32_t u = (uint32_t)unit;  // (the host keeps the units below 2^31)
-    const uint32_t half = u % 2u, rest = u / 2u, chunk = rest % chunks;
+    const uint32_t half = u % (uint32_t)kKeySlabParts, rest = u / (uint32_t)kKeySlabParts, chunk = rest % chunks;
     const int64_t o = rest / chunks;
     const int g0 = (int)chunk * GC;
     const int ng = (int)(k_groups - g0 < GC ? k_groups - g0 : GC);
@@ -542,7 +547,7 @@ __device__ __forceinline__ void key_tokens_slab_body(const KeyTokArgs &a, int64_
     __half sc[JMAX], zr[JMAX];
 #pragma unroll
     for (int j = 0; j < JMAX; j++) {
-        const int g = gq + 4 * j;
+        const int g = gq + NGQ * j;
         if (g < ng) {
             float v[G];
 #pragma unroll
@@ -556,7 +561,7 @@ __device__ __forceinline__ void key_tokens_slab_body(const KeyTokArgs &a, int64_
     __half *os = reinterpret_cast<__half *>(tile + 2 * CH * ((GC * WORDS) | 1)), *oz = os + CH * (GC | 1);
 #pragma unroll
     for (int j = 0; j < JMAX; j++) {
-        const int g = gq + 4 * j;
+        const int g = gq + NGQ * j;
         if (g < ng) {
 #pragma unroll
             for (int t = 0; t < WORDS; t++) ow[dl * wp + g * WORDS + t] = w[j][t];
