@@ -1312,9 +1312,10 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
             uint32_t v[4], u[4];
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                // words (0,0,1,2) and (0,1,2,2) of the group for lanes 0..3, funnel-shifted
+                // words (0,0,1,2) and (0,1,2,2) of the group for lanes 0..3, funnel-shifted; the second set is what the
+                // lanes loaded (lane j holds word min(j, 2)), only the first has to come from the neighbours
                 const uint32_t lo = __builtin_amdgcn_mov_dpp(w[d][t][k], 0x90, 0xf, 0xf, false);
-                const uint32_t hi = __builtin_amdgcn_mov_dpp(w[d][t][k], 0xA4, 0xf, 0xf, false);
+                const uint32_t hi = w[d][t][k];
                 v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
                 u[k] = v[k] >> 4;
             }
@@ -2087,7 +2088,7 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 const uint32_t lo = __builtin_amdgcn_mov_dpp(w[t][k], 0x90, 0xf, 0xf, false);
-                const uint32_t hi = __builtin_amdgcn_mov_dpp(w[t][k], 0xA4, 0xf, 0xf, false);
+                const uint32_t hi = w[t][k];  // (lane j holds word min(j, 2) of its group: the set (0,1,2,2))
                 v[k] = __builtin_amdgcn_alignbit(hi, lo, sh3);
                 u[k] = v[k] >> 4;
             }
