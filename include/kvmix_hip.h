@@ -298,10 +298,12 @@ int kvmix_decode_attention(const kvmix_decode_attn_t *step, void *workspace, siz
  * logits, 1/sqrt(D), mask, clamp) but not the reference's roundings after it: probabilities are not
  * rounded to fp16 and the quantized and tail halves of the output are not rounded separately, so the
  * result differs from kvmix_decode_attention's by up to about 2^-10 of the largest value magnitude.
- * Large steps (at least 512 (query head, 1024-position tile) pairs) whose keys (1, 2 or 4 bits) and values are
- * quantized to the same length of at least 1024 positions, with dense value rows, run those positions on the
- * matrix cores -- one wave per tile: logits, slab softmax and the product with the values of the same positions --
- * and only the fp16 tails through the vector-ALU slab kernel (three launches); everything else as described above.
+ * Steps whose keys (1, 2 or 4 bits, or the reference's 3-bit words) and values are both quantized over at least
+ * one tile of 1024 positions (1408 with those words), with dense value rows, run the positions quantized on both
+ * sides on the matrix cores -- a wave per tile, or the four waves of a block per tile when the step has few tiles:
+ * logits, slab softmax and the product with the values of the same positions -- and the rest (the fp16 tails, and
+ * positions only one side has quantized) as trailing blocks of the same launch (two launches); everything else as
+ * described above.  kvmix_decode_attention_fused_plan tells which.
  *
  * Supported (kvmix_decode_attention_fused_supported returns 1, else the call returns
  * KVMIX_ERR_UNSUPPORTED): D = 128; keys 1/2/4-bit or dense 3-bit in groups of 32 or the reference's 3-bit words;
@@ -328,6 +330,8 @@ typedef struct kvmix_attn_plan {
     int launches;            /* kernel launches of the step, the merge included */
     int64_t matrix_tiles;    /* tiles of 1024 positions (1408 with the reference's 3-bit keys) per query head; 0
                               * without the matrix-core kernel */
+    int matrix_tile_waves;   /* waves that share a tile: 1, or 4 for steps with few (query head, tile) pairs (each wave
+                              * then finishes a quarter of the tile as a slab of its own); 0 without the kernel */
     int64_t slab_positions;  /* positions per vector-ALU slab */
     int64_t slab_begin;      /* first position those slabs cover */
     int64_t slabs;           /* their number per query head */

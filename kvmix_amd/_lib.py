@@ -102,7 +102,7 @@ class GemvPlan(ctypes.Structure):
 class AttnPlan(ctypes.Structure):
     """kvmix_attn_plan_t"""
     _fields_ = [("matrix", ctypes.c_int), ("recommended", ctypes.c_int), ("launches", ctypes.c_int), ("matrix_tiles", ctypes.c_int64),
-                ("slab_positions", ctypes.c_int64), ("slab_begin", ctypes.c_int64), ("slabs", ctypes.c_int64),
+                ("matrix_tile_waves", ctypes.c_int), ("slab_positions", ctypes.c_int64), ("slab_begin", ctypes.c_int64), ("slabs", ctypes.c_int64),
                 ("slab_blocks", ctypes.c_int64), ("matrix_grid", ctypes.c_uint * 3), ("matrix_block", ctypes.c_uint * 3)]
 
 
@@ -211,6 +211,7 @@ def attn_plan(step: DecodeAttn) -> dict:
     plan = AttnPlan()
     check(load().kvmix_decode_attention_fused_plan(ctypes.byref(step), ctypes.byref(plan)))
     return {"matrix": bool(plan.matrix), "recommended": bool(plan.recommended), "launches": plan.launches, "matrix_tiles": plan.matrix_tiles,
+            "matrix_tile_waves": plan.matrix_tile_waves,
             "slab_positions": plan.slab_positions, "slab_begin": plan.slab_begin, "slabs": plan.slabs,
             "slab_blocks": plan.slab_blocks, "matrix_grid": tuple(plan.matrix_grid),
             "matrix_block": tuple(plan.matrix_block)}

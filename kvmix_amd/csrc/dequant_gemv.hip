@@ -2197,7 +2197,7 @@ constexpr int kSlabKeyBytes = (kColsMfma2Tile * 2 + 32 * 4 + 15) / 16 * 16;  // 
 constexpr int kSlabLds = kSlabKeyBytes + 1024 * 4;                            // ... + the slab's probabilities
 static_assert(kRowsMfmaTile * 2 <= kSlabKeyBytes, "the value phase's A tile reuses the key phase's space");
 
-template <int KBITS, int VMODE>
+template <int KBITS, int VMODE, bool COOP>
 __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64_t bx, int64_t sample, float *lds)
 {
     static_assert(KBITS == 4 || KBITS == 2 || KBITS == 1, "key codes of 1, 2 or 4 bits");
@@ -2213,9 +2213,9 @@ __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64
     float *pbuf = reinterpret_cast<float *>(mine + kSlabKeyBytes);  // [1024] probabilities of the slab
     const int64_t kv = sample / a.heads_per_kv;
     const int ngroups = (int)(a.tokens / 32);
-    const int tile = (int)bx * nw + wy;
+    const int tile = COOP ? (int)bx : (int)bx * nw + wy;
     if (ngroups < TG) return;  // (never launched so: a slab longer than the row would leave the operands)
-    if (tile * TG >= ngroups) return;
+    if (tile * TG >= ngroups) return;  // (COOP: the whole block)
     const int g_first = tile * TG + TG <= ngroups ? tile * TG : max(ngroups - TG, 0);  // (the last tile ends at `tokens`)
     const int shift = tile * TG - g_first;                                     // its first groups are the neighbour's
     float slab_m, slab_l;
@@ -2328,19 +2328,21 @@ __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64
         };
 
         constexpr int items = K / CH;
-        load_small(0);
+        // COOP: the block's four waves share the tile, each with a quarter of the 128 channel rows
+        const int it0 = COOP ? wy * (items / kColsWaves) : 0, it1 = COOP ? it0 + items / kColsWaves : items;
+        load_small(it0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < KB; t++) {
-            load_codes(0, t);
+            load_codes(it0, t);
             __builtin_amdgcn_sched_barrier(0);
         }
         for (int i = lane; i < AT / 2; i += kWave) reinterpret_cast<uint32_t *>(atile)[i] = 0u;
         wave_lds_fence();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll 1
-        for (int it = 0; it < items; it++) {
-            const int nx = it + 1 < items ? it + 1 : it;
+        for (int it = it0; it < it1; it++) {
+            const int nx = it + 1 < it1 ? it + 1 : it;
             stage();
             wave_lds_fence();
             load_small(nx);
@@ -2366,6 +2368,61 @@ __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64
         wave_lds_fence();
         const int q = lane / 4;
         const float *mrow = a.mask ? a.mask + (sample / a.heads) * a.mask_bs : nullptr;
+        if constexpr (COOP) {
+            // every wave has the sums of its rows for all 1024 positions: they meet in LDS (the waves' pbuf areas,
+            // in position order), then wave w finishes positions [256 w, 256 w + 256) as a slab of its own
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                const int elem = SPLIT ? 64 * s + lane
+                                       : 8 * q + (s == 0 ? ((j4 & 1) * 2 + (j4 >> 1)) : (4 + (j4 & 1) * 2 + (1 - (j4 >> 1))));
+                float sums[NPOS], part[NPOS];
+#pragma unroll
+                for (int p = 0; p < NPOS; p++) sums[p] = (acc[s][p][0] + acc[s][p][1]) + acc[s][p][2];
+#pragma unroll
+                for (int p = 0; p < NPOS; p++) {
+                    const float v = field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+                    part[p] = v * __uint_as_float((uint32_t)(127 + 43 - BITS * (p % FPB)) << 23);
+                }
+                *reinterpret_cast<float4 *>(pbuf + elem * 8) = float4{part[0], part[1], part[2], part[3]};
+                *reinterpret_cast<float4 *>(pbuf + elem * 8 + 4) = float4{part[4], part[5], part[6], part[7]};
+            }
+            __syncthreads();
+            const uint8_t *base = reinterpret_cast<const uint8_t *>(lds);
+            const int pos0 = 256 * wy + 4 * lane, grp = pos0 / 32;
+            float4 d = float4{0.f, 0.f, 0.f, 0.f};
+            float zt = 0.f;
+#pragma unroll
+            for (int w = 0; w < kColsWaves; w++) {
+                const float4 v = *reinterpret_cast<const float4 *>(base + w * kSlabLds + kSlabKeyBytes + 4 * pos0);
+                d.x += v.x, d.y += v.y, d.z += v.z, d.w += v.w;
+                zt += reinterpret_cast<const float *>(base + w * kSlabLds + AT * 2)[grp];
+            }
+            __syncthreads();  // (the waves' areas are read; from here on pbuf is the wave's own 256 probabilities)
+            const float dots[4] = {d.x + zt, d.y + zt, d.z + zt, d.w + zt};
+            float xs[4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float lg = h16_to_f32(f32_to_h16(dots[j])) * a.inv_sqrt_d;
+                if (mrow) lg = fmaxf(lg + mrow[(int64_t)g_first * 32 + pos0 + j], -3.4028234663852886e38f);
+                xs[j] = grp >= shift ? lg : -INFINITY;
+                mx = fmaxf(mx, xs[j]);
+            }
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float sum = 0.f, e[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                e[j] = xs[j] == -INFINITY ? 0.f : expf(xs[j] - mx);
+                sum += e[j];
+            }
+            *reinterpret_cast<float4 *>(pbuf + 4 * lane) = float4{e[0], e[1], e[2], e[3]};
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+            wave_lds_fence();
+            slab_value_phase<VMODE, 2>(a, kv, sample, tile * kColsWaves + wy, g_first * 32 + 256 * wy, atile, pbuf, mx, sum);
+            return;
+        }
         float x[2][NPOS];
         float mx = -INFINITY;
 #pragma unroll
@@ -2427,7 +2484,7 @@ constexpr int kSlabRef3Tile = kSlabRef3Words * 11;        // positions per tile
 constexpr int kSlabRef3ABytes = (kRowsMfmaTile * 2 + 15) / 16 * 16;
 constexpr int kSlabRef3Lds = 128 * 4 + kSlabRef3ABytes + kSlabRef3Tile * 4;   // query, A tile of the value phase, probabilities
 
-template <int VMODE>
+template <int VMODE, bool COOP>
 __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64_t bx, int64_t sample, float *lds)
 {
     constexpr int K = 128, U = 8, UPL = 2, VALS = 11, TW = kSlabRef3Words;
@@ -2440,9 +2497,9 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
     float *pbuf = reinterpret_cast<float *>(mine + K * 4 + kSlabRef3ABytes);      // [1408] probabilities of the slab
     const int64_t kv = sample / a.heads_per_kv;
     const int nwords = (int)(a.tokens / VALS);
-    const int tile = (int)bx * nw + wy;
+    const int tile = COOP ? (int)bx : (int)bx * nw + wy;
     if (nwords < TW) return;  // (never launched so: a slab longer than the row would leave the operands)
-    if (tile * TW >= nwords) return;
+    if (tile * TW >= nwords) return;  // (COOP: the whole block)
     const int w_first = tile * TW + TW <= nwords ? tile * TW : max(nwords - TW, 0);  // (the last tile ends at `tokens`)
     const int shift = tile * TW - w_first;                                             // its first words are the neighbour's
     float slab_m, slab_l;
@@ -2468,8 +2525,11 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
         const uint8_t *sb = reinterpret_cast<const uint8_t *>(a.k_scale + kv * a.ksz_bs);
         const uint8_t *zb = reinterpret_cast<const uint8_t *>(a.k_zero + kv * a.ksz_bs);
         const uint32_t unit0 = (uint32_t)(w_first + lane * UPL);
-        uint32_t co = unit0 * 4u, so = unit0 * 2u;
         const uint32_t c_step = (uint32_t)a.kc_rs * 4u, s_step = (uint32_t)a.ksz_rs * 2u;
+        // COOP: the block's four waves share the tile, each with a quarter of the 128 channel rows
+        constexpr int steps = COOP ? K / U / kColsWaves : K / U;
+        const int row0 = COOP ? wy * (K / kColsWaves) : 0;
+        uint32_t co = unit0 * 4u + (uint32_t)row0 * c_step, so = unit0 * 2u + (uint32_t)row0 * s_step;
         auto next_row = [&](int u) {
             cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cb + co);
             sw[u] = ld_stream<Half2x, KVMIX_COLS3_NT_SZ>(sb + so);
@@ -2497,7 +2557,6 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
                 for (int i = 0; i < VALS; i++) acc[j][i] = fmaf(mq, f[i], acc[j][i]);
             }
         };
-        constexpr int steps = K / U;
 #pragma unroll
         for (int u = 0; u < U; u++) {
             next_row(u);
@@ -2506,7 +2565,7 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
 #pragma unroll 1
         for (int st = 0; st < steps - 1; st++) {
 #pragma unroll
-            for (int u = 0; u < U; u++) xr[u] = xs[st * U + u];
+            for (int u = 0; u < U; u++) xr[u] = xs[row0 + st * U + u];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -2516,13 +2575,57 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
             }
         }
 #pragma unroll
-        for (int u = 0; u < U; u++) xr[u] = xs[(steps - 1) * U + u];
+        for (int u = 0; u < U; u++) xr[u] = xs[row0 + (steps - 1) * U + u];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; u++) compute_row(u);
 
         // the logits of this lane's 22 positions: fp16 rounding, 1/sqrt(D), mask as in the reference
         const float *mrow = a.mask ? a.mask + (sample / a.heads) * a.mask_bs + (int64_t)w_first * VALS : nullptr;
+        if constexpr (COOP) {
+            // the waves' sums over their rows meet in LDS (the waves' pbuf areas, in position order); then wave w
+            // finishes three of the tile's eleven 128-position chunks as a slab of its own: chunks 3 w .. 3 w + 2,
+            // the last wave chunks 8 .. 10 with chunk 8 (wave 2's) at probability 0
+#pragma unroll
+            for (int j = 0; j < UPL; j++) {
+#pragma unroll
+                for (int i = 0; i < VALS; i++)
+                    pbuf[(lane * UPL + j) * VALS + i] = fmaf(acc[j][i], cols3_out_scale(i), zsum[j] * kCols3ZeroDown);
+            }
+            __syncthreads();
+            constexpr int CHW = 3, SPAN = CHW * 128, PER = SPAN / kWave;  // positions per wave, per lane
+            const int begin = wy < kColsWaves - 1 ? SPAN * wy : kSlabRef3Tile - SPAN;  // first position of the wave's chunks
+            const int own = SPAN * wy;                                                  // ... of the positions it owns
+            const uint8_t *base = reinterpret_cast<const uint8_t *>(lds) + K * 4 + kSlabRef3ABytes;
+            float xv[PER];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < PER; r++) {
+                const int pos = begin + r * kWave + lane;
+                float dot = 0.f;
+#pragma unroll
+                for (int w = 0; w < kColsWaves; w++) dot += reinterpret_cast<const float *>(base + w * kSlabRef3Lds)[pos];
+                float lg = h16_to_f32(f32_to_h16(dot)) * a.inv_sqrt_d;
+                if (mrow) lg = fmaxf(lg + mrow[pos], -3.4028234663852886e38f);
+                xv[r] = pos >= own && pos / VALS >= shift ? lg : -INFINITY;
+                mx = fmaxf(mx, xv[r]);
+            }
+            __syncthreads();  // (the waves' areas are read; from here on pbuf is the wave's own 384 probabilities)
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float sum = 0.f;
+#pragma unroll
+            for (int r = 0; r < PER; r++) {
+                const float e = xv[r] == -INFINITY ? 0.f : expf(xv[r] - mx);
+                sum += e;
+                pbuf[r * kWave + lane] = e;
+            }
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+            wave_lds_fence();
+            slab_value_phase<VMODE, CHW>(a, kv, sample, tile * kColsWaves + wy, w_first * VALS + begin, atile, pbuf, mx, sum);
+            return;
+        }
         float x[UPL][VALS];
         float mx = -INFINITY;
 #pragma unroll
@@ -2569,7 +2672,7 @@ constexpr size_t step_lds(int k_mode)
     const size_t slab = fused::SlabCfg<8>::lds_floats(1) * sizeof(float);
     return tiles > slab ? tiles : slab;
 }
-template <int KBITS, int VMODE>
+template <int KBITS, int VMODE, bool COOP>
 __global__ void __launch_bounds__(64 * kColsWaves) __attribute__((amdgpu_waves_per_eu(kMfma2Occ)))
 attn_step_mfma(AttnSlabArgs m, fused::FusedArgs f, unsigned mfma_blocks, unsigned mfma_nx)
 {
@@ -2581,9 +2684,9 @@ attn_step_mfma(AttnSlabArgs m, fused::FusedArgs f, unsigned mfma_blocks, unsigne
         const int64_t xcd = l % kXcds, slot = l / kXcds, per = n / kXcds, rem = n % kXcds;
         const int64_t j = xcd * per + (xcd < rem ? xcd : rem) + slot;
         if constexpr (KBITS == 3)
-            attn_slab_ref3_body<VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
+            attn_slab_ref3_body<VMODE, COOP>(m, j % mfma_nx, j / mfma_nx, lds);
         else
-            attn_slab_mfma_body<KBITS, VMODE>(m, j % mfma_nx, j / mfma_nx, lds);
+            attn_slab_mfma_body<KBITS, VMODE, COOP>(m, j % mfma_nx, j / mfma_nx, lds);
     } else {
         fused::attn_fused_slab_body<1, 8>(f, (int64_t)blockIdx.x - mfma_blocks, (int64_t)gridDim.x - mfma_blocks,
                                           (int)(threadIdx.y * kWave + threadIdx.x), lds);
@@ -3001,28 +3104,34 @@ static void launch_cols_mfma2(GemvArgs &a, int64_t samples, hipStream_t st)
     }
 }
 
-int plan_attn_slab_mfma(int k_mode, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3])
+int plan_attn_slab_mfma(int k_mode, bool coop, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3],
+                        unsigned block[3])
 {
     const int64_t tile = k_mode == 3 ? kSlabRef3Tile : 1024, unit = k_mode == 3 ? 352 : 32;
     const int64_t tiles = (tokens + tile - 1) / tile;
     if (tokens < tile || tokens % unit != 0 || samples <= 0 || tail_blocks < 0) return KVMIX_ERR_SHAPE;
-    const int64_t nx = (tiles + kColsWaves - 1) / kColsWaves;  // blocks of four tiles per query head
+    // blocks per query head: of four tiles, or (coop) one tile shared by the block's four waves
+    const int64_t nx = coop ? tiles : (tiles + kColsWaves - 1) / kColsWaves;
     if (nx * samples + tail_blocks > 0x7fffffff) return KVMIX_ERR_SHAPE;
     grid[0] = (unsigned)(nx * samples + tail_blocks), grid[1] = 1, grid[2] = 1;
     block[0] = kWave, block[1] = kColsWaves, block[2] = 1;
     return KVMIX_OK;
 }
 
-int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, int v_mode, int64_t samples,
+int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, bool coop, int v_mode, int64_t samples,
                           int64_t tail_blocks, hipStream_t stream)
 {
     unsigned g[3], b[3];
-    const int prc = plan_attn_slab_mfma(k_bits, a.tokens, samples, tail_blocks, g, b);
+    const int prc = plan_attn_slab_mfma(k_bits, coop, a.tokens, samples, tail_blocks, g, b);
     if (prc != KVMIX_OK) return prc;
     const dim3 grid(g[0]), block(b[0], b[1]);
     const unsigned mfma_blocks = (unsigned)(g[0] - tail_blocks), mfma_nx = (unsigned)(mfma_blocks / samples);
     const size_t lds = step_lds(k_bits);
-#define KVMIX_SLAB(KB_, VM_) hipLaunchKernelGGL((attn_step_mfma<KB_, VM_>), grid, block, lds, stream, a, f, mfma_blocks, mfma_nx)
+#define KVMIX_SLAB(KB_, VM_)                                                                                   \
+    if (coop)                                                                                                  \
+        hipLaunchKernelGGL((attn_step_mfma<KB_, VM_, true>), grid, block, lds, stream, a, f, mfma_blocks, mfma_nx); \
+    else                                                                                                       \
+        hipLaunchKernelGGL((attn_step_mfma<KB_, VM_, false>), grid, block, lds, stream, a, f, mfma_blocks, mfma_nx)
 #define KVMIX_SLAB_V(KB_)                          \
     switch (v_mode) {                              \
     case 1: KVMIX_SLAB(KB_, 1); break;             \

@@ -20,6 +20,8 @@
 // slab through L2).
 #include "fused_slab.h"
 
+#include <cstdlib>
+
 namespace kvmix {
 
 using namespace fused;
@@ -115,17 +117,20 @@ static int64_t fused_slabs(const kvmix_decode_attn_t *p)
     return (fused_width(p) + s - 1) / s;
 }
 
-// How a row's positions are divided into slabs.  Large steps with keys of 1, 2 or 4 bits or in the reference's 3-bit
-// words take the positions that are quantized on both sides, [0, min(k_tokens, v_tokens)), through the matrix-core
-// tiles (attn_slab_mfma_body: 1024 positions per wave, the formats of gemv_cols_mfma2 and gemv_rows_mfma;
-// attn_slab_ref3_body: 1408 positions, gemv_cols3's arithmetic for the keys) and the rest -- the fp16 tails, and the few
-// positions quantized on one side only when keys and values are quantized to different lengths -- through slabs of
-// the vector-ALU kind that run as trailing blocks of the same launch (256 threads, 256 positions each); everything
-// else goes through attn_fused_slab (512 threads) from position 0.
+// How a row's positions are divided into slabs.  Keys of 1, 2 or 4 bits or in the reference's 3-bit words, with
+// at least one tile quantized on both sides, take the positions [0, min(k_tokens, v_tokens)) through the matrix-core
+// tiles (attn_slab_mfma_body: 1024 positions, the formats of gemv_cols_mfma2 and gemv_rows_mfma; attn_slab_ref3_body:
+// 1408 positions, gemv_cols3's arithmetic for the keys) -- one wave per tile, or, for steps with few (query head,
+// tile) pairs, the four waves of a block per tile -- and the rest -- the fp16 tails, and the few positions quantized
+// on one side only when keys and values are quantized to different lengths -- through slabs of the vector-ALU kind
+// that run as trailing blocks of the same launch (256 threads, 256 positions each); everything else goes through
+// attn_fused_slab (512 threads) from position 0.
 constexpr int64_t kSmallStepEntries = 1 << 19, kSmallStepEntriesRef3 = 360000;  // (see kvmix_decode_attention_fused_plan)
-constexpr int64_t kSlabMfmaMinWaves = 512;  // (measured: 512 waves 34 against 38 us, 256 waves 33 against 25 us)
+constexpr int64_t kSlabMfmaMinWaves = 512;   // one wave per tile from this many (query head, tile) pairs on
+constexpr int64_t kSlabRef3MaxPairs = 768;   // the reference's 3-bit keys: the single pass is ahead up to here
 struct FusedLayout {
     bool mfma;
+    bool coop;           // four waves per tile (attn_step_mfma<.., true>): four workspace slabs per tile
     int64_t tiles;       // slabs of the matrix-core kernel (first in the workspace)
     int64_t tail_slabs;  // vector-ALU slabs, from position t_begin on
     int64_t t_begin;
@@ -133,9 +138,29 @@ struct FusedLayout {
     int64_t slabs() const { return tiles + tail_slabs; }
 };
 
+// With fewer (query head, tile) pairs than this, four waves share a tile (attn_step_mfma<.., true>).  Measured,
+// one wave per tile -> four (us, Llama-2-7B heads): 4-bit keys 4 x 2304: 30.3 -> 20.1, 1 x 4096: 18.5 -> 13.8 (those two
+// against the vector-ALU slabs, which took these sizes before), 4 x 4224 (512 pairs): 26.1 -> 29.7, 8 x 2304 (768):
+// 27.7 -> 34.1; reference 3-bit keys 8 x 2304 (512 pairs): 34.6 -> 31.3, 8 x 4224 (768): 38.3 -> 46.6.  With the
+// reference's 3-bit keys and fewer than 128 pairs the vector-ALU slabs stay ahead (2 x 1664: 21.2 against 23.1).
+static int64_t coop_below(int km)
+{
+#ifdef KVMIX_EXPERIMENT
+    if (const char *e = getenv("KVMIX_DBG_COOP_BELOW")) return atoll(e);
+#endif
+    return km == 3 ? kSlabRef3MaxPairs : kSlabMfmaMinWaves;
+}
+static bool coop_ok(int km, int64_t pairs)
+{
+#ifdef KVMIX_EXPERIMENT
+    if (const char *e = getenv("KVMIX_DBG_COOP")) return atoi(e) != 0;
+#endif
+    return km == 3 ? pairs >= 128 : true;
+}
+
 static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
 {
-    FusedLayout l{false, 0, fused_slabs(p), 0, fused_slab(p)};
+    FusedLayout l{false, false, 0, fused_slabs(p), 0, fused_slab(p)};
     const int km = fused_key_mode(p), vm = fused_value_mode(p);
     const int vbits = vm == 3 ? 3 : vm;
     // positions quantized on both sides, in whole words of the keys and whole groups of the values; tiles of 1024
@@ -148,9 +173,10 @@ static FusedLayout fused_layout(const kvmix_decode_attn_t *p)
         (kFusedD + 1) * p->k_code_row_stride < (1ll << 29) && (kFusedD + 1) * p->k_sz_row_stride < (1ll << 30) &&
         // (the value phase forms 32-bit byte offsets of code rows and 32-bit element offsets of scale rows)
         p->v_tokens * p->v_code_row_stride < (1ll << 30) && p->v_tokens * p->v_sz_row_stride < (1ll << 31) &&
-        p->samples * tiles >= kSlabMfmaMinWaves) {
+        (p->samples * tiles >= coop_below(km) || coop_ok(km, p->samples * tiles))) {
         l.mfma = true;
-        l.tiles = tiles;
+        l.coop = p->samples * tiles < coop_below(km);
+        l.tiles = l.coop ? 4 * tiles : tiles;
         l.t_begin = both;
         l.slab = km == 3 ? SlabCfg<8>::kSlabRef3 : SlabCfg<8>::kSlabG32;
         l.tail_slabs = (fused_width(p) - both + l.slab - 1) / l.slab;
@@ -222,24 +248,34 @@ extern "C" int kvmix_decode_attention_fused_plan(const kvmix_decode_attn_t *p, k
     if (rc != KVMIX_OK || p->samples == 0) return rc;
     const FusedLayout lay = fused_layout(p);
     plan->matrix = lay.mfma ? 1 : 0;
-    // Which form is faster (MI355X, Llama-2-7B heads, graph-replayed; four launches -> single pass, us): the
-    // vector-ALU slabs up to about 2^19 (query head x position) entries -- 1 x 4096: 29 -> 19, 4 x 2304: 31 -> 27..30 --
-    // earlier with the reference's 3-bit keys; beyond that only on the matrix cores, with keys of 1, 2 or 4 bits
-    // (8 x 8192: 4/4 bits 71 -> 61, 2/2 bits 54 -> 45, 2/4 bits 63 -> 52; 16 x 8192: 129 -> 116, 90 -> 80, 110 -> 98).
-    // The reference's 3-bit keys on the matrix-core tiles are correct but behind there (8 x 8192, 2-bit values:
-    // 69 -> 72, 16 x 8192: 124 -> 140): the key phase of a tile is one wave's vector arithmetic over all 128 rows.
+    // Which form is faster (MI355X, Llama-2-7B heads, graph-replayed; four launches -> single pass, us).  Keys of 1,
+    // 2 or 4 bits: the single pass wherever the matrix-core tiles take it (1 x 4096: 29 -> 14, 4 x 2304 4/4 bits: 32 ->
+    // 20, 2/2 bits: 30 -> 18; 8 x 8192: 4/4 bits 71 -> 61, 2/2 bits 54 -> 45, 2/4 bits 63 -> 52; 16 x 8192: 129 -> 116,
+    // 90 -> 80, 110 -> 98), else (rows under 1024 quantized positions) the vector-ALU slabs up to about 2^19 (query head
+    // x position) entries.  The reference's 3-bit keys: on the tiles up to 768 (query head, tile) pairs (4 x 4224: 37 ->
+    // 27, 8 x 4224: 47 -> 38, 4 x 8192: 49 -> 40); behind beyond (8 x 8192: 69 -> 72, 16 x 8192: 124 -> 140: the key phase
+    // of a tile is vector arithmetic over all 128 rows in a block that also holds the value phase's registers);
+    // without tiles the vector-ALU slabs up to 360 000 entries.
     {
         const int64_t entries = p->samples * fused_width(p);
         const bool ref3 = p->k_tokens > 0 && fused_key_mode(p) == 3;
-        plan->recommended = entries <= (ref3 ? kSmallStepEntriesRef3 : kSmallStepEntries) ? 1 : (lay.mfma && !ref3 ? 1 : 0);
+        const int64_t pairs = p->samples * (lay.coop ? lay.tiles / 4 : lay.tiles);
+        // (the positions past the tiles run as vector-ALU slabs: no more of them than those do well on their own)
+        const int64_t rest = p->samples * (fused_width(p) - lay.t_begin);
+        if (lay.mfma)
+            plan->recommended = (!ref3 || pairs <= kSlabRef3MaxPairs) && rest <= kSmallStepEntries ? 1 : 0;
+        else
+            plan->recommended = entries <= (ref3 ? kSmallStepEntriesRef3 : kSmallStepEntries) ? 1 : 0;
     }
-    plan->matrix_tiles = lay.tiles;
+    plan->matrix_tile_waves = lay.mfma ? (lay.coop ? 4 : 1) : 0;
+    plan->matrix_tiles = lay.coop ? lay.tiles / 4 : lay.tiles;
     plan->slab_positions = lay.slab;
     plan->slab_begin = lay.t_begin;
     plan->slabs = lay.tail_slabs;
     if (lay.mfma) {
         // one launch: the tiles' blocks, then the slabs' blocks
-        const int prc = plan_attn_slab_mfma(fused_key_mode(p), lay.t_begin, p->samples, lay.tail_slabs * p->samples, plan->matrix_grid, plan->matrix_block);
+        const int prc = plan_attn_slab_mfma(fused_key_mode(p), lay.coop, lay.t_begin, p->samples, lay.tail_slabs * p->samples,
+                                            plan->matrix_grid, plan->matrix_block);
         if (prc != KVMIX_OK) return prc;
         plan->slab_blocks = lay.tail_slabs * p->samples;
         plan->launches++;
@@ -328,7 +364,7 @@ extern "C" int kvmix_decode_attention_fused(const kvmix_decode_attn_t *p, void *
         m.heads_per_kv = p->heads_per_kv, m.heads = p->heads;
         m.slabs = (int)slabs;
         m.inv_sqrt_d = a.inv_sqrt_d;
-        rc = launch_attn_step_mfma(m, a, k_mode, v_mode == 3 ? 30 : v_mode, p->samples, lay.tail_slabs * p->samples, st);
+        rc = launch_attn_step_mfma(m, a, k_mode, lay.coop, v_mode == 3 ? 30 : v_mode, p->samples, lay.tail_slabs * p->samples, st);
     } else if (lay.tail_slabs > 0) {
         const dim3 grid((unsigned)(lay.tail_slabs * kv_samples * p->heads_per_kv));
         hipLaunchKernelGGL(attn_fused_slab<1>, grid, dim3(kFusedThreads), 0, st, a);

@@ -504,10 +504,14 @@ __device__ __forceinline__ void attn_fused_slab_body(const FusedArgs &a, int64_t
 // f.t_begin = a.tokens, f.slab0 = the number of tiles) over the rest.  k_bits in {1, 2, 4} (tiles of 1024 positions,
 // a.tokens a multiple of 32) or 3 = the reference's 3-bit words (tiles of 1408, a.tokens a multiple of 352); v_mode
 // in {1, 2, 4, 30 (dense 3-bit)}.
-int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, int v_mode, int64_t samples,
+// coop (k_bits 1, 2, 4 only): a block's four waves share one tile -- a quarter of the channel rows each in the key
+// phase, then 256 positions each as a slab of its own (four workspace slabs per tile) -- for steps with too few
+// (query head, tile) pairs to fill the GPU with one wave each.
+int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int k_bits, bool coop, int v_mode, int64_t samples,
                           int64_t tail_blocks, hipStream_t stream);
 // grid and block of that launch (KVMIX_ERR_SHAPE for sizes the kernel does not take: fewer positions than one tile,
 // not whole groups, too many blocks for a grid)
-int plan_attn_slab_mfma(int k_mode, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3], unsigned block[3]);
+int plan_attn_slab_mfma(int k_mode, bool coop, int64_t tokens, int64_t samples, int64_t tail_blocks, unsigned grid[3],
+                        unsigned block[3]);
 
 }  // namespace kvmix

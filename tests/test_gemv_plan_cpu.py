@@ -173,9 +173,19 @@ def test_attention_step_plans_of_the_measured_shapes():
     p = _lib.attn_plan(_step(8, 32, 32, 3, REF, 8063, 2, REF, 8064, 8192))
     assert p["matrix"] and (p["matrix_tiles"], p["slab_begin"], p["slab_positions"], p["slabs"]) == (6, 7744, 352, 2)
     assert p["matrix_grid"][0] == 2 * 256 + 2 * 256 and p["launches"] == 2
-    # configs[4]'s size: the vector-ALU slab kernel from position 0
+    assert p["matrix_tile_waves"] == 1
+    # configs[4]'s size: few (query head, tile) pairs, so the four waves of a block share a tile (a block per tile)
     p = _lib.attn_plan(_step(4, 32, 32, 4, REF, 2176, 4, REF, 2176, 2304))
-    assert not p["matrix"] and p["slab_begin"] == 0 and p["slabs"] == 5 and p["launches"] == 2
+    assert p["matrix"] and p["matrix_tile_waves"] == 4 and p["matrix_tiles"] == 3 and p["slab_begin"] == 2176
+    assert p["matrix_grid"][0] == 3 * 128 + 128 and p["slabs"] == 1 and p["launches"] == 2 and p["recommended"]
+    # ... also with the reference's 3-bit keys from 128 pairs on (2167 -> 2112 = 6 * 352 positions, two tiles of 1408)
+    p = _lib.attn_plan(_step(4, 32, 32, 3, REF, 2167, 2, REF, 2176, 2304))
+    assert p["matrix"] and p["matrix_tile_waves"] == 4 and p["matrix_tiles"] == 2 and p["slab_begin"] == 2112
+    p = _lib.attn_plan(_step(1, 32, 32, 3, REF, 2167, 2, REF, 2176, 2304))
+    assert not p["matrix"] and p["slab_begin"] == 0 and p["slabs"] == 4 and p["launches"] == 2
+    # under one tile of quantized positions: the vector-ALU slab kernel from position 0
+    p = _lib.attn_plan(_step(4, 32, 32, 4, REF, 896, 4, REF, 896, 1024))
+    assert not p["matrix"] and p["matrix_tile_waves"] == 0 and p["slab_begin"] == 0 and p["slabs"] == 2 and p["launches"] == 2
     # one slab: the slab kernel stores the result itself
     p = _lib.attn_plan(_step(8, 32, 32, 2, REF, 384, 2, REF, 384, 512))
     assert not p["matrix"] and p["slabs"] == 1 and p["launches"] == 1
@@ -214,10 +224,13 @@ def test_no_attention_step_is_given_a_tile_longer_than_its_quantized_part():
                                 assert plan.slab_begin == both and plan.matrix_tiles == (both + tile - 1) // tile
                                 assert plan.slab_positions == (352 if unit == 11 else 256)
                                 blocks_per_head = (plan.matrix_grid[0] - plan.slab_blocks) // (batch * heads)
-                                assert blocks_per_head * plan.matrix_block[1] >= plan.matrix_tiles and plan.matrix_block[1] == 4
+                                assert plan.matrix_tile_waves in (1, 4) and plan.matrix_block[1] == 4
+                                # a wave per tile (blocks of four tiles) or a block per tile
+                                assert blocks_per_head * (4 // plan.matrix_tile_waves) >= plan.matrix_tiles
+                                assert (blocks_per_head - 1) * (4 // plan.matrix_tile_waves) < plan.matrix_tiles
                                 assert plan.matrix_grid[0] == blocks_per_head * batch * heads + plan.slabs * batch * heads
                             else:
-                                assert plan.slab_begin == 0 and plan.matrix_tiles == 0
+                                assert plan.slab_begin == 0 and plan.matrix_tiles == 0 and plan.matrix_tile_waves == 0
                             assert plan.slab_begin + plan.slabs * plan.slab_positions >= width
                             checked += 1
     assert checked > 5000

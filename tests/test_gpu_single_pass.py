@@ -316,3 +316,43 @@ def test_matrix_core_steps_with_the_reference_three_bit_keys(dev, v_bits, tk, tv
     vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
     logits = (q[sl, :2 * rep].double() @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
     check(out_s[sl, :2 * rep], torch.softmax(logits, -1) @ vals, vm)
+
+
+@pytest.mark.parametrize("k_bits", [1, 2, 3, 4])
+@pytest.mark.parametrize("v_bits,tk,dv", [(1, 2176, 0), (2, 1152, 32), (3, 2560, -64), (4, 3072, 0)])
+def test_steps_with_few_tiles_share_a_tile_among_four_waves(dev, k_bits, v_bits, tk, dv):
+    """Steps with few (query head, tile) pairs -- the sizes of a small-batch decode loop -- run a block per tile: the
+    four waves take a quarter of the channel rows each for the logits and then a quarter of the tile's positions
+    each as a slab of its own.  Query heads sharing kv heads, a padding mask, last tiles moved back by up to 7/8 of
+    their length, values quantized further or less far than the keys; against the four-launch step and, for two rows,
+    fp64 attention over the dequantized cache."""
+    from kvmix_amd import ops, _lib
+    from helpers import dequantize_torch
+
+    kg = 11 if k_bits == 3 else 32
+    tk = tk // 352 * 352 + 33 * 11 if k_bits == 3 else tk  # (the reference's words: whole words, not whole tiles)
+    tv = tk // 32 * 32 + dv
+    gen = torch.Generator(device=dev).manual_seed(700 + 10 * k_bits + v_bits)
+    rng = np.random.default_rng(31 * k_bits + v_bits)
+    B, nkv, rep = 4, 8, 4
+    n = max(tk, tv) + 93
+    plan = _lib.attn_plan(_lib.attn_step_descriptor(B, nkv * rep, nkv, 128, k_bits, 0, kg, tk, v_bits, 1 if v_bits == 3 else 0, 32, tv,
+                                                   n - tk, n - tv))
+    assert plan["matrix"] and plan["matrix_tile_waves"] == 4 and plan["launches"] == 2 and plan["recommended"], plan
+    q, kq, vq, k_tail, v_tail, kg, mask, fmt, lk, lv = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tv, n, mask_rng=rng)
+    out_f, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, **fmt)
+    out_s, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
+    vm = v_magnitude(vq, v_tail, v_bits)
+    check(out_s, out_f, vm)
+    sl = slice(B - 1, B)
+    kd = dequantize_torch(kq[0][sl, :2], kq[1][sl, :2], kq[2][sl, :2], k_bits, kg).double()
+    vd = dequantize_torch(vq[0][sl, :2], vq[1][sl, :2], vq[2][sl, :2], v_bits, 32, dense3=v_bits == 3).double()
+    keys = torch.cat([kd.transpose(2, 3), k_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    vals = torch.cat([vd, v_tail[sl, :2].double()], 2).repeat_interleave(rep, 1)
+    logits = (q[sl, :2 * rep].double() @ keys.transpose(2, 3)).half().double() / np.sqrt(128.0) + mask[sl].double()
+    check(out_s[sl, :2 * rep], torch.softmax(logits, -1) @ vals, vm)
+    # a second call on other data of the same sizes, then the first again: nothing is carried between calls
+    q2 = torch.randn(q.shape, device=dev, generator=gen).half()
+    ops.decode_attention(q2, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
+    again, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
+    assert torch.equal(again, out_s)
