@@ -3152,6 +3152,23 @@ int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int 
     return launch_status();
 }
 
+// gemv_cols3 with one head per pass: where tiles of 256 words with one wave each, every wave walking all 128 channel
+// rows, lay exactly one block on every CU -- 224 to 256 output rows of three or four tiles, the block = the tiles
+// of a row -- or exactly three blocks of four waves, they are ahead of the K-sliced 128-word tiles (which put 6 to
+// 24 waves on every SIMD): the waves stream 1 KiB pieces of a row and nothing queues.  Measured (us, K-sliced ->
+// whole rows): B = 8, T = 8192 (256 rows x 3 tiles): 36.3 -> 32.7; T = 7500: 33.6 -> 29.8; T = 8576: 36.8 -> 34.2;
+// T = 11264 (4 tiles): 50.3 -> 43.0; B = 7: 33.3 -> 30.7; three blocks per CU: B = 8, T = 32768: 146.5 -> 138.7; B = 24,
+// T = 11264: 147.1 -> 140.0.  One block more than the CUs and the launch takes two rounds: B = 9, T = 8192 (288
+// rows): 39.1 -> 57.7, B = 10: 43.9 -> 58.8; fewer rows leave CUs idle: B = 6: 28.7 -> 30.3; other wave counts lose 2 to
+// 7 % (B = 16, T = 8192: 68.9 -> 71.6; B = 6, T = 32768: 108.6 -> 115.8).
+static bool cols3_whole_rows(int64_t units, int64_t rows)
+{
+    if (units < 513) return false;
+    const int64_t tiles = (units + 255) / 256;
+    if (tiles <= 4) return rows >= 224 && rows <= 256;
+    return tiles % 4 == 0 && rows * (tiles / 4) >= 736 && rows * (tiles / 4) <= 768;
+}
+
 template <int MODE>
 static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
 {
@@ -3205,8 +3222,14 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         // words per wave) that still gives the chip enough waves and fits into N
         const int64_t units = a.N / 11, batch = samples * a.M;
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
+        bool force_wide = false;
+#ifdef KVMIX_EXPERIMENT
+        if (const char *e = getenv("KVMIX_DBG_COLS3_WIDE")) force_wide = atoi(e) != 0 && units >= 256;
+#endif
         if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
+        else if (force_wide || cols3_whole_rows(units, batch))
+            launch_cols3_cfg<1, 4, 1>(a, samples, st);
         else if (units >= 128 && 2 * ((units + 127) / 128) * 128 <= 3 * units && a.K >= 64 &&
                  a.K <= 4096 && (waves(128) * 4 <= 1024 || waves(128) * 4 >= 2304))
             // tiles of 128 words (512 bytes of codes per row), each shared by four waves that slice K: measured

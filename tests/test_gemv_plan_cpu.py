@@ -51,8 +51,18 @@ def test_config1_mixed_bits_b8_t8192():
     assert plan(4, REF, 32, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols<4,")
     # the reference's 3-bit keys: 11 codes a word, 8063 = 733 * 11 tokens
     ref3 = plan(3, REF, 8, 32, 1, 8063, 128, "qk")
-    # 128-word tiles, four waves a tile, each with a quarter of the channel rows
-    assert ref3["kernel"] == "gemv_cols3<2,4,8,1>" and ref3["ksplit"] == 4 and ref3["grid"][:2] == (6, 256)
+    # 256 rows of three 256-word tiles: a block per row, a wave per tile that walks all channel rows -- one block on
+    # every CU
+    assert ref3["kernel"] == "gemv_cols3<1,4,8,1>" and ref3["ksplit"] == 1 and ref3["grid"][:2] == (1, 256)
+    assert ref3["block"] == (64, 3, 1)
+    # one row more than there are CUs, or a longer row: 128-word tiles, four waves a tile, each with a quarter of
+    # the channel rows
+    ref3 = plan(3, REF, 9, 32, 1, 8063, 128, "qk")
+    assert ref3["kernel"] == "gemv_cols3<2,4,8,1>" and ref3["ksplit"] == 4 and ref3["grid"][:2] == (6, 288)
+    ref3 = plan(3, REF, 8, 32, 1, 1477 * 11, 128, "qk")
+    assert ref3["kernel"] == "gemv_cols3<2,4,8,1>" and ref3["ksplit"] == 4
+    # ... and again whole rows where they make three blocks of four waves per CU
+    assert plan(3, REF, 8, 32, 1, 2967 * 11, 128, "qk")["kernel"] == "gemv_cols3<1,4,8,1>"
     assert plan(3, DENSE3, 8, 32, 1, 8064, 128, "qk")["kernel"].startswith("gemv_cols<30,")
     for bits, mode in ((4, 4), (2, 2)):
         assert plan(bits, REF, 8, 32, 1, 8064, 128, "pv")["kernel"] == f"gemv_rows_mfma<{mode},1,1>"

@@ -104,6 +104,11 @@ def test_reference_3bit_kernel_edges(oracle, dev):
     run_case(oracle, dev, 3, 11, B=1, nh=3, nkv=3, K=65, N=11 * 128, seed=59)       # ... one tile exactly, a one-row last slice
     run_case(oracle, dev, 3, 11, B=1, nh=1, nkv=1, K=4096, N=11 * 250, seed=60)     # ... the most rows the sliced form takes
     run_case(oracle, dev, 3, 11, B=32, nh=32, nkv=32, K=32, N=11 * 1024, seed=61)   # too few rows to slice: widest tiles, one wave each
+    # whole rows: a block per output row, a wave per 256-word tile over all channel rows (one block per CU, or three)
+    from kvmix_amd import _lib
+    for B, words in ((8, 733), (7, 1012), (8, 2967)):
+        assert _lib.gemv_plan(11, 3, 0, B * 32, 1, 1, 128, 11 * words)["kernel"] == "gemv_cols3<1,4,8,1>"
+        run_case(oracle, dev, 3, 11, B=B, nh=32, nkv=32, K=128, N=11 * words, seed=62 + B + words)
 
 
 @pytest.mark.parametrize("bits,g", [(4, 8), (2, 16), (1, 64), (4, 64), (3, 11)])
