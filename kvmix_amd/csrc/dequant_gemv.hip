@@ -853,10 +853,11 @@ gemv_cols3(GemvArgs a)
         uint16_t *op = reinterpret_cast<uint16_t *>(a.out) + (sample0 + h) * a.o_bs + m * a.o_rs + (int64_t)unit0 * VALS;
         if constexpr (RQ == 1) {
 #pragma unroll
-            for (int e = 0; e < TOT; e += 2) {
+            for (int e = 0; e + 1 < TOT; e += 2) {
                 const uint32_t pk = f32_to_h16(flat[e]) | ((uint32_t)f32_to_h16(flat[e + 1]) << 16);
                 __builtin_memcpy(op + e, &pk, 4);
             }
+            if constexpr (TOT % 2 == 1) op[TOT - 1] = f32_to_h16(flat[TOT - 1]);
         } else {
             // halving butterfly: each section ends with its share of the sums (TOT / RQ each)
             static_assert(RQ == 2 && TOT % 2 == 0, "two sections, equal shares");
@@ -3160,7 +3161,8 @@ int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int 
 // T = 11264 (4 tiles): 50.3 -> 43.0; B = 7: 33.3 -> 30.7; three blocks per CU: B = 8, T = 32768: 146.5 -> 138.7; B = 24,
 // T = 11264: 147.1 -> 140.0.  One block more than the CUs and the launch takes two rounds: B = 9, T = 8192 (288
 // rows): 39.1 -> 57.7, B = 10: 43.9 -> 58.8; fewer rows leave CUs idle: B = 6: 28.7 -> 30.3; other wave counts lose 2 to
-// 7 % (B = 16, T = 8192: 68.9 -> 71.6; B = 6, T = 32768: 108.6 -> 115.8).
+// 7 % (B = 16, T = 8192: 68.9 -> 71.6; B = 6, T = 32768: 108.6 -> 115.8).  Tiles of 192 words (three per lane), which
+// would put a wave on every SIMD at 256 rows x 733 words, lose to the 12- and 6-byte loads they need (32.8 -> 39.1).
 static bool cols3_whole_rows(int64_t units, int64_t rows)
 {
     if (units < 513) return false;
@@ -3224,7 +3226,7 @@ static void launch_cols(GemvArgs &a, int64_t samples, hipStream_t st)
         auto waves = [&](int64_t tu) { return batch * ((units + tu - 1) / tu); };
         bool force_wide = false;
 #ifdef KVMIX_EXPERIMENT
-        if (const char *e = getenv("KVMIX_DBG_COLS3_WIDE")) force_wide = atoi(e) != 0 && units >= 256;
+        if (const char *e = getenv("KVMIX_DBG_COLS3_WIDE")) force_wide = atoi(e) == 1 && units >= 256;
 #endif
         if (heads_per_block(a.heads_per_kv) == 4 && a.K <= 2048)  // GQA: four query heads per pass over the
             launch_cols3_cfg<2, 2, 4>(a, samples, st);              // words (their x rows must fit into LDS)
