@@ -104,10 +104,19 @@ def build_layers(torch, ops, lib, B, H, D, T, R, kbits, vbits, dev):
         L.vtail = V[:, :, L.Tqv:L.Tqv + L.nv].contiguous()
         del V, vin
         L.q = torch.randn(B, H, 1, D, device=dev, dtype=torch.float16, generator=gen)
-        L.p = torch.softmax(torch.randn(B, H, 1, L.Tqv, device=dev, generator=gen), -1).half()
-        # outputs (fixed buffers: the state of the cache does not change between steps)
-        L.logits = torch.empty(B, H, 1, L.Tqk, device=dev, dtype=torch.float16)
-        L.out = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+        # Scratch of the attention step -- logits out, probabilities in, output -- is one buffer each for all layers,
+        # as in a decode loop, whose allocator hands the same blocks to every layer (the logits of a layer are
+        # consumed before the next layer runs, the probabilities have just been written by its softmax).  Measured
+        # against a buffer set per layer: 2.195 / 2.171 ms (shared outputs / also the probabilities) against 2.229 ms.
+        # The packed caches, the flush sources and the flush targets are per layer.
+        if not layers:
+            shared = Layer()
+            shared.p = torch.softmax(torch.randn(B, H, 1, ((T - R) // 32) * 32, device=dev, generator=gen), -1).half()
+            shared.logits = torch.empty(B * H * (T - R), device=dev, dtype=torch.float16)
+            shared.out = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+        L.p = shared.p
+        L.logits = shared.logits[:B * H * L.Tqk].view(B, H, 1, L.Tqk)
+        L.out = shared.out
         kw = L.nk // 11 if kb == 3 else L.nk * kb // 32
         L.fk_code = torch.empty(B, H, D, kw, device=dev, dtype=torch.int32)
         L.fk_s = torch.empty(B, H, D, L.nk // L.kg, device=dev, dtype=torch.float16)
@@ -925,6 +934,8 @@ def main():
             "batch": B, "context": T, "heads": H, "head_dim": D, "group": 32, "residual": R, "layers": args.layers,
             "k_bits": kbits, "v_bits": vbits, "k3_format": "reference 11-per-word (group 11)",
             "v3_format": "dense 3-bit stream (extension)", "launch": mode,
+            "scratch": "logits, probabilities and attention output: one buffer each shared by the layers, as a decode "
+                       "loop reuses them; packed caches, flush sources and flush targets per layer",
         },
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "kv_path_only_decode_tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
