@@ -3162,7 +3162,9 @@ int launch_attn_step_mfma(const AttnSlabArgs &a, const fused::FusedArgs &f, int 
 // T = 11264: 147.1 -> 140.0.  One block more than the CUs and the launch takes two rounds: B = 9, T = 8192 (288
 // rows): 39.1 -> 57.7, B = 10: 43.9 -> 58.8; fewer rows leave CUs idle: B = 6: 28.7 -> 30.3; other wave counts lose 2 to
 // 7 % (B = 16, T = 8192: 68.9 -> 71.6; B = 6, T = 32768: 108.6 -> 115.8).  Tiles of 192 words (three per lane), which
-// would put a wave on every SIMD at 256 rows x 733 words, lose to the 12- and 6-byte loads they need (32.8 -> 39.1).
+// would put a wave on every SIMD at 256 rows x 733 words, lose to the 12- and 6-byte loads they need (32.8 -> 39.1);
+// so does a fourth wave per block that takes the last quarter of the channel rows of all three tiles and hands its
+// sums over in LDS (33.7 -> 36.6).
 static bool cols3_whole_rows(int64_t units, int64_t rows)
 {
     if (units < 513) return false;
