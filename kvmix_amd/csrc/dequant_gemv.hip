@@ -2180,19 +2180,21 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
 }
 
 // ---------------------------------------------------------------------------------------
-// attn_slab_mfma<KBITS, VMODE>   the single-pass decode step over the quantized positions, on the matrix
-// cores: one wave = one slab of 1024 positions of one query head (D = 128).
-//   1. logits of the slab: the q.K^T tile of gemv_cols_mfma2 (one tile per wave), the sums kept in registers;
-//      each is rounded to fp16, scaled by 1/sqrt(D) and masked as the reference does it.
+// attn_slab_mfma_body<KBITS, VMODE, COOP>   a tile of the single-pass decode step (attn_step_mfma below) over the
+// quantized positions, on the matrix cores: 1024 positions of one query head (D = 128).
+//   1. logits of the tile: the q.K^T tile of gemv_cols_mfma2, the sums kept in registers; each is rounded to fp16,
+//      scaled by 1/sqrt(D) and masked as the reference does it.
 //   2. slab maximum m, p = exp(logit - m) (fp32), their sum l; p goes to the wave's LDS row in position order.
-//   3. p.V over the same 1024 positions, as gemv_rows_mfma does it (eight 128-row chunks), with p taken from
-//      LDS instead of an fp16 vector in memory.
-//   (m, l) and the 128 unnormalised outputs go to the workspace as slab `tile` of the row; the fp16 tails are
-//   further slabs (attn_fused_slab) and attn_fused_merge combines them all.
-//   The last tile of a row is moved back to end at `tokens`; the positions it shares with its neighbour get
-//   p = 0 there.  No block barrier anywhere: a wave without a tile simply leaves.
-//   block = (64, 2..4) waves on neighbouring tiles; grid = (tiles / waves, samples), XCD-swizzled;
-//   dynamic LDS = waves * kSlabLds bytes.
+//   3. p.V over the same positions, as gemv_rows_mfma does it (128-row chunks), with p taken from LDS instead of an
+//      fp16 vector in memory.
+//   (m, l) and the 128 unnormalised outputs go to the workspace as a slab of the row; the vector-ALU slabs over the
+//   remaining positions (trailing blocks of the same launch) are further slabs and attn_fused_merge combines all.
+//   The last tile of a row is moved back to end at `tokens`; the positions it shares with its neighbour get p = 0.
+//   COOP = false: one wave per tile (slab = tile), block = (64, 4) waves on neighbouring tiles, no block barrier: a
+//   wave without a tile simply leaves.  COOP = true: the block's four waves share ONE tile: wave w takes channel
+//   rows [32 w, 32 w + 32) in step 1, the partial sums of all 1024 positions meet in LDS (two block barriers),
+//   then wave w runs steps 2 and 3 on positions [256 w, 256 w + 256) as a slab of its own (four slabs per tile).
+//   Dynamic LDS = 4 * kSlabLds bytes either way.
 // ---------------------------------------------------------------------------------------
 constexpr int kSlabKeyBytes = (kColsMfma2Tile * 2 + 32 * 4 + 15) / 16 * 16;  // A tile of the key phase + 32 zero terms
 constexpr int kSlabLds = kSlabKeyBytes + 1024 * 4;                            // ... + the slab's probabilities

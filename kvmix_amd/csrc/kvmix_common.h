@@ -118,7 +118,7 @@ __device__ __forceinline__ int scatter_reduce(float *v, int lane)
     }
 }
 
-// One slab of the single-pass decode step on the matrix cores (attn_slab_mfma in dequant_gemv.hip, launched for
+// The matrix-core tiles of the single-pass decode step (attn_step_mfma in dequant_gemv.hip, launched for
 // kvmix_decode_attention_fused in fused_attn.hip): the quantized positions [0, tokens) of keys and values alike.
 struct AttnSlabArgs {
     const uint16_t *q;        // [samples, 128] fp16
