@@ -181,7 +181,7 @@ def run_step(calls):
             raise RuntimeError(f"kvmix call failed: {rc}")
 
 
-def time_kernels(torch, calls, reps=3):
+def time_kernels(torch, calls, reps=10):
     """Per kernel kind: average duration of one launch (events on the launch stream), over the
     step's own launches (each on its own layer's buffers, so nothing is served from cache)."""
     kinds = {}
