@@ -910,6 +910,12 @@ def main():
             traffic = tj.get(dname)
             traffic_source = ("profiles/hbm_traffic.json (static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                               + str(tj.get("_measured", "date not recorded")) + "; not re-measured in this run)")
+            # the figure belongs to the device kernel that ran when the counters were taken: if the dispatch has
+            # moved on since, it is not this kernel's traffic
+            then, now = tj.get("_kernels", {}).get(dname), device_kernel(_lib, dname, B, H, D, T - R)
+            if then is not None and then != now:
+                traffic = None
+                traffic_source += f" -- stale: measured on {then}, the step now runs {now}"
         except Exception:
             traffic = None
     gemv_us = sum(v["launches_per_step"] * v["avg_us"] for k, v in per_kernel.items() if k.startswith("gemv"))

@@ -448,6 +448,16 @@ def test_full_size_properties_batch128_t4096(dev, bits):
         assert torch.equal(out[:, :, 0].to(torch.int32), _unpack_torch(vcode[:, :, :2016], bits).sum(2))
 
 
+@pytest.mark.parametrize("batch", [1, 16, 64])
+@pytest.mark.parametrize("bits", [1, 2])
+def test_config3_sizes_against_the_oracle(oracle, dev, bits, batch):
+    """BASELINE configs[3] at its smaller batches (T = 4096, residual 32: 4064 quantized tokens, 32 heads, 1 and 2
+    bits): whole q.K^T and p.V launches of those sizes against the oracle (the largest batch has its closed-form
+    test above)."""
+    run_case(oracle, dev, bits, 32, B=batch, nh=32, nkv=32, K=128, N=4064, seed=300 + batch + bits)
+    run_case(oracle, dev, bits, 32, B=batch, nh=32, nkv=32, K=4064, N=128, seed=400 + batch + bits)
+
+
 def test_more_slices_than_one_grid_dimension_holds(oracle, dev):
     """B x heads beyond 65535 (the limit of grid.y): the call goes out in parts over whole kv heads."""
     run_case(oracle, dev, 4, 32, B=16385, nh=4, nkv=4, K=16, N=64, seed=71)      # 65540 slices, two parts
