@@ -244,3 +244,23 @@ def test_no_attention_step_is_given_a_tile_longer_than_its_quantized_part():
                             assert plan.slab_begin + plan.slabs * plan.slab_positions >= width
                             checked += 1
     assert checked > 5000
+
+
+def test_committed_traffic_figures_belong_to_the_kernels_the_step_runs():
+    """profiles/hbm_traffic.json carries, beside every HBM-traffic figure bench.py quotes as roofline.traffic, the
+    device kernel it was measured on; the bench drops a figure whose kernel the dispatch no longer picks.  Here:
+    the committed file is current -- every GEMV of the bench step (B = 8, T = 8192, R = 128) still gets that kernel."""
+    import json
+    import os
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, root)
+    import bench
+
+    tj = json.load(open(os.path.join(root, "profiles", "hbm_traffic.json")))
+    names = tj["_kernels"]
+    gemvs = [t for t in names if t.startswith("gemv")]
+    assert sorted(gemvs) == sorted(t for t in tj if t.startswith("gemv"))
+    for tag in gemvs:
+        assert bench.device_kernel(_lib, tag, 8, 32, 128, 8192 - 128) == names[tag], tag
