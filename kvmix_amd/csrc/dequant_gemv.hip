@@ -73,7 +73,10 @@ constexpr int kMfma2ResidentWaves = 3072;   // gemv_cols_mfma2: 3 waves on each 
 constexpr int64_t kMfma2WideMinCodes = 6144;    // gemv_cols_mfma2: rows from this many codes on may take the wide tiles
 constexpr int64_t kMfma2WideMaxWaves = 2048;    // ... in launches of up to this many of them (one round, two waves per SIMD)
 constexpr int kMfma2KsplitWaves = 1536;     // gemv_cols_mfma2: waves share a tile (slicing K) while that keeps the launch below this many waves
-constexpr int kRowsChunksPerWave = 8;       // p.V: chunks a wave should get before more waves per row are used
+#ifndef KVMIX_ROWS_CHUNKS_PER_WAVE
+#define KVMIX_ROWS_CHUNKS_PER_WAVE 8
+#endif
+constexpr int kRowsChunksPerWave = KVMIX_ROWS_CHUNKS_PER_WAVE;  // p.V: chunks a wave should get before more waves per row are used
 constexpr int kRowsSingleBlockChunks = 2;   // p.V: keep one block per output row up to this many chunks per wave
 constexpr int kCols3WideWaves = 4096;       // gemv_cols3: widest tiles (one wave each) from this many of them on
 constexpr int kCols3MinWaves = 2048;        // gemv_cols3: 128-word one-wave tiles from this many of them on
@@ -2866,6 +2869,14 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
         if (lean < want) want = lean;
     }
     if (want < 1) want = 1;
+    // a block whose wave count is no multiple of four loads the CU's four SIMDs unevenly (measured at T = 8k, 2 / 4
+    // bits, us: 24 x 32 rows with 6 waves 54.5 / 79.6, with 4 waves 48.7 / 75.5; 20 x 32 rows, 7 -> 4 waves: 47.3 ->
+    // 45.2 / 68.8 -> 66.3; 12 x 32 rows, 6 waves 38.1 / 45.6 against 8 waves 33.6 / 43.2): up to the next multiple
+    // while all waves of the launch stay resident (four per SIMD), else down
+    if (want > 4 && want < max_waves && want % 4 != 0) {
+        const int64_t up = (want + 3) / 4 * 4;
+        want = batch_rows * up <= target ? up : want / 4 * 4;
+    }
 #ifdef KVMIX_EXPERIMENT
     if (const char *e = getenv("KVMIX_DBG_ROWS_WAVES")) want = atoll(e);
 #endif
