@@ -2869,10 +2869,11 @@ static RowsPlan plan_rows(int64_t batch_rows, int64_t K, int64_t N, int max_wave
         if (lean < want) want = lean;
     }
     if (want < 1) want = 1;
-    // a block whose wave count is no multiple of four loads the CU's four SIMDs unevenly (measured at T = 8k, 2 / 4
-    // bits, us: 24 x 32 rows with 6 waves 54.5 / 79.6, with 4 waves 48.7 / 75.5; 20 x 32 rows, 7 -> 4 waves: 47.3 ->
-    // 45.2 / 68.8 -> 66.3; 12 x 32 rows, 6 waves 38.1 / 45.6 against 8 waves 33.6 / 43.2): up to the next multiple
-    // while all waves of the launch stay resident (four per SIMD), else down
+    // blocks of 5, 6 or 7 waves are slower than blocks of 4 or 8 (four SIMDs per CU, and a launch a little larger
+    // than the resident waves).  Measured at T = 8k, 2 / 4 bits, us: 28 x 32 rows, 5 -> 4 waves: 76.1 -> 59.7 / 104.5 ->
+    // 90.8; 24 x 32 rows, 6 -> 4: 53.2 -> 49.0 / 79.6 -> 75.6; 20 x 32 rows, 7 -> 4: 49.1 -> 46.7 / 69.0 -> 66.6; 12 x 32
+    // rows, 6 waves 38.1 / 45.6 against 8 waves 33.6 / 43.2.  Up to the next multiple of four while all waves of the
+    // launch stay resident (four per SIMD), else down
     if (want > 4 && want < max_waves && want % 4 != 0) {
         const int64_t up = (want + 3) / 4 * 4;
         want = batch_rows * up <= target ? up : want / 4 * 4;
