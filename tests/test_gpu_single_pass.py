@@ -356,3 +356,34 @@ def test_steps_with_few_tiles_share_a_tile_among_four_waves(dev, k_bits, v_bits,
     ops.decode_attention(q2, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
     again, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, attention_mask=mask, single_pass=True, **fmt)
     assert torch.equal(again, out_s)
+
+
+@pytest.mark.parametrize("k_bits", [4, 3])
+def test_shared_tiles_with_device_side_lengths_and_eight_heads_per_kv_head(dev, k_bits):
+    """The four-waves-per-tile form with eight query heads per kv head, tails in longer windows whose lengths live on
+    the device, and a second tile that is moved back almost wholly (4-bit keys: 1056 positions; the reference's
+    3-bit keys: 1408 + 352)."""
+    from kvmix_amd import ops, _lib
+
+    gen = torch.Generator(device=dev).manual_seed(900 + k_bits)
+    B, nkv, rep, v_bits = 2, 8, 8, 2
+    kg = 11 if k_bits == 3 else 32
+    tk = 1408 + 352 + 11 * 5 if k_bits == 3 else 1056
+    tv = tk // 32 * 32
+    lk = 41 + (tk - tv)
+    n = tv + lk
+    plan = _lib.attn_plan(_lib.attn_step_descriptor(B, nkv * rep, nkv, 128, k_bits, 0, kg, tk, v_bits, 0, 32, tv, n - tk, n - tv))
+    assert plan["matrix"] and plan["matrix_tile_waves"] == 4, plan
+    q, kq, vq, k_tail, v_tail, kg, _, fmt, lk_, lv_ = make_case(dev, gen, B, nkv, rep, k_bits, v_bits, tk, tv, n)
+    want, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, **fmt)
+    got, _ = ops.decode_attention(q, kq, vq, k_tail, v_tail, kg, k_bits, 32, v_bits, single_pass=True, **fmt)
+    check(got, want, v_magnitude(vq, v_tail, v_bits))
+    R = max(lk_, lv_) + 23
+    kwin = torch.full((B, nkv, R, 128), 77.0, dtype=torch.float16, device=dev)
+    vwin = torch.full((B, nkv, R, 128), float("nan"), dtype=torch.float16, device=dev)
+    kwin[:, :, :lk_], vwin[:, :, :lv_] = k_tail, v_tail
+    klen = torch.tensor([lk_], dtype=torch.int64, device=dev)
+    vlen = torch.tensor([lv_], dtype=torch.int64, device=dev)
+    got2, _ = ops.decode_attention(q, kq, vq, kwin, vwin, kg, k_bits, 32, v_bits, k_tail_len=klen, v_tail_len=vlen,
+                                   single_pass=True, **fmt)
+    assert torch.equal(got2, got)
