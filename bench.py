@@ -154,9 +154,6 @@ def make_calls(torch, _lib, lib, layers, B, H, D, stream):
                                    L.fv_code.stride(2), L.fv_s.data_ptr(), L.fv_z.data_ptr(), L.fv_s.stride(1),
                                    L.fv_s.stride(2))
 
-        def fl(L=L):
-            return lib.kvmix_quant_pack_kv_flush(ctypes.byref(L.kflush), ctypes.byref(L.vflush), stream)
-
         def qk(L=L):
             return lib.kvmix_quantized_gemv(
                 L.kg, L.q.data_ptr(), D, D, L.kc.data_ptr(), L.kc.stride(1), L.kc.stride(2), L.ks.data_ptr(),
@@ -169,9 +166,21 @@ def make_calls(torch, _lib, lib, layers, B, H, D, stream):
                 L.vz.data_ptr(), L.vs.stride(1), L.vs.stride(2), L.vb, vfmt, B * H, 1, 1, L.Tqv, D,
                 L.out.data_ptr(), D, D, L.ws.data_ptr(), L.wsb, stream)
 
-        calls += [(f"quant_kv_flush[{L.kfmt},{L.vfmt}]", L.bytes_fk + L.bytes_fv, fl),
-                  (f"gemv_cols[{L.kfmt}]", L.bytes_qk, qk), (f"gemv_rows[{L.vfmt}]", L.bytes_pv, pv)]
-    return calls
+        calls += [(f"gemv_cols[{L.kfmt}]", L.bytes_qk, qk), (f"gemv_rows[{L.vfmt}]", L.bytes_pv, pv)]
+    # The flushes of the step, batched: what a layer flushes in a decode step are the oldest tokens of its fp16
+    # tails (models/modeling_llama_KVmix.py:122-127,152-156), tokens of earlier steps, so the flushes of all layers
+    # go out before the first layer runs -- kvmix_quant_pack_kv_flush_batch, eight layers to a launch.
+    flushes = []
+    for i in range(0, len(layers), 8):
+        part = layers[i:i + 8]
+        ka = (ctypes.POINTER(_lib.KeyFlush) * len(part))(*[ctypes.pointer(L.kflush) for L in part])
+        va = (ctypes.POINTER(_lib.ValueFlush) * len(part))(*[ctypes.pointer(L.vflush) for L in part])
+
+        def fl(ka=ka, va=va, n=len(part)):
+            return lib.kvmix_quant_pack_kv_flush_batch(ka, va, n, stream)
+
+        flushes.append((f"quant_kv_flush_batch[{len(part)} layers]", sum(L.bytes_fk + L.bytes_fv for L in part), fl))
+    return flushes + calls
 
 
 def run_step(calls):
@@ -936,7 +945,8 @@ def main():
         "dtype": "u32 codes / fp16 scale,zero / fp32 accumulate",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE configs[1]: 32-layer Llama-2-7B KV shape, mixed per-layer bits, one flush + q.K^T + p.V per layer",
+            "workload": "BASELINE configs[1]: 32-layer Llama-2-7B KV shape, mixed per-layer bits, one flush + q.K^T + p.V per layer "
+                        "(the layers' flushes batched eight to a launch at the head of the step: they take tokens of earlier steps only)",
             "batch": B, "context": T, "heads": H, "head_dim": D, "group": 32, "residual": R, "layers": args.layers,
             "k_bits": kbits, "v_bits": vbits, "k3_format": "reference 11-per-word (group 11)",
             "v3_format": "dense 3-bit stream (extension)", "launch": mode,

@@ -147,6 +147,20 @@ int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *key, const kvmix_value_fl
                               kvmix_stream_t stream);
 
 /*
+ * The flushes of several layers (or caches) at once: `count` (key, value) pairs as arrays of descriptor pointers,
+ * eight pairs to a launch, the results those of kvmix_quant_pack_kv_flush on each pair, bit for bit.  In the
+ * reference every layer flushes inside its own forward (models/modeling_llama_KVmix.py:119-167), but what a layer
+ * flushes in a decode step are the OLDEST tokens of its fp16 tail (`key_states_full[:, :, :to_quantize_length]`,
+ * lines 122-127, 152-156) -- tokens of earlier steps -- and how many follows from the tail's length alone: the
+ * flushes of all layers of a step can be issued together before its first layer runs.  A flush is a latency-bound
+ * launch of about 10 us whatever its size; eight layers in one launch take about as long as two alone.
+ * All pairs are validated before anything is launched; a pair that kvmix_quant_pack_kv_flush would run as separate
+ * launches (an empty half, a value half that is not the group-32 fp16 case) is run so here too.
+ */
+int kvmix_quant_pack_kv_flush_batch(const kvmix_key_flush_t *const *keys, const kvmix_value_flush_t *const *values,
+                                    int count, kvmix_stream_t stream);
+
+/*
  * Fused dequantize + matrix-vector product over the packed cache.
  * Replaces quantized_gemm (quant_cuda/csrc/dequantization_gemv_cuda.h:22-29,
  * dequantization_gemv_cuda.cu:7-248):

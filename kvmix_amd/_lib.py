@@ -24,6 +24,7 @@ EXPORTS = (
     "kvmix_quant_pack_last_dim",
     "kvmix_quant_pack_key_tokens",
     "kvmix_quant_pack_kv_flush",
+    "kvmix_quant_pack_kv_flush_batch",
     "kvmix_gemv_workspace_bytes",
     "kvmix_quantized_gemv",
     "kvmix_quantized_gemv_static",
@@ -132,6 +133,9 @@ def load() -> ctypes.CDLL:
                                               vp, i64, i64, vp, vp, i64, i64, vp]
     L.kvmix_quant_pack_kv_flush.restype = i32
     L.kvmix_quant_pack_kv_flush.argtypes = [ctypes.POINTER(KeyFlush), ctypes.POINTER(ValueFlush), vp]
+    L.kvmix_quant_pack_kv_flush_batch.restype = i32
+    L.kvmix_quant_pack_kv_flush_batch.argtypes = [ctypes.POINTER(ctypes.POINTER(KeyFlush)),
+                                                  ctypes.POINTER(ctypes.POINTER(ValueFlush)), ctypes.c_int, vp]
     L.kvmix_gemv_workspace_bytes.restype = sz
     L.kvmix_gemv_workspace_bytes.argtypes = [i64, i64, i64, i64]
     L.kvmix_quantized_gemv.restype = i32
@@ -215,6 +219,16 @@ def attn_plan(step: DecodeAttn) -> dict:
             "slab_positions": plan.slab_positions, "slab_begin": plan.slab_begin, "slabs": plan.slabs,
             "slab_blocks": plan.slab_blocks, "matrix_grid": tuple(plan.matrix_grid),
             "matrix_block": tuple(plan.matrix_block)}
+
+
+def flush_batch(keys, values, stream) -> int:
+    """kvmix_quant_pack_kv_flush_batch over sequences of KeyFlush / ValueFlush descriptors; returns the library's code."""
+    n = len(keys)
+    if n != len(values):
+        raise ValueError("as many key as value descriptors")
+    ka = (ctypes.POINTER(KeyFlush) * n)(*[ctypes.pointer(k) for k in keys])
+    va = (ctypes.POINTER(ValueFlush) * n)(*[ctypes.pointer(v) for v in values])
+    return load().kvmix_quant_pack_kv_flush_batch(ka, va, n, stream)
 
 
 def strerror(code: int) -> str:

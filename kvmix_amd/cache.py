@@ -28,12 +28,16 @@ def flush_length(tail_len: int, ratio: float, group: int, residual_length: Optio
 
     Ratio rule (models/modeling_llama_KVmix.py:119-127,152-155 and, for the prompt, :219-224):
     keep int(ratio * L) tokens in fp16, quantize the rest rounded down to a multiple of the group.
-    Fixed window (residual_length = R): once the tail holds R tokens, flush floor(R/g)*g; for a
-    prompt, everything but the newest R tokens, rounded down to a multiple of the group."""
+    Fixed window (residual_length = R): once the tail holds more than R tokens, flush the oldest
+    floor(R/g)*g; for a prompt, everything but the newest R tokens, rounded down to a multiple of the
+    group.  Under either rule the newest token stays in fp16 (the ratio rule keeps int(ratio * L) >= 1
+    tokens whenever it flushes at all): what a decode step flushes are tokens of earlier steps, which is
+    what lets the flushes of all layers of a step be issued together before its first layer runs
+    (flush_ahead below)."""
     if residual_length is not None:
         if prompt:
             return (max(tail_len - residual_length, 0) // group) * group
-        return (residual_length // group) * group if tail_len >= residual_length else 0
+        return (residual_length // group) * group if tail_len > residual_length else 0
     keep = int(ratio * tail_len)
     if tail_len > keep and keep >= 0:
         return ((tail_len - keep) // group) * group
@@ -120,6 +124,7 @@ class PackedKVCache:
         self._k: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None  # code, scale, min
         self._v: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None
         self._packed_views = (None,) * 6  # views of the quantized part, rebuilt after a flush
+        self._flushed_ahead = False       # flush_ahead() has run the coming one-token append's flush
 
     # -- sizes -----------------------------------------------------------------------------
     def _words(self, n: int, bits: int, fmt: int) -> int:
@@ -193,24 +198,36 @@ class PackedKVCache:
             reserve = steady + 2 * self.Vgroup_size + n
             self._k_tail.append(key_states, reserve)
             self._v_tail.append(value_states, reserve)
-            nk = flush_length(self._k_tail.len, self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
-            nv = flush_length(self._v_tail.len, self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
+            if self._flushed_ahead and n == 1:
+                nk = nv = 0  # (flush_ahead has already run this step's flush)
+            else:
+                nk = flush_length(self._k_tail.len, self.k_residual_ratio, self.Kgroup_size, self.residual_length, prompt)
+                nv = flush_length(self._v_tail.len, self.v_residual_ratio, self.Vgroup_size, self.residual_length, prompt)
+        self._flushed_ahead = False
         self.kv_seq_len += n
         if nk == 0 and nv == 0:
             return
         self._reserve(key_states, nk, nv)
+        ops.quantize_kv_flush_into(*self._flush_args(nk, nv, key_states if direct else None, value_states if direct else None))
+        self._flush_done(nk, nv, direct)
+
+    def _flush_args(self, nk: int, nv: int, k_src=None, v_src=None):
+        """Arguments of ops.quantize_kv_flush_into for flushing nk key and nv value tokens into the packed buffers
+        (already reserved) at the write position: from the front of the tails, or of k_src / v_src."""
         k_out = v_out = None
         k_chunk = v_chunk = None
         if nk > 0:
             w0, g0 = self._words(self.k_tokens, self.k_bits, self.k_fmt), self.k_tokens // self.Kgroup_size
             w1, g1 = self._words(self.k_tokens + nk, self.k_bits, self.k_fmt), (self.k_tokens + nk) // self.Kgroup_size
             k_out = (self._k[0][..., w0:w1], self._k[1][..., g0:g1], self._k[2][..., g0:g1])
-            k_chunk = key_states[:, :, :nk] if direct else self._k_tail.view()[:, :, :nk]
+            k_chunk = (k_src if k_src is not None else self._k_tail.view())[:, :, :nk]
         if nv > 0:
             v_out = tuple(t[:, :, self.v_tokens:self.v_tokens + nv] for t in self._v)
-            v_chunk = value_states[:, :, :nv] if direct else self._v_tail.view()[:, :, :nv]
-        ops.quantize_kv_flush_into(k_chunk, self.Kgroup_size, self.k_bits, k_out, v_chunk, self.Vgroup_size,
-                                   self.v_bits, v_out, self.k_fmt, self.v_fmt)
+            v_chunk = (v_src if v_src is not None else self._v_tail.view())[:, :, :nv]
+        return (k_chunk, self.Kgroup_size, self.k_bits, k_out, v_chunk, self.Vgroup_size, self.v_bits, v_out,
+                self.k_fmt, self.v_fmt)
+
+    def _flush_done(self, nk: int, nv: int, direct: bool) -> None:
         if not direct:
             self._k_tail.drop_front(nk)
             self._v_tail.drop_front(nv)
@@ -227,6 +244,8 @@ class PackedKVCache:
     # -- hooks for a decode step replayed from a captured graph --------------------------------
     def flushes_on_next_append(self) -> bool:
         """Would appending one token make either tail flush?"""
+        if self._flushed_ahead:
+            return False  # (flush_ahead has run it)
         nk = flush_length(self._k_tail.len + 1, self.k_residual_ratio, self.Kgroup_size, self.residual_length)
         nv = flush_length(self._v_tail.len + 1, self.v_residual_ratio, self.Vgroup_size, self.residual_length)
         return nk > 0 or nv > 0
@@ -242,6 +261,7 @@ class PackedKVCache:
         self._k_tail.len += 1
         self._v_tail.len += 1
         self.kv_seq_len += 1
+        self._flushed_ahead = False
 
     def reset(self) -> None:
         """Forget every token; the buffers stay allocated and are reused by the next prompt."""
@@ -251,6 +271,7 @@ class PackedKVCache:
             if tail.buf is not None:
                 tail.buf.zero_()  # window() relies on slots past the live length reading as zero
         self._packed_views = (None,) * 6
+        self._flushed_ahead = False
 
     # -- views -----------------------------------------------------------------------------
     def as_tuple(self) -> Tuple:
@@ -264,3 +285,29 @@ class PackedKVCache:
 
     def __len__(self) -> int:
         return 9
+
+
+def flush_ahead(caches) -> int:
+    """Run now, batched over the caches (kvmix_quant_pack_kv_flush_batch: eight to a launch), the flush that the
+    next ONE-token append of each of them would run, and mark those appends as flushed.  Call it right before a
+    decode step: what a layer flushes in a step are the oldest tokens of its tails, tokens of earlier steps
+    (models/modeling_llama_KVmix.py:122-127,152-156: `[:, :, :to_quantize_length]`), and how many follows from the
+    tails' lengths alone, so nothing of the step itself is needed -- and the packed bits, the tails and every later
+    decision are those of flushing inside the appends (a cache whose rule would take the coming token itself is left
+    to its append).  Returns the number of caches flushed."""
+    todo = []
+    for c in caches:
+        if not isinstance(c, PackedKVCache) or c._k_tail.buf is None or c._flushed_ahead:
+            continue
+        nk = flush_length(c._k_tail.len + 1, c.k_residual_ratio, c.Kgroup_size, c.residual_length)
+        nv = flush_length(c._v_tail.len + 1, c.v_residual_ratio, c.Vgroup_size, c.residual_length)
+        if (nk == 0 and nv == 0) or nk > c._k_tail.len or nv > c._v_tail.len:
+            continue
+        c._reserve(c._k_tail.buf, nk, nv)
+        todo.append((c, nk, nv))
+    if todo:
+        ops.quantize_kv_flush_batch([c._flush_args(nk, nv) for c, nk, nv in todo])
+        for c, nk, nv in todo:
+            c._flush_done(nk, nv, direct=False)
+            c._flushed_ahead = True
+    return len(todo)

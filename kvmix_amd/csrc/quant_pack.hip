@@ -22,6 +22,8 @@
 
 #include "kvmix_common.h"
 
+#include <vector>
+
 namespace kvmix {
 
 #ifndef KVMIX_FLUSH_VALUE_PIECES
@@ -603,43 +605,78 @@ __global__ void __launch_bounds__(128) quant_key_tokens(KeyTokArgs a)
 // The two parts touch disjoint tensors; a launch of this size is latency-bound, so one
 // launch costs about what either part costs alone.
 // ---------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) quant_kv_flush(KeyTokArgs ka, int kmode, int64_t k_groups,
-                                                      int64_t k_threads, unsigned k_blocks, int k_tiled,
-                                                      QuantArgs va, int64_t v_groups_per_row,
-                                                      int64_t v_total_groups)
+// One block of a layer's flush: blocks [0, k_blocks) run the key-token quantizer (slabs where the rows can be tiled,
+// one thread per (group, channel) otherwise), the rest the value quantizer.  `bx`: the block's index within the layer.
+struct FlushItem {
+    KeyTokArgs ka;
+    QuantArgs va;
+    int64_t k_groups, k_threads, v_groups_per_row, v_total_groups;
+    unsigned k_blocks, blocks;  // key blocks; key + value blocks
+    int kmode, k_tiled;
+};
+
+__device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uint16_t *tile)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
-    if (blockIdx.x < k_blocks && k_tiled) {
-        switch (kmode) {
-        case 1: key_tokens_slab_body<32, 1>(ka, k_groups, blockIdx.x, tile); break;
-        case 2: key_tokens_slab_body<32, 2>(ka, k_groups, blockIdx.x, tile); break;
-        case 3: key_tokens_slab_body<11, 3>(ka, k_groups, blockIdx.x, tile); break;
-        case 4: key_tokens_slab_body<32, 4>(ka, k_groups, blockIdx.x, tile); break;
-        default: key_tokens_slab_body<32, 30>(ka, k_groups, blockIdx.x, tile); break;
+    if (bx < f.k_blocks && f.k_tiled) {
+        switch (f.kmode) {
+        case 1: key_tokens_slab_body<32, 1>(f.ka, f.k_groups, bx, tile); break;
+        case 2: key_tokens_slab_body<32, 2>(f.ka, f.k_groups, bx, tile); break;
+        case 3: key_tokens_slab_body<11, 3>(f.ka, f.k_groups, bx, tile); break;
+        case 4: key_tokens_slab_body<32, 4>(f.ka, f.k_groups, bx, tile); break;
+        default: key_tokens_slab_body<32, 30>(f.ka, f.k_groups, bx, tile); break;
         }
-    } else if (blockIdx.x < k_blocks) {
-        const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
-        if (id >= k_threads) return;
+    } else if (bx < f.k_blocks) {
+        const int64_t id = (int64_t)bx * 256 + threadIdx.x;
+        if (id >= f.k_threads) return;
         // (32-bit divisions: the host keeps the thread count below 2^31)
-        const uint32_t id32 = (uint32_t)id, D32 = (uint32_t)ka.D, pair = id32 / D32;
+        const uint32_t id32 = (uint32_t)id, D32 = (uint32_t)f.ka.D, pair = id32 / D32;
         const int64_t d = id32 - pair * D32;
-        const int64_t o = pair / (uint32_t)k_groups, gi = pair - (uint32_t)o * (uint32_t)k_groups;
-        switch (kmode) {
-        case 1: key_tokens_body<32, 1>(ka, gi, o, d); break;
-        case 2: key_tokens_body<32, 2>(ka, gi, o, d); break;
-        case 3: key_tokens_body<11, 3>(ka, gi, o, d); break;
-        case 4: key_tokens_body<32, 4>(ka, gi, o, d); break;
-        default: key_tokens_body<32, 30>(ka, gi, o, d); break;
+        const int64_t o = pair / (uint32_t)f.k_groups, gi = pair - (uint32_t)o * (uint32_t)f.k_groups;
+        switch (f.kmode) {
+        case 1: key_tokens_body<32, 1>(f.ka, gi, o, d); break;
+        case 2: key_tokens_body<32, 2>(f.ka, gi, o, d); break;
+        case 3: key_tokens_body<11, 3>(f.ka, gi, o, d); break;
+        case 4: key_tokens_body<32, 4>(f.ka, gi, o, d); break;
+        default: key_tokens_body<32, 30>(f.ka, gi, o, d); break;
         }
     } else {
-        const int64_t tid = (int64_t)(blockIdx.x - k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
-        switch (va.bits) {
-        case 1: rows_g32_f16_body<1, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
-        default: rows_g32_f16_body<4, kFlushValuePieces, kFlushIdx32>(va, v_groups_per_row, v_total_groups, tid); break;
+        const int64_t tid = (int64_t)(bx - f.k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
+        switch (f.va.bits) {
+        case 1: rows_g32_f16_body<1, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        case 2: rows_g32_f16_body<2, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        case 3: rows_g32_f16_body<3, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        default: rows_g32_f16_body<4, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
         }
     }
+}
+
+__global__ void __launch_bounds__(256) quant_kv_flush(FlushItem f)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
+    flush_block(f, blockIdx.x, tile);
+}
+
+// The flushes of up to kFlushBatch layers in one launch (kvmix_quant_pack_kv_flush_batch): first the key blocks of all
+// layers -- the longer chains of dependent steps -- then the value blocks.  The items travel as kernel arguments.
+constexpr int kFlushBatch = 8;
+struct FlushBatchArgs {
+    FlushItem item[kFlushBatch];
+    unsigned k_first[kFlushBatch + 1];  // first key block of item i among the launch's key blocks
+    unsigned v_first[kFlushBatch + 1];  // first value block of item i among the launch's value blocks
+    int count;
+};
+
+__global__ void __launch_bounds__(256) quant_kv_flush_batch(FlushBatchArgs b)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
+    const unsigned k_all = b.k_first[b.count];
+    const bool key = blockIdx.x < k_all;
+    const unsigned bx = key ? blockIdx.x : blockIdx.x - k_all;
+    const unsigned *first = key ? b.k_first : b.v_first;
+    int i = 0;
+    while (i + 1 < b.count && bx >= first[i + 1]) i++;  // (uniform over the block; at most kFlushBatch - 1 steps)
+    const FlushItem &f = b.item[i];
+    flush_block(f, key ? bx - first[i] : f.k_blocks + (bx - first[i]), tile);
 }
 
 static int64_t gcd64(int64_t a, int64_t b)
@@ -920,42 +957,106 @@ extern "C" int kvmix_quant_pack_key_tokens(const void *k, int64_t outer, int64_t
     return launch_key_tokens(a, mode, groups, outer, (hipStream_t)stream);
 }
 
-extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf,
-                                         kvmix_stream_t stream)
+// Both halves of a layer's flush checked and laid out.  KVMIX_OK with `fused` false: one half is empty or the value
+// half needs the generic quantizer -- the halves then go out as launches of their own.
+struct FlushSetup {
+    FlushItem item;
+    bool kempty, vempty, vfast, fused;
+    int vpw;
+};
+static int setup_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf, FlushSetup &fs)
 {
     if (!kf || !vf) return KVMIX_ERR_NULL;
-    KeyTokArgs ka;
-    QuantArgs va;
-    int kmode = 0, vpw = 0;
-    int64_t kgroups = 0;
-    bool kempty, vempty, vfast;
+    FlushItem &f = fs.item;
     int rc = setup_key_tokens(kf->k, kf->outer, kf->n, kf->D, kf->k_outer_stride, kf->k_token_stride, kf->group,
                               kf->bits, kf->fmt, kf->scale_mode, kf->code, kf->code_outer_stride,
                               kf->code_inner_stride, kf->scale, kf->zero, kf->sz_outer_stride, kf->sz_inner_stride,
-                              ka, kmode, kgroups, kempty);
+                              f.ka, f.kmode, f.k_groups, fs.kempty);
     if (rc != KVMIX_OK) return rc;
     rc = setup_last_dim(vf->x, KVMIX_F16, vf->outer, vf->inner, vf->steps, vf->x_outer_stride, vf->x_inner_stride,
                         vf->group, vf->bits, vf->fmt, vf->scale_mode, vf->code, vf->code_outer_stride,
-                        vf->code_inner_stride, vf->scale, vf->zero, vf->sz_outer_stride, vf->sz_inner_stride, va, vpw,
-                        vempty, vfast);
+                        vf->code_inner_stride, vf->scale, vf->zero, vf->sz_outer_stride, vf->sz_inner_stride, f.va, fs.vpw,
+                        fs.vempty, fs.vfast);
     if (rc != KVMIX_OK) return rc;  // (nothing was launched: both halves are checked first)
+    fs.fused = !(fs.kempty || fs.vempty || !fs.vfast);
+    if (!fs.fused) return KVMIX_OK;
+    // key slab path: D = 128, token rows 16-byte aligned
+    f.k_tiled = key_rows_tileable(f.ka);
+    f.k_threads = f.k_groups * kf->outer * kf->D;
+    const int64_t k_blocks = f.k_tiled ? key_slab_units(f.kmode, kf->outer, f.k_groups) : (f.k_threads + 255) / 256;
+    f.v_groups_per_row = f.va.steps / 32;
+    f.v_total_groups = f.va.outer * f.va.inner * f.v_groups_per_row;
+    const int64_t v_blocks = (f.v_total_groups * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
+    if (k_blocks + v_blocks > 0x7fffffff || f.k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
+    f.k_blocks = (unsigned)k_blocks;
+    f.blocks = (unsigned)(k_blocks + v_blocks);
+    return KVMIX_OK;
+}
+
+// the halves of a flush that cannot share a launch
+static int launch_flush_halves(const kvmix_key_flush_t *kf, const FlushSetup &fs, hipStream_t st)
+{
+    if (!fs.kempty) {
+        const int rc = launch_key_tokens(fs.item.ka, fs.item.kmode, fs.item.k_groups, kf->outer, st);
+        if (rc != KVMIX_OK) return rc;
+    }
+    return fs.vempty ? KVMIX_OK : launch_last_dim(fs.item.va, KVMIX_F16, fs.vpw, fs.vfast, st);
+}
+
+extern "C" int kvmix_quant_pack_kv_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf,
+                                         kvmix_stream_t stream)
+{
+    FlushSetup fs;
+    const int rc = setup_flush(kf, vf, fs);
+    if (rc != KVMIX_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
-    if (kempty || vempty || !vfast) {
-        // one half is empty or the value half needs the generic quantizer: separate launches
-        if (!kempty) {
-            rc = launch_key_tokens(ka, kmode, kgroups, kf->outer, st);
+    if (!fs.fused) return launch_flush_halves(kf, fs, st);
+    hipLaunchKernelGGL(quant_kv_flush, dim3(fs.item.blocks), dim3(256), 0, st, fs.item);
+    return launch_status();
+}
+
+extern "C" int kvmix_quant_pack_kv_flush_batch(const kvmix_key_flush_t *const *kf, const kvmix_value_flush_t *const *vf,
+                                               int count, kvmix_stream_t stream)
+{
+    if (count < 0) return KVMIX_ERR_SHAPE;
+    if (count == 0) return KVMIX_OK;
+    if (!kf || !vf) return KVMIX_ERR_NULL;
+    // every layer is checked before anything is launched
+    std::vector<FlushSetup> fs((size_t)count);
+    for (int i = 0; i < count; i++) {
+        const int rc = setup_flush(kf[i], vf[i], fs[(size_t)i]);
+        if (rc != KVMIX_OK) return rc;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    FlushBatchArgs b;
+    b.count = 0;
+    uint64_t k_blocks = 0, v_blocks = 0;
+    auto flush_launch = [&]() {
+        if (b.count == 0) return KVMIX_OK;
+        b.k_first[b.count] = (unsigned)k_blocks;
+        b.v_first[b.count] = (unsigned)v_blocks;
+        hipLaunchKernelGGL(quant_kv_flush_batch, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, b);
+        b.count = 0;
+        k_blocks = v_blocks = 0;
+        return launch_status();
+    };
+    for (int i = 0; i < count; i++) {
+        const FlushSetup &s = fs[(size_t)i];
+        if (!s.fused) {
+            const int rc = launch_flush_halves(kf[i], s, st);
+            if (rc != KVMIX_OK) return rc;
+            continue;
+        }
+        if (b.count == kFlushBatch || k_blocks + v_blocks + s.item.blocks > 0x7fffffffull) {
+            const int rc = flush_launch();
             if (rc != KVMIX_OK) return rc;
         }
-        return vempty ? KVMIX_OK : launch_last_dim(va, KVMIX_F16, vpw, vfast, st);
+        b.item[b.count] = s.item;
+        b.k_first[b.count] = (unsigned)k_blocks;
+        b.v_first[b.count] = (unsigned)v_blocks;
+        k_blocks += s.item.k_blocks;
+        v_blocks += s.item.blocks - s.item.k_blocks;
+        b.count++;
     }
-    // key slab path: D = 128, token rows 16-byte aligned
-    const int k_tiled = key_rows_tileable(ka);
-    const int64_t k_threads = kgroups * kf->outer * kf->D;
-    const int64_t k_blocks = k_tiled ? key_slab_units(kmode, kf->outer, kgroups) : (k_threads + 255) / 256;
-    const int64_t v_groups = va.steps / 32, v_total = va.outer * va.inner * v_groups;
-    const int64_t v_blocks = (v_total * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
-    if (k_blocks + v_blocks > 0x7fffffff || k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
-    hipLaunchKernelGGL(quant_kv_flush, dim3((unsigned)(k_blocks + v_blocks)), dim3(256), 0, st, ka, kmode, kgroups,
-                       k_threads, (unsigned)k_blocks, k_tiled, va, v_groups, v_total);
-    return launch_status();
+    return flush_launch();
 }

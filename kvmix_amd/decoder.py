@@ -117,6 +117,12 @@ class Decoder:
         if Q > 1:  # causal mask of the prompt, as the model builds it: 0 / dtype-min, fp32 logits
             mask = torch.full((Q, Q), torch.finfo(torch.float32).min, device=x.device, dtype=torch.float32)
             mask = torch.triu(mask, 1)[None, None]
+        if Q == 1:
+            # what the layers would flush in this step are tokens of earlier steps: all layers' flushes in one
+            # batched launch sequence, before the first layer runs (in-place caches; others flush in their append)
+            from .cache import flush_ahead
+
+            flush_ahead(self.caches)
         for li, lw in enumerate(self.w["layers"]):
             h = rms_norm(x, lw["input_norm"], cfg.rms_norm_eps)
             q, k, v = project_qkv(cfg, h, lw["wqkv"], cos, sin)
@@ -155,8 +161,9 @@ class GraphDecoder(Decoder):
     three numbers (the position and the lengths of the two fp16 tails); those live in device
     counters that the graph itself increments, the new token goes to slot `tail length` of a
     fixed-size tail window through an indexed copy, and the attention step reads the tail lengths
-    from the counters, so that the window's unused slots get probability zero.  A step in which some layer flushes runs eagerly (the flush changes the packed
-    lengths, which are launch arguments), after which the graph is captured again.
+    from the counters, so that the window's unused slots get probability zero.  Before a step in which layers flush, the flushes of all
+    layers are run at once (cache.flush_ahead: they take tokens of earlier steps only); the flush changes the packed
+    lengths, which are launch arguments, so that step is captured anew and replayed like the others.
     Needs in-place caches (PackedKVCache) that all follow the same kind of flush policy: one fixed residual window,
     or the reference's ratio rule (models/modeling_llama_KVmix.py:119-127,152-155: residual_length None) -- there the
     tails stay short (a flush every group / (1 - ratio) tokens per layer, every 14 tokens with the reference's
@@ -175,7 +182,7 @@ class GraphDecoder(Decoder):
         self._ids = self._logits = None
         self._pos = self._len = None
         self._counters = {}
-        self.graph_steps = self.eager_steps = self.captures = 0
+        self.graph_steps = self.eager_steps = self.captures = self.flush_steps = 0
 
     # one decode step with static shapes; mutates the device counters
     def _static_step(self, ids: torch.Tensor) -> torch.Tensor:
@@ -278,7 +285,16 @@ class GraphDecoder(Decoder):
         self.captures += 1
 
     def forward(self, input_ids: torch.Tensor) -> torch.Tensor:
+        if input_ids.shape[1] == 1 and self.position > 0 and any(c.flushes_on_next_append() for c in self.caches):
+            # a step in which layers flush: the flushes of all layers now, batched (they take tokens of earlier
+            # steps only); the packed lengths have changed, so the step is captured anew
+            from .cache import flush_ahead
+
+            flush_ahead(self.caches)
+            self._stale = True
+            self.flush_steps += 1
         if input_ids.shape[1] != 1 or self.position == 0 or any(c.flushes_on_next_append() for c in self.caches):
+            # (a prompt, or a cache whose rule takes the coming token itself: the eager loop)
             self._stale = True
             self.eager_steps += 1
             return super().forward(input_ids)

@@ -162,22 +162,19 @@ def quantize_kv_flush(k_chunk: torch.Tensor, k_group: int, k_bits: int, v_chunk:
     return kc, ks, km, vc, vs, vm
 
 
-def quantize_kv_flush_into(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v_group: int, v_bits: int, v_out,
-                           k_fmt: int = _lib.FMT_REF, v_fmt: int = _lib.FMT_REF) -> None:
-    """quantize_kv_flush writing into tensors the caller owns: k_out = (code [B,H,D,n/vpw],
-    scale, min [B,H,D,n/g]) and v_out = (code [B,H,nv,D/vpw], scale, min [B,H,nv,D/g]) may be
-    slices of larger pre-allocated cache buffers (unit stride along the last dimension, (B, H)
-    collapsible).  Either half may be None (k_chunk and k_out, or v_chunk and v_out)."""
-    import ctypes
-
-    L = _lib.load()
+def _flush_descriptors(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v_group: int, v_bits: int, v_out,
+                       k_fmt: int = _lib.FMT_REF, v_fmt: int = _lib.FMT_REF):
+    """The (KeyFlush, ValueFlush, tensors to keep alive) of one flush, or None when there is nothing to do.  Keys in
+    groups the token-major key kernel does not take (other than 32, or 11 for the reference's 3 bits) are quantized
+    here and now through the one-shot quantizer; the key descriptor then stays empty."""
     kf, vf = _lib.KeyFlush(), _lib.ValueFlush()
     kf.group, kf.bits, kf.fmt, kf.scale_mode = max(k_group, 1), k_bits, k_fmt, _lib.SCALE_RECIPROCAL
     vf.group, vf.bits, vf.fmt, vf.scale_mode = max(v_group, 1), v_bits, v_fmt, _lib.SCALE_RECIPROCAL
     ref = k_chunk if k_chunk is not None else v_chunk
     if ref is None:
-        return
+        return None
     _need_gpu(ref)
+    keep = [ref]
 
     def out_strides(code, scale, mn, B, H):
         for t in (code, scale, mn):
@@ -202,6 +199,7 @@ def quantize_kv_flush_into(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v
             kf.code, kf.code_outer_stride, kf.code_inner_stride = kc.data_ptr(), kc.stride(1), kc.stride(2)
             kf.scale, kf.zero = ks.data_ptr(), km.data_ptr()
             kf.sz_outer_stride, kf.sz_inner_stride = ks.stride(1), ks.stride(2)
+            keep += [k_chunk, kc, ks, km]
     if v_chunk is not None and v_chunk.shape[2] > 0:
         Bv, Hv, nv, Dv = v_chunk.shape
         v_chunk, vo, vi = _rows3(v_chunk)
@@ -212,8 +210,40 @@ def quantize_kv_flush_into(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v
         vf.code, vf.code_outer_stride, vf.code_inner_stride = vc.data_ptr(), vc.stride(1), vc.stride(2)
         vf.scale, vf.zero = vs.data_ptr(), vm.data_ptr()
         vf.sz_outer_stride, vf.sz_inner_stride = vs.stride(1), vs.stride(2)
-    with torch.cuda.device(ref.device):
-        _lib.check(L.kvmix_quant_pack_kv_flush(ctypes.byref(kf), ctypes.byref(vf), _stream(ref)))
+        keep += [v_chunk, vc, vs, vm]
+    return kf, vf, keep
+
+
+def quantize_kv_flush_into(k_chunk, k_group: int, k_bits: int, k_out, v_chunk, v_group: int, v_bits: int, v_out,
+                           k_fmt: int = _lib.FMT_REF, v_fmt: int = _lib.FMT_REF) -> None:
+    """quantize_kv_flush writing into tensors the caller owns: k_out = (code [B,H,D,n/vpw],
+    scale, min [B,H,D,n/g]) and v_out = (code [B,H,nv,D/vpw], scale, min [B,H,nv,D/g]) may be
+    slices of larger pre-allocated cache buffers (unit stride along the last dimension, (B, H)
+    collapsible).  Either half may be None (k_chunk and k_out, or v_chunk and v_out)."""
+    import ctypes
+
+    d = _flush_descriptors(k_chunk, k_group, k_bits, k_out, v_chunk, v_group, v_bits, v_out, k_fmt, v_fmt)
+    if d is None:
+        return
+    kf, vf, keep = d
+    with torch.cuda.device(keep[0].device):
+        _lib.check(_lib.load().kvmix_quant_pack_kv_flush(ctypes.byref(kf), ctypes.byref(vf), _stream(keep[0])))
+
+
+def quantize_kv_flush_batch(flushes) -> None:
+    """The flushes of several caches at once (kvmix_quant_pack_kv_flush_batch: eight to a launch): `flushes` is a
+    sequence of argument tuples of quantize_kv_flush_into, all on one device; the results are those of calling it
+    on each tuple, bit for bit.  What a decode step flushes are the oldest tokens of the fp16 tails
+    (models/modeling_llama_KVmix.py:122-127,152-156), so a caller can issue the flushes of all layers of a step
+    together before its first layer runs."""
+    ds = [d for d in (_flush_descriptors(*f) for f in flushes) if d is not None]
+    if not ds:
+        return
+    dev = ds[0][2][0].device
+    if any(d[2][0].device != dev for d in ds):
+        raise RuntimeError("the flushes of one batch must be on one device")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.flush_batch([d[0] for d in ds], [d[1] for d in ds], _stream(ds[0][2][0])))
 
 
 def _batched3(t: torch.Tensor) -> Tuple[torch.Tensor, int, int]:

@@ -468,7 +468,7 @@ def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_rat
     q [B,nh,1,D] f16; k_new, v_new [B,nh_kv,1,D] f16; cache = the reference's 9-tuple
     (Kcode, K_tail, Kscale, Kmin, Vcode, V_tail, Vscale, Vmin, kv_seq_len), entries may
     be None.  Returns (attn_output [B,nh,1,D] f16, probs f16, new cache).
-    fixed_window=R replaces the ratio rule by: when the tail reaches R tokens, flush
+    fixed_window=R replaces the ratio rule by: when the tail holds more than R tokens, flush
     floor(R/g)*g of the oldest ones (the benchmark's fixed residual window).
     k_dense3 / v_dense3 (with 3 bits): that side is kept in the dense 3-bit stream -- an
     extension without reference counterpart -- in groups of group_size; the flow around the
@@ -493,7 +493,7 @@ def attention_decode_step(q, k_new, v_new, cache, k_bits, v_bits, k_ratio, v_rat
 
     def n_flush(tail_len, ratio, g):
         if fixed_window is not None:
-            return (fixed_window // g) * g if tail_len >= fixed_window else 0
+            return (fixed_window // g) * g if tail_len > fixed_window else 0
         return flush_length(tail_len, ratio, g)
 
     nk = n_flush(k_tail.shape[2], k_ratio, kg)

@@ -76,6 +76,18 @@ def test_host_validation_needs_no_gpu(lib):
     assert g(*gargs(g=4)) == -9     # a word of eight 4-bit codes would straddle two groups
     assert lib.kvmix_gemv_workspace_bytes(32, 1, 4096, 128) > 0
     assert lib.kvmix_gemv_workspace_bytes(0, 1, 4096, 128) == 0
+    # the batched flush: every pair is checked before anything is launched
+    from kvmix_amd import _lib
+
+    fb = lib.kvmix_quant_pack_kv_flush_batch
+    assert fb(None, None, 0, None) == 0 and fb(None, None, -1, None) == -8 and fb(None, None, 2, None) == -7
+    good_k = _lib.KeyFlush(16, 1, 32, 128, 4096, 128, 32, 4, 0, 0, 16, 512, 4, 16, 16, 128, 1)
+    good_v = _lib.ValueFlush(16, 1, 32, 128, 4096, 128, 32, 4, 0, 0, 16, 512, 16, 16, 16, 128, 4)
+    bad_v = _lib.ValueFlush(16, 1, 32, 128, 4096, 128, 32, 5, 0, 0, 16, 512, 16, 16, 16, 128, 4)   # 5 bits
+    assert _lib.flush_batch([good_k, good_k], [good_v, bad_v], None) == -1
+    ka = (ctypes.POINTER(_lib.KeyFlush) * 2)(ctypes.pointer(good_k), None)
+    va = (ctypes.POINTER(_lib.ValueFlush) * 2)(ctypes.pointer(good_v), ctypes.pointer(good_v))
+    assert fb(ka, va, 2, None) == -7                                                                 # a pair without its key half
 
 
 def test_decode_attention_host_validation_needs_no_gpu(lib):

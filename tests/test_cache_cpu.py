@@ -19,9 +19,10 @@ def test_ratio_rule_hand_worked():
 
 
 def test_fixed_window_rule():
-    assert flush_length(127, 0.0, 32, residual_length=128) == 0
-    assert flush_length(128, 0.0, 32, residual_length=128) == 128
-    assert flush_length(129, 0.0, 11, residual_length=129) == 121
+    assert flush_length(128, 0.0, 32, residual_length=128) == 0
+    assert flush_length(129, 0.0, 32, residual_length=128) == 128   # the newest token stays in fp16
+    assert flush_length(129, 0.0, 11, residual_length=129) == 0
+    assert flush_length(130, 0.0, 11, residual_length=129) == 121
     assert flush_length(1000, 0.0, 32, residual_length=128, prompt=True) == 864  # (1000 - 128) // 32 * 32
     assert flush_length(100, 0.0, 32, residual_length=128, prompt=True) == 0
 

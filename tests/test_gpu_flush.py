@@ -122,3 +122,87 @@ def test_flush_with_group_64_keys_when_both_tails_flush(dev=None):
     ovc, ovs, ovm = O.quantize_pack_last_dim(v_np, 64, 2)
     for got, want in zip((kc, ks, km, vc, vs, vm), (oc, osc, omn, ovc, ovs, ovm)):
         assert same_bits(got.cpu().numpy(), want)
+
+
+def test_batched_flush_matches_the_flushes_one_by_one():
+    """kvmix_quant_pack_kv_flush_batch over 19 caches of mixed formats and sizes (three launches of eight, eight and
+    three; two pairs that cannot share a launch -- an empty key half, a value group of 64 -- in between): every
+    output bit for bit what quantize_kv_flush_into writes for the same pair."""
+    from kvmix_amd import ops
+
+    gen = torch.Generator(device="cuda").manual_seed(19)
+    specs = []
+    for i in range(19):
+        k_bits = (4, 2, 3, 1, 3)[i % 5]
+        v_bits = (2, 3, 4, 1)[i % 4]
+        kg = 11 if k_bits == 3 else 32
+        B, H, D = (2, 4, 128) if i % 3 else (1, 3, 64)
+        nk = kg * (1 + i % 4) if i != 5 else 0          # (pair 5: nothing to flush on the key side)
+        nv = 32 * (1 + i % 3)
+        vg = 64 if i == 11 else 32                      # (pair 11: a value group the fused launch does not take)
+        specs.append((k_bits, v_bits, kg, vg, B, H, D, nk, nv))
+
+    def outputs(spec):
+        k_bits, v_bits, kg, vg, B, H, D, nk, nv = spec
+        kw = nk // 11 if k_bits == 3 else nk * k_bits // 32
+        vw = D * 3 // 32 if v_bits == 3 else D * v_bits // 32
+        z = lambda *s, dt=torch.float16: torch.zeros(*s, dtype=dt, device="cuda")
+        return ((z(B, H, D, kw, dt=torch.int32), z(B, H, D, nk // kg), z(B, H, D, nk // kg)),
+                (z(B, H, nv, vw, dt=torch.int32), z(B, H, nv, D // vg), z(B, H, nv, D // vg)))
+
+    args_one, args_batch, outs_one, outs_batch = [], [], [], []
+    for spec in specs:
+        k_bits, v_bits, kg, vg, B, H, D, nk, nv = spec
+        k = torch.randn(B, H, nk, D, device="cuda", generator=gen).half()
+        v = torch.randn(B, H, nv, D, device="cuda", generator=gen).half()
+        v_fmt = ops.FMT_DENSE3 if v_bits == 3 else ops.FMT_REF
+        for args, outs in ((args_one, outs_one), (args_batch, outs_batch)):
+            ko, vo = outputs(spec)
+            outs.append(ko + vo)
+            args.append((k if nk else None, kg, k_bits, ko if nk else None, v, vg, v_bits, vo, ops.FMT_REF, v_fmt))
+    for a in args_one:
+        ops.quantize_kv_flush_into(*a)
+    ops.quantize_kv_flush_batch(args_batch)
+    torch.cuda.synchronize()
+    for i, (one, batch) in enumerate(zip(outs_one, outs_batch)):
+        for a, b in zip(one, batch):
+            assert torch.equal(a, b), (i, specs[i])
+        assert i == 5 or one[0].abs().sum() > 0          # (something was written)
+
+
+@pytest.mark.parametrize("policy", ["window", "ratio"])
+def test_flush_ahead_leaves_the_caches_as_flushing_inside_the_appends_does(policy):
+    """cache.flush_ahead before every one-token append against caches that flush inside their appends: the
+    reference's 9-tuple bit for bit after every one of 200 steps, for five caches of mixed formats under the fixed
+    window and under the reference's ratio rule (where the five flush at different steps)."""
+    from kvmix_amd import ops
+    from kvmix_amd.cache import PackedKVCache, flush_ahead
+
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    kinds = [(4, 4, ops.FMT_REF), (2, 3, ops.FMT_DENSE3), (3, 2, ops.FMT_REF), (1, 4, ops.FMT_REF), (3, 3, ops.FMT_DENSE3)]
+    kw = dict(residual_length=64) if policy == "window" else {}
+
+    def make():
+        return [PackedKVCache(kb, vb, capacity=512, v_fmt=vf, **kw) for kb, vb, vf in kinds]
+
+    plain, ahead = make(), make()
+    B, H, D = 2, 4, 128
+    prompt = [(torch.randn(B, H, 150, D, device="cuda", generator=gen).half(), torch.randn(B, H, 150, D, device="cuda", generator=gen).half())
+              for _ in kinds]
+    for group in (plain, ahead):
+        for c, (k, v) in zip(group, prompt):
+            c.append(k, v, prompt=True)
+    flushed = 0
+    for step in range(200):
+        new = [(torch.randn(B, H, 1, D, device="cuda", generator=gen).half(), torch.randn(B, H, 1, D, device="cuda", generator=gen).half())
+               for _ in kinds]
+        flushed += flush_ahead(ahead)
+        assert not any(c.flushes_on_next_append() for c in ahead)
+        for group in (plain, ahead):
+            for c, (k, v) in zip(group, new):
+                c.append(k, v)
+        for i, (a, b) in enumerate(zip(plain, ahead)):
+            assert (a.k_tokens, a.v_tokens, a.kv_seq_len) == (b.k_tokens, b.v_tokens, b.kv_seq_len), (step, i)
+            for x, y in zip(a.as_tuple()[:8], b.as_tuple()[:8]):
+                assert (x is None) == (y is None) and (x is None or torch.equal(x, y)), (step, i)
+    assert flushed >= 10
