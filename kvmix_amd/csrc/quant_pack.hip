@@ -613,8 +613,10 @@ struct FlushItem {
     int64_t k_groups, k_threads, v_groups_per_row, v_total_groups;
     unsigned k_blocks, blocks;  // key blocks; key + value blocks
     int kmode, k_tiled;
+    int v_stream;               // value half: one thread per group, two groups a thread (rows_g32_f16_stream_body)
 };
 
+template <bool STREAM>  // (the streaming value form needs more registers: only the batched kernel carries it)
 __device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uint16_t *tile)
 {
     if (bx < f.k_blocks && f.k_tiled) {
@@ -639,6 +641,14 @@ __device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uin
         case 4: key_tokens_body<32, 4>(f.ka, gi, o, d); break;
         default: key_tokens_body<32, 30>(f.ka, gi, o, d); break;
         }
+    } else if (STREAM && f.v_stream) {
+        const int64_t first = (int64_t)(bx - f.k_blocks) * 512 + threadIdx.x;
+        switch (f.va.bits) {
+        case 1: rows_g32_f16_stream_body<1, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 2: rows_g32_f16_stream_body<2, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 3: rows_g32_f16_stream_body<3, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        default: rows_g32_f16_stream_body<4, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        }
     } else {
         const int64_t tid = (int64_t)(bx - f.k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
         switch (f.va.bits) {
@@ -653,12 +663,19 @@ __device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uin
 __global__ void __launch_bounds__(256) quant_kv_flush(FlushItem f)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
-    flush_block(f, blockIdx.x, tile);
+    flush_block<false>(f, blockIdx.x, tile);
 }
 
 // The flushes of up to kFlushBatch layers in one launch (kvmix_quant_pack_kv_flush_batch): first the key blocks of all
 // layers -- the longer chains of dependent steps -- then the value blocks.  The items travel as kernel arguments.
 constexpr int kFlushBatch = 8;
+#ifndef KVMIX_FLUSH_BATCH_OCC
+#define KVMIX_FLUSH_BATCH_OCC 4  // waves per SIMD the compiler plans for (107 registers; capped at 5 or 6 it spills: 206 -> 214 -> 250 us)
+#endif
+#ifndef KVMIX_FLUSH_STREAM_GROUPS
+#define KVMIX_FLUSH_STREAM_GROUPS 16384
+#endif
+constexpr int64_t kFlushStreamGroups = KVMIX_FLUSH_STREAM_GROUPS;  // value groups of a pair from which on its half streams
 struct FlushBatchArgs {
     FlushItem item[kFlushBatch];
     unsigned k_first[kFlushBatch + 1];  // first key block of item i among the launch's key blocks
@@ -666,7 +683,8 @@ struct FlushBatchArgs {
     int count;
 };
 
-__global__ void __launch_bounds__(256) quant_kv_flush_batch(FlushBatchArgs b)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KVMIX_FLUSH_BATCH_OCC)))
+quant_kv_flush_batch(FlushBatchArgs b)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kKeySlabTile];
     const unsigned k_all = b.k_first[b.count];
@@ -676,7 +694,7 @@ __global__ void __launch_bounds__(256) quant_kv_flush_batch(FlushBatchArgs b)
     int i = 0;
     while (i + 1 < b.count && bx >= first[i + 1]) i++;  // (uniform over the block; at most kFlushBatch - 1 steps)
     const FlushItem &f = b.item[i];
-    flush_block(f, key ? bx - first[i] : f.k_blocks + (bx - first[i]), tile);
+    flush_block<true>(f, key ? bx - first[i] : f.k_blocks + (bx - first[i]), tile);
 }
 
 static int64_t gcd64(int64_t a, int64_t b)
@@ -964,7 +982,7 @@ struct FlushSetup {
     bool kempty, vempty, vfast, fused;
     int vpw;
 };
-static int setup_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf, FlushSetup &fs)
+static int setup_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *vf, FlushSetup &fs, bool batched = false)
 {
     if (!kf || !vf) return KVMIX_ERR_NULL;
     FlushItem &f = fs.item;
@@ -986,7 +1004,12 @@ static int setup_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *v
     const int64_t k_blocks = f.k_tiled ? key_slab_units(f.kmode, kf->outer, f.k_groups) : (f.k_threads + 255) / 256;
     f.v_groups_per_row = f.va.steps / 32;
     f.v_total_groups = f.va.outer * f.va.inner * f.v_groups_per_row;
-    const int64_t v_blocks = (f.v_total_groups * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
+    // A flush alone is a latency-bound launch and wants many small threads (four to a group); in a batch of layers
+    // the value half is a streaming kernel and takes the prompt quantizer's form, a thread per group, two groups a
+    // thread (measured, the 32 flushes of a step in four launches: 222.8 -> 206.7 us).
+    f.v_stream = batched && f.v_total_groups >= kFlushStreamGroups && f.v_groups_per_row < (1ll << 31) ? 1 : 0;
+    const int64_t v_blocks = f.v_stream ? (f.v_total_groups + 511) / 512
+                                        : (f.v_total_groups * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
     if (k_blocks + v_blocks > 0x7fffffff || f.k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
     f.k_blocks = (unsigned)k_blocks;
     f.blocks = (unsigned)(k_blocks + v_blocks);
@@ -1024,7 +1047,7 @@ extern "C" int kvmix_quant_pack_kv_flush_batch(const kvmix_key_flush_t *const *k
     // every layer is checked before anything is launched
     std::vector<FlushSetup> fs((size_t)count);
     for (int i = 0; i < count; i++) {
-        const int rc = setup_flush(kf[i], vf[i], fs[(size_t)i]);
+        const int rc = setup_flush(kf[i], vf[i], fs[(size_t)i], true);
         if (rc != KVMIX_OK) return rc;
     }
     hipStream_t st = (hipStream_t)stream;

@@ -206,3 +206,36 @@ def test_flush_ahead_leaves_the_caches_as_flushing_inside_the_appends_does(polic
             for x, y in zip(a.as_tuple()[:8], b.as_tuple()[:8]):
                 assert (x is None) == (y is None) and (x is None or torch.equal(x, y)), (step, i)
     assert flushed >= 10
+
+
+def test_batched_flush_of_large_value_halves_streams_and_matches():
+    """Pairs with 16384 value groups or more take the streaming form of the value quantizer inside the batched launch
+    (one thread per group): four pairs of the bench step's size, one per value bit width, against the flushes one by
+    one."""
+    from kvmix_amd import ops
+
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    B, H, D, n = 8, 32, 128, 128
+    one, batch, outs = [], [], []
+    for v_bits, k_bits in ((1, 4), (2, 3), (3, 2), (4, 1)):
+        kg = 11 if k_bits == 3 else 32
+        nk = n // kg * kg
+        k = torch.randn(B, H, nk, D, device="cuda", generator=gen).half()
+        v = (torch.randn(B, H, n, D, device="cuda", generator=gen) * 3).half()
+        v_fmt = ops.FMT_DENSE3 if v_bits == 3 else ops.FMT_REF
+        for args in (one, batch):
+            kw = nk // 11 if k_bits == 3 else nk * k_bits // 32
+            vw = D * 3 // 32 if v_bits == 3 else D * v_bits // 32
+            ko = (torch.zeros(B, H, D, kw, dtype=torch.int32, device="cuda"), torch.zeros(B, H, D, nk // kg, dtype=torch.float16, device="cuda"),
+                  torch.zeros(B, H, D, nk // kg, dtype=torch.float16, device="cuda"))
+            vo = (torch.zeros(B, H, n, vw, dtype=torch.int32, device="cuda"), torch.zeros(B, H, n, D // 32, dtype=torch.float16, device="cuda"),
+                  torch.zeros(B, H, n, D // 32, dtype=torch.float16, device="cuda"))
+            args.append((k, kg, k_bits, ko, v, 32, v_bits, vo, ops.FMT_REF, v_fmt))
+            outs.append(ko + vo)
+    for a in one:
+        ops.quantize_kv_flush_into(*a)
+    ops.quantize_kv_flush_batch(batch)
+    torch.cuda.synchronize()
+    for i in range(0, len(outs), 2):
+        for a, b in zip(outs[i], outs[i + 1]):
+            assert torch.equal(a, b) and a.abs().sum() > 0, i // 2
