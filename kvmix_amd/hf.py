@@ -120,6 +120,12 @@ class KVmixCache(Cache):
     def packed(self, layer_idx: int) -> PackedKVCache:
         return self.layers[layer_idx].packed
 
+    def flush_ahead(self) -> int:
+        """Run now, batched, the flushes the coming one-token step would run layer by layer (cache.flush_ahead)."""
+        from .cache import flush_ahead
+
+        return flush_ahead([layer.packed for layer in self.layers])
+
     def to_legacy_tuple(self, layer_idx: int):
         """The reference's 9-entry tuple for one layer (models/modeling_llama_KVmix.py:270-273), as views."""
         return self.layers[layer_idx].packed.as_tuple()
@@ -165,6 +171,10 @@ class _KVmixAttentionForward:
             elif attention_mask.dtype != mask_dtype:
                 attention_mask = attention_mask.clamp(min=torch.finfo(mask_dtype).min).to(mask_dtype)
         packed = None if past_key_values is None else past_key_values.packed(self.layer_idx)
+        if packed is not None and q_len == 1 and self.layer_idx == 0:
+            # a decode step: what its layers flush are tokens of earlier steps -- all layers' flushes at once,
+            # batched, before the first layer runs (cache.flush_ahead)
+            past_key_values.flush_ahead()
         attn_output, attn_weights, _ = self.kvmix(query_states, key_states, value_states, packed,
                                                   attention_mask=attention_mask, use_cache=packed is not None,
                                                   need_weights=bool(kwargs.get("output_attentions", False)))
