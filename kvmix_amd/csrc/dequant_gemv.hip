@@ -61,10 +61,22 @@ constexpr int kMaxDevices = 64;  // per-device set-up state is kept for device o
 // Measured constants of the dispatch (MI355X: 256 CUs x 4 SIMDs).  tests/test_gemv_plan_cpu.py pins the kernel
 // each benchmark shape ends up with.
 constexpr int kTargetWaves = 4096;          // 16 waves on each of 256 CUs
-constexpr int kCols3HeadsU = 4;             // gemv_cols3, four heads per pass: rows in flight per lane
+#ifndef KVMIX_COLS3_HEADS_U
+#define KVMIX_COLS3_HEADS_U 4
+#endif
+#ifndef KVMIX_COLS3_HEADS_OCC
+#define KVMIX_COLS3_HEADS_OCC 2
+#endif
+constexpr int kCols3HeadsU = KVMIX_COLS3_HEADS_U;   // gemv_cols3, four heads per pass: rows in flight per lane
 constexpr int kCols3U = 8;                  // gemv_cols3, one head per pass: rows in flight per lane
-constexpr int kCols3HeadsOcc = 2;           // waves per SIMD the compiler may plan for: gemv_cols3, four heads
-constexpr int kMfmaHeadsOcc = 2;            // ... gemv_rows_mfma / gemv_cols_mfma, four heads
+constexpr int kCols3HeadsOcc = KVMIX_COLS3_HEADS_OCC;   // waves per SIMD the compiler may plan for: gemv_cols3, four heads
+#ifndef KVMIX_MFMA_HEADS_OCC
+#define KVMIX_MFMA_HEADS_OCC 2
+#endif
+#ifndef KVMIX_ROWS_HEADS_PACK
+#define KVMIX_ROWS_HEADS_PACK 1
+#endif
+constexpr int kMfmaHeadsOcc = KVMIX_MFMA_HEADS_OCC;   // ... gemv_rows_mfma / gemv_cols_mfma, four heads
 constexpr int kMfma2Occ = 2;                // ... gemv_cols_mfma2 (at least; it comes out at three)
 constexpr int kHeadsWaveDiv = 2;            // p.V, four heads per pass: half as many waves wanted
 constexpr int kMfma2MaxWaves = kTargetWaves;    // two-element matrix-core q.K^T kernel up to this many tiles
@@ -1168,7 +1180,41 @@ __device__ __forceinline__ float field_sum(float cur, float prev, int f)
     return f > 0 ? cur - prev : cur;
 }
 
-constexpr int rows_mfma_sets(int nrep) { return (3 * nrep + 3) / 4; }
+// bf16 parts x*scale*2^90 is split into.  One query head: three (24 significant bits hold the product of two fp16
+// exactly, and three rows fit one MFMA anyway).  Four heads per pass: two parts, rounded to nearest after 16
+// significant bits (every product off by at most 2^-17 of itself, either way: far inside the fp16 rounding of the
+// output; cutting off instead leaves all products of a p.V too small, which sums), so that the eight (head, part)
+// rows are two MFMAs per B operand instead of three and a third of the staging goes.
+#ifndef KVMIX_HEADS_PARTS
+#define KVMIX_HEADS_PARTS 2
+#endif
+constexpr int rows_mfma_parts(int nrep) { return nrep > 1 ? KVMIX_HEADS_PARTS : 3; }   // p.V: 128 rows or more, x = probabilities
+constexpr int cols_mfma_parts(int) { return 3; }                                        // q.K^T: exact at any K
+constexpr int mfma_sets(int parts, int nrep) { return (parts * nrep + 3) / 4; }
+constexpr int rows_mfma_sets(int nrep) { return mfma_sets(rows_mfma_parts(nrep), nrep); }
+constexpr int cols_mfma_sets(int nrep) { return mfma_sets(cols_mfma_parts(nrep), nrep); }
+// v (= x*scale*2^90) as NP bf16, part i in the high half of part[i]: all but the last by truncation (the
+// remainders are exact); the last holds what is left exactly when NP = 3 and is rounded to nearest otherwise
+// (a carry into the exponent is the next power of two, as it should be; v is far from overflow)
+template <int NP>
+__device__ __forceinline__ void split_bf16_parts(float v, uint32_t *part)
+{
+#pragma unroll
+    for (int i = 0; i + 1 < NP; i++) {
+        part[i] = __float_as_uint(v) & 0xffff0000u;
+        v -= __uint_as_float(part[i]);
+    }
+    part[NP - 1] = NP >= 3 ? __float_as_uint(v) : __float_as_uint(v) + 0x8000u;
+}
+// the sum over the parts' accumulators of head h at code position p
+template <int NP, int NM, int NPOS>
+__device__ __forceinline__ float parts_sum(const f32x4_t (&acc)[NM][NPOS], int h, int p)
+{
+    float s = acc[(NP * h) / 4][p][(NP * h) % 4];
+#pragma unroll
+    for (int i = 1; i < NP; i++) s += acc[(NP * h + i) / 4][p][(NP * h + i) % 4];
+    return s;
+}
 constexpr int kRowsMfmaTile = (32 * 17 + 1) * 4 + 4;  // bf16 elements of one A tile (32 skewed rows), 8-byte multiple
 
 constexpr int kRowsMfmaWaves = 16;  // waves per block at most (register budget of 128 per lane)
@@ -1188,6 +1234,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     constexpr int CH = 128;            // rows per chunk: 512 scales = one 128-bit load per lane
     constexpr int KB = CH / RKB;       // k-blocks per chunk (8)
     constexpr int AT = kRowsMfmaTile;  // bf16 elements of one A tile
+    constexpr int NP = rows_mfma_parts(NREP); // bf16 parts of x*scale
     constexpr int NM = rows_mfma_sets(NREP);  // MFMAs per B operand
     constexpr int NPOS = 8;            // code positions per lane
     constexpr int FPB = 8 / FB;        // whole fields per byte window
@@ -1263,7 +1310,12 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     // DEPTH chunks are in flight per wave: register set d holds chunk c with c % DEPTH == d
     Half8 s8[DEPTH], z8[DEPTH];
     Half2x xh[DEPTH][NREP];
-    Elem w[DEPTH][KB][4];
+    // four heads, 1 and 2 bits: the elements of two rows share a register (16-bit halves, loaded in place), which
+    // is what brings the kernel under the register count of three waves per SIMD
+    constexpr bool PK = NREP > 1 && sizeof(Elem) <= 2 && KVMIX_ROWS_HEADS_PACK;
+    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+    Elem w[PK ? 1 : DEPTH][PK ? 1 : KB][4];
+    u16x2_t wp[PK ? DEPTH : 1][PK ? KB : 1][2];
 
     auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : max(ke32 - CH, 0); };
     auto load_small = [&](int d, int k0) {
@@ -1276,8 +1328,13 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     auto load_codes = [&](int d, int k0, int t) {
         const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-            w[d][t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
+        for (int k = 0; k < 4; k++) {
+            const Elem e = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
+            if constexpr (PK)
+                wp[d][t][k / 2][k % 2] = (uint16_t)e;
+            else
+                w[d][t][k] = e;
+        }
     };
     auto stage = [&](int d, int k0) {
         const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
@@ -1288,16 +1345,12 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
                 const int q = e / LPR, g = e % LPR;
                 const float xv = row0 + q >= skip ? h16_to_f32(xh[d][h].v[q]) : 0.f;
                 zacc[h][g] = fmaf(xv, h16_to_f32(z8[d].v[e]), zacc[h][g]);
-                // x * scale * 2^90, split into three bf16 by truncation (exact)
-                const float v0 = (xv * 1237940039285380274899124224.0f) * h16_to_f32(s8[d].v[e]);
-                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
-                const float v1 = v0 - __uint_as_float(b0);
-                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
-                const float v2 = v1 - __uint_as_float(b1);
-                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+                // x * scale * 2^90, split into bf16 parts by truncation (three parts: exact)
+                uint32_t part[NP];
+                split_bf16_parts<NP>((xv * 1237940039285380274899124224.0f) * h16_to_f32(s8[d].v[e]), part);
 #pragma unroll
-                for (int pt = 0; pt < 3; pt++) {  // A row 3h+pt: MFMA (3h+pt)/4, lanes 4g + (3h+pt)%4
-                    const int ar = 3 * h + pt;
+                for (int pt = 0; pt < NP; pt++) {  // A row NP*h+pt: MFMA (NP*h+pt)/4, lanes 4g + (NP*h+pt)%4
+                    const int ar = NP * h + pt;
                     atile[(ar / 4) * AT + aoff[q] + g * 16 + (ar % 4) * 4] = (uint16_t)(part[pt] >> 16);
                 }
             }
@@ -1347,9 +1400,17 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
 #pragma unroll
             for (int b = 0; b < EB; b++) {
                 // byte b of rows k and k+1 -> low bytes of the two halves
-                const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
-                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+                uint32_t t01, t23;
+                if constexpr (PK) {
+                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(2 + b) << 16);
+                    const uint32_t w01 = __builtin_bit_cast(uint32_t, wp[d][t][0]), w23 = __builtin_bit_cast(uint32_t, wp[d][t][1]);
+                    t01 = EB == 1 ? w01 : __builtin_amdgcn_perm(w01, w01, sel);  // (one byte per element: already in place)
+                    t23 = EB == 1 ? w23 : __builtin_amdgcn_perm(w23, w23, sel);
+                } else {
+                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+                    t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
+                    t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+                }
 #pragma unroll
                 for (int f = 0; f < FPB; f++) {
                     const bf16x4_t bv =
@@ -1428,8 +1489,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
         float sums[NPOS];
 #pragma unroll
         for (int p = 0; p < NPOS; p++)
-            sums[p] = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
-                      acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
+            sums[p] = parts_sum<NP>(acc, h, p);
 #pragma unroll
         for (int p = 0; p < NPOS; p++) {
             // (bit offset of code p's field in its byte: dense 3-bit 0 3 2 5 0 3 2 5, else FB * (p % FPB))
@@ -1493,7 +1553,8 @@ __global__ void __launch_bounds__(64 * kColsWaves)
     constexpr int CH = 32;             // rows per chunk
     constexpr int KB = CH / 4;         // MFMA k-steps per chunk
     constexpr int AT = kColsMfmaTile;
-    constexpr int NM = rows_mfma_sets(NREP);
+    constexpr int NP = cols_mfma_parts(NREP);
+    constexpr int NM = cols_mfma_sets(NREP);
     constexpr int NPOS = 8;
     constexpr int FPB = 8 / BITS;
     constexpr int TG = 16;             // groups per tile
@@ -1585,15 +1646,11 @@ __global__ void __launch_bounds__(64 * kColsWaves)
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 zacc[h][j] = fmaf(xv, h16_to_f32(z8.v[j]), zacc[h][j]);
-                const float v0 = x2 * h16_to_f32(s8.v[j]);  // split into three bf16 by truncation (exact)
-                const uint32_t b0 = __float_as_uint(v0) & 0xffff0000u;
-                const float v1 = v0 - __uint_as_float(b0);
-                const uint32_t b1 = __float_as_uint(v1) & 0xffff0000u;
-                const float v2 = v1 - __uint_as_float(b1);
-                const uint32_t part[3] = {b0, b1, __float_as_uint(v2)};
+                uint32_t part[NP];
+                split_bf16_parts<NP>(x2 * h16_to_f32(s8.v[j]), part);  // (three parts: exact)
 #pragma unroll
-                for (int pt = 0; pt < 3; pt++) {  // A row 3h+pt: MFMA (3h+pt)/4, lanes 4g + (3h+pt)%4
-                    const int ar = 3 * h + pt;
+                for (int pt = 0; pt < NP; pt++) {  // A row NP*h+pt: MFMA (NP*h+pt)/4, lanes 4g + (NP*h+pt)%4
+                    const int ar = NP * h + pt;
                     atile[(ar / 4) * AT + aoff + (4 * j + ar % 4) * 4] = (uint16_t)(part[pt] >> 16);
                 }
             }
@@ -1643,8 +1700,7 @@ __global__ void __launch_bounds__(64 * kColsWaves)
             float sums[NPOS];
 #pragma unroll
             for (int p = 0; p < NPOS; p++)
-                sums[p] = (acc[(3 * h) / 4][p][(3 * h) % 4] + acc[(3 * h + 1) / 4][p][(3 * h + 1) % 4]) +
-                          acc[(3 * h + 2) / 4][p][(3 * h + 2) % 4];
+                sums[p] = parts_sum<NP>(acc, h, p);
 #pragma unroll
             for (int p = 0; p < NPOS; p++) {
                 const float sum = field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
@@ -3054,7 +3110,7 @@ static void launch_cols_mfma(GemvArgs &a, int64_t samples, hipStream_t st)
     const int wpb = pick_waves_per_block(slots);
     a.splits = (int)tpw;
     const dim3 grid((unsigned)((slots + wpb - 1) / wpb), (unsigned)(samples / NREP), (unsigned)a.M);
-    const size_t lds = (size_t)wpb * (rows_mfma_sets(NREP) * kColsMfmaTile * sizeof(uint16_t) + NREP * 16 * sizeof(float));
+    const size_t lds = (size_t)wpb * (cols_mfma_sets(NREP) * kColsMfmaTile * sizeof(uint16_t) + NREP * 16 * sizeof(float));
     KVMIX_LAUNCH((gemv_cols_mfma<BITS, NREP>), grid, dim3(kWave, wpb), lds, st, a, "gemv_cols_mfma<%d,%d>", BITS, NREP);
 }
 
