@@ -73,9 +73,6 @@ constexpr int kCols3HeadsOcc = KVMIX_COLS3_HEADS_OCC;   // waves per SIMD the co
 #ifndef KVMIX_MFMA_HEADS_OCC
 #define KVMIX_MFMA_HEADS_OCC 2
 #endif
-#ifndef KVMIX_ROWS_HEADS_PACK
-#define KVMIX_ROWS_HEADS_PACK 1
-#endif
 constexpr int kMfmaHeadsOcc = KVMIX_MFMA_HEADS_OCC;   // ... gemv_rows_mfma / gemv_cols_mfma, four heads
 constexpr int kMfma2Occ = 2;                // ... gemv_cols_mfma2 (at least; it comes out at three)
 constexpr int kHeadsWaveDiv = 2;            // p.V, four heads per pass: half as many waves wanted
@@ -1310,12 +1307,7 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     // DEPTH chunks are in flight per wave: register set d holds chunk c with c % DEPTH == d
     Half8 s8[DEPTH], z8[DEPTH];
     Half2x xh[DEPTH][NREP];
-    // four heads, 1 and 2 bits: the elements of two rows share a register (16-bit halves, loaded in place), which
-    // is what brings the kernel under the register count of three waves per SIMD
-    constexpr bool PK = NREP > 1 && sizeof(Elem) <= 2 && KVMIX_ROWS_HEADS_PACK;
-    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
-    Elem w[PK ? 1 : DEPTH][PK ? 1 : KB][4];
-    u16x2_t wp[PK ? DEPTH : 1][PK ? KB : 1][2];
+    Elem w[DEPTH][KB][4];
 
     auto chunk_base = [&](int k0) { return k0 + CH <= ke32 ? k0 : max(ke32 - CH, 0); };
     auto load_small = [&](int d, int k0) {
@@ -1328,13 +1320,8 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
     auto load_codes = [&](int d, int k0, int t) {
         const uint8_t *base = cp + (uint32_t)(chunk_base(k0) + rs) * (EPR * EB);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const Elem e = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
-            if constexpr (PK)
-                wp[d][t][k / 2][k % 2] = (uint16_t)e;
-            else
-                w[d][t][k] = e;
-        }
+        for (int k = 0; k < 4; k++)
+            w[d][t][k] = ld_stream<Elem>(base + (t * RKB + RL * k) * (EPR * EB));
     };
     auto stage = [&](int d, int k0) {
         const int skip = k0 - chunk_base(k0);  // rows of this chunk that an earlier one covered
@@ -1400,17 +1387,9 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
 #pragma unroll
             for (int b = 0; b < EB; b++) {
                 // byte b of rows k and k+1 -> low bytes of the two halves
-                uint32_t t01, t23;
-                if constexpr (PK) {
-                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(2 + b) << 16);
-                    const uint32_t w01 = __builtin_bit_cast(uint32_t, wp[d][t][0]), w23 = __builtin_bit_cast(uint32_t, wp[d][t][1]);
-                    t01 = EB == 1 ? w01 : __builtin_amdgcn_perm(w01, w01, sel);  // (one byte per element: already in place)
-                    t23 = EB == 1 ? w23 : __builtin_amdgcn_perm(w23, w23, sel);
-                } else {
-                    const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-                    t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
-                    t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
-                }
+                const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
+                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
+                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
 #pragma unroll
                 for (int f = 0; f < FPB; f++) {
                     const bf16x4_t bv =
