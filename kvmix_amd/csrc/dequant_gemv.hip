@@ -50,6 +50,18 @@
 #ifndef KVMIX_COLS_NT_CODES
 #define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal (the matrix-core kernels: 2 and 4 bits only -- a wave's 1-bit row piece is 64 or 128 bytes and shares its cache lines with the neighbours')
 #endif
+#ifndef KVMIX_SLAB3_NT_CODES
+#define KVMIX_SLAB3_NT_CODES KVMIX_COLS_NT_CODES  // attention step, reference 3-bit keys: codes / scales and zeros non-temporal
+#endif
+#ifndef KVMIX_SLAB3_NT_SZ
+#define KVMIX_SLAB3_NT_SZ 1
+#endif
+#ifndef KVMIX_SLAB_BARRIER
+#define KVMIX_SLAB_BARRIER 1   // attention step, 1/2/4-bit keys: one s_barrier per 16-row chunk of the key phase
+#endif
+#ifndef KVMIX_SLAB3_BARRIER
+#define KVMIX_SLAB3_BARRIER 1  // ... one s_barrier per step of the key phase
+#endif
 #ifndef KVMIX_COLS3_NT_SZ
 #define KVMIX_COLS3_NT_SZ 1  // q.K^T, reference 3-bit words, one head per pass: scales and zeros (as large as the codes) non-temporal
 #endif
@@ -2384,6 +2396,8 @@ __device__ __forceinline__ void attn_slab_mfma_body(const AttnSlabArgs &a, int64
 #pragma unroll 1
         for (int it = it0; it < it1; it++) {
             const int nx = it + 1 < it1 ? it + 1 : it;
+            // (as in gemv_cols_mfma2: the block's waves, on neighbouring tiles of the same rows, kept in step)
+            if constexpr (!COOP && KVMIX_SLAB_BARRIER) __builtin_amdgcn_s_barrier();
             stage();
             wave_lds_fence();
             load_small(nx);
@@ -2572,9 +2586,9 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
         const int row0 = COOP ? wy * (K / kColsWaves) : 0;
         uint32_t co = unit0 * 4u + (uint32_t)row0 * c_step, so = unit0 * 2u + (uint32_t)row0 * s_step;
         auto next_row = [&](int u) {
-            cw[u] = ld_stream<Words<UPL>, KVMIX_COLS_NT_CODES>(cb + co);
-            sw[u] = ld_stream<Half2x, KVMIX_COLS3_NT_SZ>(sb + so);
-            zw[u] = ld_stream<Half2x, KVMIX_COLS3_NT_SZ>(zb + so);
+            cw[u] = ld_stream<Words<UPL>, KVMIX_SLAB3_NT_CODES>(cb + co);
+            sw[u] = ld_stream<Half2x, KVMIX_SLAB3_NT_SZ>(sb + so);
+            zw[u] = ld_stream<Half2x, KVMIX_SLAB3_NT_SZ>(zb + so);
             co += c_step;
             so += s_step;
         };
@@ -2608,6 +2622,11 @@ __device__ __forceinline__ void attn_slab_ref3_body(const AttnSlabArgs &a, int64
 #pragma unroll
             for (int u = 0; u < U; u++) xr[u] = xs[row0 + st * U + u];
             __builtin_amdgcn_sched_barrier(0);
+            // the block's waves -- neighbouring tiles of the same rows -- stay in step: a row piece does not end on a
+            // cache line, and the line two tiles share is then fetched from memory once (measured, 2-bit values, us:
+            // B = 8 72.2 -> 68.6, B = 16 141.2 -> 134.2).  A wave whose tile lies past the row has left: the barrier
+            // counts the waves that remain
+            if constexpr (!COOP && KVMIX_SLAB3_BARRIER) __builtin_amdgcn_s_barrier();
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 compute_row(u);
