@@ -1189,16 +1189,18 @@ __device__ __forceinline__ float field_sum(float cur, float prev, int f)
     return f > 0 ? cur - prev : cur;
 }
 
-// bf16 parts x*scale*2^90 is split into.  One query head: three (24 significant bits hold the product of two fp16
-// exactly, and three rows fit one MFMA anyway).  Four heads per pass: two parts, rounded to nearest after 16
-// significant bits (every product off by at most 2^-17 of itself, either way: far inside the fp16 rounding of the
-// output; cutting off instead leaves all products of a p.V too small, which sums), so that the eight (head, part)
-// rows are two MFMAs per B operand instead of three and a third of the staging goes.
+// bf16 parts x*scale*2^90 is split into: three (24 significant bits hold the product of two fp16 exactly).  One
+// query head: its three rows fit one MFMA.  Four heads per pass: twelve rows, three MFMAs per B operand.
+// KVMIX_HEADS_PARTS = 2 (measurement only; p.V kernel) rounds the second part to nearest instead -- every product off
+// by up to 2^-17 of itself, eight rows, two MFMAs per B operand, a third of the staging gone: 2-bit p.V at B = 16,
+// 32 / 8 heads, T = 32768 70 -> 55 us.  Not shipped: where the code term and the zero term of an output nearly cancel
+// (a peaked probability row on a value near zero) that error comes on top of the two sums' fp32 rounding and took a
+// 4-bit case at K = 128 from 0.65 to 1.4 times the GEMV tolerance (tests/test_gpu_gemv.py holds the case).
 #ifndef KVMIX_HEADS_PARTS
-#define KVMIX_HEADS_PARTS 2
+#define KVMIX_HEADS_PARTS 3
 #endif
-constexpr int rows_mfma_parts(int nrep) { return nrep > 1 ? KVMIX_HEADS_PARTS : 3; }   // p.V: 128 rows or more, x = probabilities
-constexpr int cols_mfma_parts(int) { return 3; }                                        // q.K^T: exact at any K
+constexpr int rows_mfma_parts(int nrep) { return nrep > 1 ? KVMIX_HEADS_PARTS : 3; }   // p.V
+constexpr int cols_mfma_parts(int) { return 3; }                                        // q.K^T
 constexpr int mfma_sets(int parts, int nrep) { return (parts * nrep + 3) / 4; }
 constexpr int rows_mfma_sets(int nrep) { return mfma_sets(rows_mfma_parts(nrep), nrep); }
 constexpr int cols_mfma_sets(int nrep) { return mfma_sets(cols_mfma_parts(nrep), nrep); }

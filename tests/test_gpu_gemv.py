@@ -90,6 +90,60 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
     run_case(oracle, dev, bits, g, B=1, nh=4, nkv=4, K=777, N=128, seed=45, M=2)
 
 
+@pytest.mark.parametrize("nkv", [2, 8])
+@pytest.mark.parametrize("bits", [4, 2, 1])
+def test_pv_with_probability_rows(oracle, dev, bits, nkv):
+    """p.V with four query heads per kv head, and one, and probabilities as x -- flat, peaked and one-hot rows -- against
+    float64.  With x >= 0 the code term sum p*scale*code and the zero term sum p*zero of an output are large and of
+    opposite sign where the values straddle zero; the kernels sum the two separately in fp32, so an output in which
+    they cancel carries the rounding of both sums, which the reference's element-wise (code*scale + zero) does not.
+    Tolerance, stated: the library's general one (1e-3 relative + 2e-5 of sum |terms|) plus 2^-18 of the code term's
+    magnitude; the one-hot row -- one product, no sum -- has to meet the general tolerance alone, which it does
+    because x*scale goes to the matrix cores in three bf16 parts that hold the product exactly (two parts, measured
+    faster for four heads per pass and not shipped, are off by up to 2^-17 of every product)."""
+    import KVmix
+    from helpers import GEMV_ABS_TERM, GEMV_RTOL
+
+    g, B, nh, N = 32, 2, 8, 128
+    for K, seed in ((128, 1), (1000, 2), (4096, 3)):
+        rng = np.random.default_rng(100 * bits + seed)
+        w = kv_like(rng, (B, nkv, K, N), outlier_axis=2, n_outliers=2)
+        code, scale, zero = oracle.quantize_pack_last_dim(w, g, bits)
+        logits = rng.standard_normal((B, nh, 1, K)) * np.array([0.1, 1.0, 4.0, 12.0] * 2).reshape(1, nh, 1, 1)
+        x = np.exp(logits - logits.max(-1, keepdims=True))
+        x = (x / x.sum(-1, keepdims=True)).astype(np.float16)
+        x[0, 0, 0, :] = 0
+        x[0, 0, 0, K // 3] = 1  # one-hot: the output is one dequantized row
+        _, want64, abs64 = oracle.quantized_gemm(g, x, code, scale, zero, bits, want_f64=True)
+        _lib_plan_heads(g, bits, B, nh, nkv, K, N)
+        got = KVmix.quantized_gemm(g, tt(x, dev), tt(code, dev), tt(scale, dev), tt(zero, dev), bits).cpu().numpy()
+        ok, worst = gemv_close(got[0, 0], want64[0, 0], abs64[0, 0])
+        assert ok, ("one-hot row, general tolerance", bits, K, worst)
+        # sum over tokens of p * scale * code, per (batch, head, dim)
+        codes = unpack_codes_np(code, bits)                                     # [B, nkv, K, N]
+        sc = np.repeat(scale.astype(np.float64), g, axis=-1)                    # [B, nkv, K, N]
+        terms = np.repeat(sc * codes, nh // nkv, axis=1)                        # [B, nh, K, N]
+        mag = np.einsum("bhk,bhkn->bhn", x[:, :, 0, :].astype(np.float64), terms)[:, :, None, :]
+        tol = GEMV_RTOL * np.abs(want64) + GEMV_ABS_TERM * abs64 + 2.0 ** -18 * mag
+        err = np.abs(got.astype(np.float64) - want64)
+        assert (err <= tol).all(), (bits, K, float((err / tol).max()))
+
+
+def _lib_plan_heads(g, bits, B, nh, nkv, K, N):
+    from kvmix_amd import _lib
+
+    plan = _lib.gemv_plan(g, bits, 0, B * nh, nh // nkv, 1, K, N)
+    assert plan["kernel"].startswith("gemv_rows_mfma<%d,%d," % (bits, 4 if nh // nkv == 4 else 1)), plan
+
+
+def unpack_codes_np(code, bits):
+    """[..., W] packed int32 words -> [..., W * 32 / bits] codes (code i of a word at bit i * bits)."""
+    w = code.astype(np.int64) & 0xFFFFFFFF
+    per = 32 // bits
+    out = np.stack([(w >> (bits * i)) & ((1 << bits) - 1) for i in range(per)], axis=-1)
+    return out.reshape(code.shape[:-1] + (code.shape[-1] * per,)).astype(np.float64)
+
+
 def test_reference_3bit_kernel_edges(oracle, dev):
     """gemv_cols3: four and two words per lane, GQA head groups (four query heads per pass), K ragged
     against the 8-row rotation, N ragged against the tile, M = 2."""
