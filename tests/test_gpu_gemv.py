@@ -93,14 +93,18 @@ def test_matrix_core_kernel_edges(oracle, dev, bits, g):
 @pytest.mark.parametrize("nkv", [2, 8])
 @pytest.mark.parametrize("bits", [4, 2, 1])
 def test_pv_with_probability_rows(oracle, dev, bits, nkv):
-    """p.V with four query heads per kv head, and one, and probabilities as x -- flat, peaked and one-hot rows -- against
-    float64.  With x >= 0 the code term sum p*scale*code and the zero term sum p*zero of an output are large and of
-    opposite sign where the values straddle zero; the kernels sum the two separately in fp32, so an output in which
-    they cancel carries the rounding of both sums, which the reference's element-wise (code*scale + zero) does not.
-    Tolerance, stated: the library's general one (1e-3 relative + 2e-5 of sum |terms|) plus 2^-18 of the code term's
-    magnitude; the one-hot row -- one product, no sum -- has to meet the general tolerance alone, which it does
-    because x*scale goes to the matrix cores in three bf16 parts that hold the product exactly (two parts, measured
-    faster for four heads per pass and not shipped, are off by up to 2^-17 of every product)."""
+    """p.V with four query heads per kv head, and one, and probabilities as x -- flat, peaked and one-hot rows --
+    against float64.  With x >= 0 the code term sum p*scale*code and the zero term sum p*zero of an output are large
+    and of opposite sign where the values straddle zero, and the kernels form the two separately (the reference adds
+    code*scale + zero per element first).  The code term comes from the matrix cores with the codes as subnormal
+    bf16 patterns, and a sum of four such products keeps fewer bits than fp32 when the patterns have leading zeros
+    (measured with a probe: one product exact, four products off by up to 2^-17 of their sum; the low fields of a
+    2-bit byte are the worst).  A row with one dominant probability shows that against an output in which the two
+    terms cancel.  Tolerance, stated: the library's general one (1e-3 relative + 2e-5 of sum |terms|) plus 2^-18 of
+    the code term's magnitude (worst seen without it: 1.7 times the general tolerance, on one 2-bit output of
+    -0.0007 between terms of +-2.28).  The one-hot row -- one product, no sum -- has to meet the general tolerance
+    alone: x*scale goes in as three bf16 parts that hold the product exactly (two parts, measured faster for four
+    heads per pass and not shipped, are off by up to 2^-17 of every product)."""
     import KVmix
     from helpers import GEMV_ABS_TERM, GEMV_RTOL
 
