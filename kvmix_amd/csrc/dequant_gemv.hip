@@ -47,6 +47,9 @@
 #ifndef KVMIX_STREAM_NT
 #define KVMIX_STREAM_NT 1  // non-temporal loads for the packed operands
 #endif
+#ifndef KVMIX_ROWS_RAW_PERM
+#define KVMIX_ROWS_RAW_PERM 1
+#endif
 #ifndef KVMIX_COLS_NT_CODES
 #define KVMIX_COLS_NT_CODES 1  // q.K^T kernels: codes non-temporal (the matrix-core kernels: 2 and 4 bits only -- a wave's 1-bit row piece is 64 or 128 bytes and shares its cache lines with the neighbours')
 #endif
@@ -1151,6 +1154,22 @@ __global__ void __launch_bounds__(NREP > 1 ? 64 * kRowsHeadsWaves : 64 * kRowsMa
 typedef short bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+// v_perm_b32 of two elements of one, two or four bytes.  Two-byte elements go in as they sit in their registers
+// (as half-precision operands: an integer operand of 16 bits would be extended first): the selectors used here
+// never pick a byte above the element, and written in C++ the compiler zero-extends a narrow value that lives
+// across loop iterations again at every use (one v_and_b32 per element and k-block).
+template <typename T>
+__device__ __forceinline__ uint32_t perm_elems(T hi, T lo, uint32_t sel)
+{
+    if constexpr (sizeof(T) != 2 || !KVMIX_ROWS_RAW_PERM) {
+        return __builtin_amdgcn_perm((uint32_t)hi, (uint32_t)lo, sel);
+    } else {
+        uint32_t r;
+        asm("v_perm_b32 %0, %1, %2, %3" : "=v"(r) : "v"(__builtin_bit_cast(_Float16, hi)), "v"(__builtin_bit_cast(_Float16, lo)), "s"(sel));
+        return r;
+    }
+}
+
 template <int BITS>
 struct CodeElem;
 template <>
@@ -1187,6 +1206,45 @@ __device__ __forceinline__ uint32_t field_operand(uint32_t t, int f)
 __device__ __forceinline__ float field_sum(float cur, float prev, int f)
 {
     return f > 0 ? cur - prev : cur;
+}
+// The same two with the low fields moved up in their byte (p.V kernels).  The matrix cores align the four
+// products of a sum by their operands' exponent fields, which all byte patterns share, so a pattern with leading
+// zeros leaves that many fewer bits for a sum its product dominates -- a row of probabilities with one large entry
+// (measured with a probe: one product exact, four off by up to 2^-17 of their sum; with the fields in place a
+// 2-bit p.V then carries 18 bits of the dominant product, which shows where code term and zero term cancel).
+#ifndef KVMIX_ROWS_FIELDS_TOP
+#define KVMIX_ROWS_FIELDS_TOP 1
+#endif
+// bits the fields 0..f are moved up by: the fields of the low nibble by four, so that one shifted copy of the
+// register serves them all and no operand of a dominant product has more than three leading zeros (1-bit codes;
+// two for 2-bit codes, none for 4-bit codes) where in place it has up to seven (six, four)
+template <int BITS>
+__device__ __forceinline__ constexpr int field_shift(int f)
+{
+    return BITS * (f + 1) <= 4 ? 4 : 0;
+}
+template <int BITS>
+__device__ __forceinline__ uint32_t field_operand_top(uint32_t t, int f)
+{
+    constexpr int FPB = 8 / BITS;
+    if (f == FPB - 1) return t;
+    const int sh = field_shift<BITS>(f);
+    const uint32_t mask = ((1u << (BITS * (f + 1))) - 1u) * 0x00010001u;
+    return sh > 0 ? (t << sh) & (mask << sh) : t & mask;
+}
+// sum of field f alone, counting 2^(BITS * f + field_shift(f))-fold
+template <int BITS>
+__device__ __forceinline__ float field_sum_top(float cur, float prev, int f)
+{
+    if (f == 0) return cur;
+    const int d = field_shift<BITS>(f - 1) - field_shift<BITS>(f);  // prev counts 2^d-fold against cur
+    return fmaf(prev, -1.0f / (float)(1 << d), cur);
+}
+// bit offset field f of a byte counts with
+template <int BITS>
+__device__ __forceinline__ constexpr int field_offset_top(int f)
+{
+    return BITS * f + field_shift<BITS>(f);
 }
 
 // bf16 parts x*scale*2^90 is split into: three (24 significant bits hold the product of two fp16 exactly).  One
@@ -1407,12 +1465,13 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
             for (int b = 0; b < EB; b++) {
                 // byte b of rows k and k+1 -> low bytes of the two halves
                 const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[d][t][1], (uint32_t)w[d][t][0], sel);
-                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[d][t][3], (uint32_t)w[d][t][2], sel);
+                const uint32_t t01 = perm_elems(w[d][t][1], w[d][t][0], sel);
+                const uint32_t t23 = perm_elems(w[d][t][3], w[d][t][2], sel);
 #pragma unroll
                 for (int f = 0; f < FPB; f++) {
-                    const bf16x4_t bv =
-                        __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
+                    const bf16x4_t bv = __builtin_bit_cast(
+                        bf16x4_t, KVMIX_ROWS_FIELDS_TOP ? make_uint2(field_operand_top<FB>(t01, f), field_operand_top<FB>(t23, f))
+                                                        : make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
 #pragma unroll
                     for (int q = 0; q < NM; q++)
                         acc[q][b * FPB + f] =
@@ -1491,8 +1550,10 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
 #pragma unroll
         for (int p = 0; p < NPOS; p++) {
             // (bit offset of code p's field in its byte: dense 3-bit 0 3 2 5 0 3 2 5, else FB * (p % FPB))
-            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
-            const float sum = BITS == 30 ? sums[p] : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
+            const float sum = BITS == 30 ? sums[p]
+                              : KVMIX_ROWS_FIELDS_TOP ? field_sum_top<FB>(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB)
+                                                      : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
             flat[h * NPOS + p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
         }
     }
@@ -2170,12 +2231,13 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
 #pragma unroll
             for (int b = 0; b < EB; b++) {
                 const uint32_t sel = 0x0c000c00u | (uint32_t)b | ((uint32_t)(4 + b) << 16);
-                const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)w[t][1], (uint32_t)w[t][0], sel);
-                const uint32_t t23 = __builtin_amdgcn_perm((uint32_t)w[t][3], (uint32_t)w[t][2], sel);
+                const uint32_t t01 = perm_elems(w[t][1], w[t][0], sel);
+                const uint32_t t23 = perm_elems(w[t][3], w[t][2], sel);
 #pragma unroll
                 for (int f = 0; f < FPB; f++) {
-                    const bf16x4_t bv =
-                        __builtin_bit_cast(bf16x4_t, make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
+                    const bf16x4_t bv = __builtin_bit_cast(
+                        bf16x4_t, KVMIX_ROWS_FIELDS_TOP ? make_uint2(field_operand_top<FB>(t01, f), field_operand_top<FB>(t23, f))
+                                                        : make_uint2(field_operand<FB>(t01, f), field_operand<FB>(t23, f)));
                     acc[b * FPB + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[b * FPB + f], 0, 0, 0);
                 }
             }
@@ -2221,8 +2283,10 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
     for (int p = 0; p < NPOS; p++) sums[p] = (acc[p][0] + acc[p][1]) + acc[p][2];
 #pragma unroll
     for (int p = 0; p < NPOS; p++) {
-        const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : FB * (p % FPB);
-        const float sum = BITS == 30 ? sums[p] : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
+        const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
+        const float sum = BITS == 30 ? sums[p]
+                          : KVMIX_ROWS_FIELDS_TOP ? field_sum_top<FB>(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB)
+                                                  : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
         flat[p] = sum * __uint_as_float((uint32_t)(127 + 43 - off) << 23);
     }
     const int first = scatter_reduce<NPOS, 16, 1>(flat, lane);  // two of the lane's eight columns are left
