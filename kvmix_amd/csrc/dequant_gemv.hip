@@ -1447,11 +1447,15 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
                 const uint32_t *src = from_u ? u : v;
                 const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
                 const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
-                const int o0 = mm % 2 == 0 ? 0 : 2;  // bit offset of the pair's first field in its byte
+                // bit offset of the pair's first field in its byte: 0 or 2; a pair at 0 is moved up by two (see
+                // field_operand_top: its first field would have five leading zeros)
+                constexpr bool UP = KVMIX_ROWS_FIELDS_TOP;
+                const uint32_t s01 = UP && mm % 2 == 0 ? t01 << 2 : t01, s23 = UP && mm % 2 == 0 ? t23 << 2 : t23;
+                const int o0 = UP || mm % 2 != 0 ? 2 : 0;
 #pragma unroll
                 for (int f = 0; f < 2; f++) {
                     const uint32_t mask = 0x00070007u << (o0 + 3 * f);
-                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(s01 & mask, s23 & mask));
 #pragma unroll
                     for (int q = 0; q < NM; q++)
                         acc[q][mm * 2 + f] =
@@ -1547,8 +1551,9 @@ __global__ void __launch_bounds__(64 * (NREP > 1 ? kRowsHeadsWaves : kRowsMfmaWa
             sums[p] = parts_sum<NP>(acc, h, p);
 #pragma unroll
         for (int p = 0; p < NPOS; p++) {
-            // (bit offset of code p's field in its byte: dense 3-bit 0 3 2 5 0 3 2 5, else FB * (p % FPB))
-            const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
+            // (bit offset code p's field counts with: dense 3-bit 2 5 2 5 2 5 2 5 -- in its byte 0 3 2 5 0 3 2 5, the pairs at
+            // 0 moved up by two --, else see field_offset_top)
+            const int off = BITS == 30 ? 3 * (p % 2) + (KVMIX_ROWS_FIELDS_TOP ? 2 : 2 * ((p / 2) % 2)) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
             const float sum = BITS == 30 ? sums[p]
                               : KVMIX_ROWS_FIELDS_TOP ? field_sum_top<FB>(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB)
                                                       : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);
@@ -2217,11 +2222,13 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
                 const uint32_t *src = from_u ? u : v;
                 const uint32_t t01 = __builtin_amdgcn_perm(src[1], src[0], sel);
                 const uint32_t t23 = __builtin_amdgcn_perm(src[3], src[2], sel);
-                const int o0 = mm % 2 == 0 ? 0 : 2;
+                constexpr bool UP = KVMIX_ROWS_FIELDS_TOP;  // (a pair at bit 0 is moved up by two, as in gemv_rows_mfma)
+                const uint32_t s01 = UP && mm % 2 == 0 ? t01 << 2 : t01, s23 = UP && mm % 2 == 0 ? t23 << 2 : t23;
+                const int o0 = UP || mm % 2 != 0 ? 2 : 0;
 #pragma unroll
                 for (int f = 0; f < 2; f++) {
                     const uint32_t mask = 0x00070007u << (o0 + 3 * f);
-                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(t01 & mask, t23 & mask));
+                    const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, make_uint2(s01 & mask, s23 & mask));
                     acc[mm * 2 + f] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc[mm * 2 + f], 0, 0, 0);
                 }
             }
@@ -2281,7 +2288,7 @@ __device__ __forceinline__ void slab_value_phase(const AttnSlabArgs &a, int64_t 
     for (int p = 0; p < NPOS; p++) sums[p] = (acc[p][0] + acc[p][1]) + acc[p][2];
 #pragma unroll
     for (int p = 0; p < NPOS; p++) {
-        const int off = BITS == 30 ? 3 * (p % 2) + 2 * ((p / 2) % 2) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
+        const int off = BITS == 30 ? 3 * (p % 2) + (KVMIX_ROWS_FIELDS_TOP ? 2 : 2 * ((p / 2) % 2)) : (KVMIX_ROWS_FIELDS_TOP ? field_offset_top<FB>(p % FPB) : FB * (p % FPB));
         const float sum = BITS == 30 ? sums[p]
                           : KVMIX_ROWS_FIELDS_TOP ? field_sum_top<FB>(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB)
                                                   : field_sum(sums[p], sums[p > 0 ? p - 1 : 0], p % FPB);

@@ -63,6 +63,30 @@ def test_gemv_matches_oracle(oracle, dev, K, N, B, nh, nkv):
     assert ok, worst
 
 
+@pytest.mark.parametrize("nkv", [2, 8])
+def test_pv_with_probability_rows(oracle, dev, nkv):
+    """p.V over dense 3-bit values with probabilities as x (flat, peaked and one-hot rows; four query heads per kv
+    head, and one): the case of tests/test_gpu_gemv.py::test_pv_with_probability_rows, in which the code term and
+    the zero term of an output cancel, within the same general tolerance (the field pairs that sit at bit 0 of
+    their byte are moved up by two before they become matrix-core operands)."""
+    from kvmix_amd import ops
+
+    B, nh, N = 2, 8, 128
+    for K, seed in ((128, 1), (1000, 2), (4096, 3)):
+        rng = np.random.default_rng(300 + seed)
+        w = kv_like(rng, (B, nkv, K, N), outlier_axis=2, n_outliers=2)
+        code, scale, zero = oracle.quantize_pack_dense3(w, 32)
+        logits = rng.standard_normal((B, nh, 1, K)) * np.array([0.1, 1.0, 4.0, 12.0] * 2).reshape(1, nh, 1, 1)
+        x = np.exp(logits - logits.max(-1, keepdims=True))
+        x = (x / x.sum(-1, keepdims=True)).astype(np.float16)
+        x[0, 0, 0, :] = 0
+        x[0, 0, 0, K // 3] = 1
+        _, want64, abs64 = oracle.quantized_gemm_dense3(32, x, code, scale, zero, want_f64=True)
+        got = ops.quantized_gemm(32, tt(x, dev), tt(code, dev), tt(scale, dev), tt(zero, dev), 3, fmt=ops.FMT_DENSE3)
+        ok, worst = gemv_close(got.cpu().numpy(), want64, abs64)
+        assert ok, (nkv, K, worst)
+
+
 def test_one_hot_row_is_exact(oracle, dev):
     from kvmix_amd import ops
 
