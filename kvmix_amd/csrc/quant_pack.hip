@@ -616,49 +616,56 @@ struct FlushItem {
     int v_stream;               // value half: one thread per group, two groups a thread (rows_g32_f16_stream_body)
 };
 
+// One case of a switch over the formats, kept apart from its siblings: the value passes through an empty asm, so the
+// compiler cannot merge the cases' common heads above the switch -- merged, the batched kernel needs 107 registers
+// where its largest case alone needs 77 (four waves per SIMD instead of six).
+#define KVMIX_CASE_V(var) asm volatile("" : "+v"(var))
+#define KVMIX_CASE_S(var) asm volatile("" : "+s"(var))
 template <bool STREAM>  // (the streaming value form needs more registers: only the batched kernel carries it)
 __device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uint16_t *tile)
 {
     if (bx < f.k_blocks && f.k_tiled) {
         switch (f.kmode) {
-        case 1: key_tokens_slab_body<32, 1>(f.ka, f.k_groups, bx, tile); break;
-        case 2: key_tokens_slab_body<32, 2>(f.ka, f.k_groups, bx, tile); break;
-        case 3: key_tokens_slab_body<11, 3>(f.ka, f.k_groups, bx, tile); break;
-        case 4: key_tokens_slab_body<32, 4>(f.ka, f.k_groups, bx, tile); break;
-        default: key_tokens_slab_body<32, 30>(f.ka, f.k_groups, bx, tile); break;
+        case 1: KVMIX_CASE_S(bx); key_tokens_slab_body<32, 1>(f.ka, f.k_groups, bx, tile); break;
+        case 2: KVMIX_CASE_S(bx); key_tokens_slab_body<32, 2>(f.ka, f.k_groups, bx, tile); break;
+        case 3: KVMIX_CASE_S(bx); key_tokens_slab_body<11, 3>(f.ka, f.k_groups, bx, tile); break;
+        case 4: KVMIX_CASE_S(bx); key_tokens_slab_body<32, 4>(f.ka, f.k_groups, bx, tile); break;
+        default: KVMIX_CASE_S(bx); key_tokens_slab_body<32, 30>(f.ka, f.k_groups, bx, tile); break;
         }
     } else if (bx < f.k_blocks) {
         const int64_t id = (int64_t)bx * 256 + threadIdx.x;
         if (id >= f.k_threads) return;
         // (32-bit divisions: the host keeps the thread count below 2^31)
         const uint32_t id32 = (uint32_t)id, D32 = (uint32_t)f.ka.D, pair = id32 / D32;
-        const int64_t d = id32 - pair * D32;
+        int64_t d = id32 - pair * D32;
         const int64_t o = pair / (uint32_t)f.k_groups, gi = pair - (uint32_t)o * (uint32_t)f.k_groups;
         switch (f.kmode) {
-        case 1: key_tokens_body<32, 1>(f.ka, gi, o, d); break;
-        case 2: key_tokens_body<32, 2>(f.ka, gi, o, d); break;
-        case 3: key_tokens_body<11, 3>(f.ka, gi, o, d); break;
-        case 4: key_tokens_body<32, 4>(f.ka, gi, o, d); break;
-        default: key_tokens_body<32, 30>(f.ka, gi, o, d); break;
+        case 1: KVMIX_CASE_V(d); key_tokens_body<32, 1>(f.ka, gi, o, d); break;
+        case 2: KVMIX_CASE_V(d); key_tokens_body<32, 2>(f.ka, gi, o, d); break;
+        case 3: KVMIX_CASE_V(d); key_tokens_body<11, 3>(f.ka, gi, o, d); break;
+        case 4: KVMIX_CASE_V(d); key_tokens_body<32, 4>(f.ka, gi, o, d); break;
+        default: KVMIX_CASE_V(d); key_tokens_body<32, 30>(f.ka, gi, o, d); break;
         }
     } else if (STREAM && f.v_stream) {
-        const int64_t first = (int64_t)(bx - f.k_blocks) * 512 + threadIdx.x;
+        int64_t first = (int64_t)(bx - f.k_blocks) * 512 + threadIdx.x;
         switch (f.va.bits) {
-        case 1: rows_g32_f16_stream_body<1, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        case 2: rows_g32_f16_stream_body<2, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        case 3: rows_g32_f16_stream_body<3, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        default: rows_g32_f16_stream_body<4, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 1: KVMIX_CASE_V(first); rows_g32_f16_stream_body<1, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 2: KVMIX_CASE_V(first); rows_g32_f16_stream_body<2, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 3: KVMIX_CASE_V(first); rows_g32_f16_stream_body<3, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        default: KVMIX_CASE_V(first); rows_g32_f16_stream_body<4, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
         }
     } else {
-        const int64_t tid = (int64_t)(bx - f.k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
+        int64_t tid = (int64_t)(bx - f.k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
         switch (f.va.bits) {
-        case 1: rows_g32_f16_body<1, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
-        case 2: rows_g32_f16_body<2, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
-        case 3: rows_g32_f16_body<3, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
-        default: rows_g32_f16_body<4, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        case 1: KVMIX_CASE_V(tid); rows_g32_f16_body<1, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        case 2: KVMIX_CASE_V(tid); rows_g32_f16_body<2, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        case 3: KVMIX_CASE_V(tid); rows_g32_f16_body<3, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
+        default: KVMIX_CASE_V(tid); rows_g32_f16_body<4, kFlushValuePieces, kFlushIdx32>(f.va, f.v_groups_per_row, f.v_total_groups, tid); break;
         }
     }
 }
+#undef KVMIX_CASE_V
+#undef KVMIX_CASE_S
 
 __global__ void __launch_bounds__(256) quant_kv_flush(FlushItem f)
 {
