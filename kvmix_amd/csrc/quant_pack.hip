@@ -616,6 +616,11 @@ struct FlushItem {
     int v_stream;               // value half: one thread per group, two groups a thread (rows_g32_f16_stream_body)
 };
 
+#ifndef KVMIX_FLUSH_STREAM_P
+#define KVMIX_FLUSH_STREAM_P 1
+#endif
+constexpr int kFlushStreamP = KVMIX_FLUSH_STREAM_P;  // groups a thread of the streaming value form takes (measured per launch
+                                                     // of eight layers: two groups, 80 registers, six waves per SIMD 51 us; one group, 58, eight waves 47 us)
 // One case of a switch over the formats, kept apart from its siblings: the value passes through an empty asm, so the
 // compiler cannot merge the cases' common heads above the switch -- merged, the batched kernel needs 107 registers
 // where its largest case alone needs 77 (four waves per SIMD instead of six).
@@ -647,12 +652,12 @@ __device__ __forceinline__ void flush_block(const FlushItem &f, unsigned bx, uin
         default: KVMIX_CASE_V(d); key_tokens_body<32, 30>(f.ka, gi, o, d); break;
         }
     } else if (STREAM && f.v_stream) {
-        int64_t first = (int64_t)(bx - f.k_blocks) * 512 + threadIdx.x;
+        int64_t first = (int64_t)(bx - f.k_blocks) * (256 * kFlushStreamP) + threadIdx.x;
         switch (f.va.bits) {
-        case 1: KVMIX_CASE_V(first); rows_g32_f16_stream_body<1, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        case 2: KVMIX_CASE_V(first); rows_g32_f16_stream_body<2, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        case 3: KVMIX_CASE_V(first); rows_g32_f16_stream_body<3, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
-        default: KVMIX_CASE_V(first); rows_g32_f16_stream_body<4, 2>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 1: KVMIX_CASE_V(first); rows_g32_f16_stream_body<1, kFlushStreamP>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 2: KVMIX_CASE_V(first); rows_g32_f16_stream_body<2, kFlushStreamP>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        case 3: KVMIX_CASE_V(first); rows_g32_f16_stream_body<3, kFlushStreamP>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
+        default: KVMIX_CASE_V(first); rows_g32_f16_stream_body<4, kFlushStreamP>(f.va, (uint32_t)f.v_groups_per_row, f.v_total_groups, first); break;
         }
     } else {
         int64_t tid = (int64_t)(bx - f.k_blocks) * (256 * kFlushValuePieces) + threadIdx.x;
@@ -677,7 +682,7 @@ __global__ void __launch_bounds__(256) quant_kv_flush(FlushItem f)
 // layers -- the longer chains of dependent steps -- then the value blocks.  The items travel as kernel arguments.
 constexpr int kFlushBatch = 8;
 #ifndef KVMIX_FLUSH_BATCH_OCC
-#define KVMIX_FLUSH_BATCH_OCC 4  // waves per SIMD the compiler plans for (107 registers; capped at 5 or 6 it spills: 206 -> 214 -> 250 us)
+#define KVMIX_FLUSH_BATCH_OCC 8  // waves per SIMD the compiler plans for (58 registers with one group a thread in the streaming value form)
 #endif
 #ifndef KVMIX_FLUSH_STREAM_GROUPS
 #define KVMIX_FLUSH_STREAM_GROUPS 16384
@@ -1012,10 +1017,10 @@ static int setup_flush(const kvmix_key_flush_t *kf, const kvmix_value_flush_t *v
     f.v_groups_per_row = f.va.steps / 32;
     f.v_total_groups = f.va.outer * f.va.inner * f.v_groups_per_row;
     // A flush alone is a latency-bound launch and wants many small threads (four to a group); in a batch of layers
-    // the value half is a streaming kernel and takes the prompt quantizer's form, a thread per group, two groups a
-    // thread (measured, the 32 flushes of a step in four launches: 222.8 -> 206.7 us).
+    // the value half is a streaming kernel and takes the prompt quantizer's form, a thread per group (measured, the
+    // 32 flushes of a step in four launches: 222.8 -> 206.7 us).
     f.v_stream = batched && f.v_total_groups >= kFlushStreamGroups && f.v_groups_per_row < (1ll << 31) ? 1 : 0;
-    const int64_t v_blocks = f.v_stream ? (f.v_total_groups + 511) / 512
+    const int64_t v_blocks = f.v_stream ? (f.v_total_groups + 256 * kFlushStreamP - 1) / (256 * kFlushStreamP)
                                         : (f.v_total_groups * 4 + 256 * kFlushValuePieces - 1) / (256 * kFlushValuePieces);
     if (k_blocks + v_blocks > 0x7fffffff || f.k_threads > 0x7fffffff) return KVMIX_ERR_SHAPE;
     f.k_blocks = (unsigned)k_blocks;
